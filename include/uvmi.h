@@ -1,0 +1,142 @@
+/*
+ * uvmi.h - C ABI of the MI355X (gfx950) decode engine kernels for UV-50M.
+ *
+ * Every entry point takes raw device pointers, explicit sizes and strides (in ELEMENTS unless a name says
+ * bytes) and a HIP stream handle (hipStream_t passed as void*; NULL = the default stream).  No entry point
+ * allocates device memory, synchronises the device or throws: the return value is 0 on success or a negative
+ * UVMI_E* code, and uvmi_last_error() returns a thread-local message for the last failure on this thread.
+ * All launches go to the device that is current on the calling thread, so callers running a second Python
+ * thread under another device (reference: scripts/rl_grpo.py:519-521) are served without global state.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the reference checkout).
+ */
+#ifndef UVMI_H
+#define UVMI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UVMI_OK 0
+#define UVMI_EINVAL (-1)      /* malformed argument (null pointer, negative size, bad enum) */
+#define UVMI_EUNSUPPORTED (-2) /* shape / dtype / alignment the kernels do not cover */
+#define UVMI_EWORKSPACE (-3)  /* workspace pointer missing or too small */
+#define UVMI_EHIP (-4)        /* a HIP runtime call failed (message holds hipGetErrorString) */
+
+/* element types */
+#define UVMI_F16 0
+#define UVMI_BF16 1
+#define UVMI_F32 2
+#define UVMI_I8 3
+#define UVMI_I32 4
+#define UVMI_I64 5
+
+int uvmi_version(void);
+const char* uvmi_last_error(void);
+/* Number of compute units of the current device (used by the split heuristics); <0 on error. */
+int uvmi_device_cus(void);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * int8 KV quantizer and cache writes.  Replaces ultraviolet/kernels/kv_quant.py.
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* quantize_kv (kv_quant.py:12-19): n_rows rows of hd elements (x_row_stride elements apart, unit inner stride)
+ * -> q int8 (n_rows, hd) contiguous, scale fp16 (n_rows,) contiguous.  s16 = fp16(absmax/127); the row is divided
+ * by max(float(s16), 1e-30) with IEEE fp32 division, rounded half-to-even and clamped to +-127.  Bit-exact. */
+int uvmi_quantize_rows(const void* x, int x_dtype, int64_t n_rows, int hd, int64_t x_row_stride,
+                       int8_t* q, uint16_t* scale, void* stream);
+
+/* dequantize_kv (kv_quant.py:22-23): out[r, :] = q[r, :] * float(scale[r]) cast to out_dtype. */
+int uvmi_dequantize_rows(const int8_t* q, const uint16_t* scale, int64_t n_rows, int hd, void* out, int out_dtype,
+                         void* stream);
+
+/* kv_write (kv_quant.py:26-36): quantize row r of x and store it at row flat_idx[r] of the contiguous
+ * (cache_rows, hd) int8 view of the cache and at element flat_idx[r] of the flat fp16 scale view.
+ * flat_idx is int64 (idx_dtype UVMI_I64) or int32; rows whose index falls outside [0, cache_rows) are skipped.
+ * If scale is NULL the cache holds cache_dtype (F16/BF16) values and rows are copied with a cast. */
+int uvmi_kv_write(void* cache, int cache_dtype, uint16_t* scale, int64_t cache_rows, const void* flat_idx,
+                  int idx_dtype, const void* x, int x_dtype, int64_t n_rows, int hd, int64_t x_row_stride,
+                  void* stream);
+
+/* Fused decode-time append of K and V of one layer (fast_decode.py:291-294, 315-317): for every row b and kv
+ * head h, quantize k[b, h, :] and v[b, h, :] and store them at slot pos[b] (linear cache) or pos[b] % S (ring)
+ * of k_cache / v_cache (B, KH, S, hd; batch/head/slot strides given) with their fp16 scales (B, KH, S).
+ * One launch for both tensors.  Rows with pos[b] < 0, or pos[b] >= S on a linear cache, are skipped. */
+typedef struct uvmi_kv_append_args {
+  const void* k; const void* v; int x_dtype;            /* (B, KH, hd) new keys / values */
+  int64_t sxb, sxh;                                     /* strides of k and v (shared) */
+  int8_t* k_cache; int8_t* v_cache;                     /* (B, KH, S, hd) */
+  int64_t scb, sch, scs;                                /* cache strides (shared by K and V) */
+  uint16_t* k_scale; uint16_t* v_scale;                 /* (B, KH, S) fp16 */
+  int64_t ssb, ssh;                                     /* scale strides (slot stride 1) */
+  const void* pos; int idx_dtype;                       /* (B,) position being written */
+  const void* rows;                                     /* optional (B,) cache row of each input row (same
+                                                           idx_dtype); NULL = identity */
+  int B, KH, S, hd, ring;
+} uvmi_kv_append_args;
+int uvmi_kv_append(const uvmi_kv_append_args* a, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Ragged single-query decode attention.  Replaces decode_attention / mathk::decode_attn
+ * (ultraviolet/kernels/decode_attn.py:174-230, kernels/decode_attn_cuda.py:273-309).
+ * ---------------------------------------------------------------------------------------------------------- */
+typedef struct uvmi_attn_args {
+  const void* q; int q_dtype;              /* (B, H, hd) F16 or BF16, inner stride 1 */
+  int64_t sqb, sqh;
+  const void* k_cache; const void* v_cache; int kv_dtype; /* (B, KH, S, hd) I8, F16 or BF16, inner stride 1 */
+  int64_t skb, skh, sks, svb, svh, svs;
+  const void* k_scale; const void* v_scale; /* (B, KH, S) fp16 when kv_dtype == I8, else NULL */
+  int64_t ssb, ssh, stb, sth;
+  const void* pos; const void* starts; int idx_dtype; /* (B,) I64 or I32: position of the current key (already
+                                                         written) and first valid position of each row */
+  void* out; int out_dtype;                /* (B, H, hd) F16 / BF16 / F32, inner stride 1 */
+  int64_t sob, soh;
+  int B, H, KH, S, hd;
+  float scale;                             /* softmax scale applied to q.k */
+  int window;                              /* 0 = unlimited; else keys pos-window+1..pos */
+  int ring;                                /* slot of position t is t % S (else t) */
+  int num_splits;                          /* >= 1: chunks each row's key range is cut into */
+  void* workspace; size_t workspace_bytes; /* >= uvmi_decode_attn_workspace_bytes(...) when num_splits > 1 */
+} uvmi_attn_args;
+
+/* Keys attended by row b: absolute positions max(starts[b], pos[b]-window+1, 0) .. pos[b]; a row with no valid
+ * key yields zeros.  fp32 accumulation; int8 caches are dequantised in registers (K scale on the score column,
+ * V scale on the probability).  Deterministic for a given num_splits. */
+int uvmi_decode_attn(const uvmi_attn_args* a, void* stream);
+size_t uvmi_decode_attn_workspace_bytes(int B, int H, int KH, int hd, int num_splits);
+/* default_splits (decode_attn.py:121-129) re-derived for 256 CUs x wave64: enough (row, kv head, split) work
+ * items to fill the device, each chunk >= min_chunk keys, at most 64.  n_cus <= 0: query the current device. */
+int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus);
+/* 1 if uvmi_decode_attn runs the MFMA kernel for these arguments, 0 if the generic kernel (any hd <= 256,
+ * G <= 16), negative if unsupported.  Mirrors decode_attn_cuda.supported (decode_attn_cuda.py:265-270). */
+int uvmi_decode_attn_path(const uvmi_attn_args* a);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Fused softcap + categorical draw + behaviour log-prob.  Replaces fused_sample
+ * (ultraviolet/kernels/fused_sample.py:68-77) and the torch.rand call feeding it (ultraviolet/perf.py:595).
+ * ---------------------------------------------------------------------------------------------------------- */
+typedef struct uvmi_sample_args {
+  const void* x; int x_dtype;      /* (B, V) raw head output before the softcap; F16 / BF16 / F32 */
+  int64_t stride;                  /* row stride of x */
+  const float* u;                  /* (B,) uniforms in [0, 1), or NULL to draw them from Philox4x32-10 */
+  uint64_t seed;                   /* Philox key when u == NULL */
+  const int64_t* req_id;           /* (B,) counter word: request id of each row (u == NULL) */
+  const int64_t* tok_idx;          /* (B,) counter word: index of the token being drawn (u == NULL) */
+  int64_t* tok; float* logp;       /* (B,) outputs */
+  float* u_out;                    /* optional (B,): the uniform that was used */
+  int B, V;
+  float cap_a, cap_b, cap_c;       /* softcap a * sigmoid((x + b) / c) */
+  float temperature;               /* > 0 draws from softmax(z / T); <= 0 takes argmax (first maximal index) and
+                                      logp is log softmax(z)[tok] */
+} uvmi_sample_args;
+int uvmi_fused_sample(const uvmi_sample_args* a, void* stream);
+/* Host-side Philox4x32-10 (Random123) for tests and host tooling: out[4] = philox(ctr[4], key[2]). */
+void uvmi_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UVMI_H */

@@ -1,0 +1,386 @@
+"""GPU parity: HIP kernels (through the C ABI, via the ultraviolet_amd.kernels mirror) vs the CPU oracle.
+
+The cases restate the reference's kernel tests (tests/test_math_kernels.py, tests/test_perf_fz.py) on the same shapes
+and edge vectors.  Bars: int8 bytes / fp16 scales / indices bit-exact; attention atol = rtol = 2e-3 on the rounded
+output (the reference's own criterion, test_math_kernels.py:52) and 2e-3 relative on the fp32 pre-rounding output."""
+import numpy as np
+import pytest
+import torch
+
+from util import attn_case, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _oracle():
+    from oracle import decode_attn, fused_sample, kv_quant, philox
+    return decode_attn, fused_sample, kv_quant, philox
+
+
+def _attn_check(q, k, v, ks, vs, pos, starts, scale, window=0, ring=None, splits=None, kview=None):
+    """Run kernel (fp32 output and rounded output) and compare with the oracle."""
+    from ultraviolet_amd.kernels import decode_attention
+    da = _oracle()[0]
+    d = lambda t: None if t is None else t.to(DEV)
+    kk, vv, kss, vss = (d(k), d(v), d(ks), d(vs))
+    if kview is not None:
+        kk, vv = kk[:, :, :kview], vv[:, :, :kview]
+        if kss is not None:
+            kss, vss = kss[:, :, :kview], vss[:, :, :kview]
+    kw = dict(window=window, ring=ring, k_scale=kss, v_scale=vss, num_splits=splits)
+    out32 = decode_attention(d(q), kk, vv, d(pos), d(starts), scale, out_fp32=True, **kw)
+    out = decode_attention(d(q), kk, vv, d(pos), d(starts), scale, **kw)
+    torch.cuda.synchronize()
+    ref = da.decode_attention_ref(to_np(q), to_np(k), to_np(v), to_np(pos), to_np(starts), scale, window=window,
+                                  ring=ring, k_scale=None if ks is None else to_np(ks),
+                                  v_scale=None if vs is None else to_np(vs))
+    o32 = to_np(out32)
+    assert np.isfinite(o32).all()
+    np.testing.assert_allclose(o32, ref, atol=2e-3, rtol=2e-3)
+    np.testing.assert_allclose(to_np(out), ref.astype(np.float32), atol=2e-3 + 4e-3 * np.abs(ref).max() * (q.dtype == torch.bfloat16),
+                               rtol=2e-3 if q.dtype == torch.float16 else 8e-3)
+    return o32, ref
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("int8", [False, True])
+@pytest.mark.parametrize("B,KH,G,hd", [(1, 1, 1, 128), (3, 1, 4, 128), (17, 1, 5, 128), (5, 2, 4, 64),
+                                       (9, 1, 8, 64), (4, 2, 2, 16), (6, 1, 7, 128), (33, 1, 8, 64)])
+@pytest.mark.parametrize("splits", [1, 3, None])
+def test_global_ragged(dtype, int8, B, KH, G, hd, splits):
+    """reference: tests/test_math_kernels.py:36-52."""
+    S = 700
+    q, k, v, ks, vs = attn_case(B, KH, G, hd, S, int8, dtype=dtype)
+    g = torch.Generator().manual_seed(1)
+    pos = torch.randint(0, S, (B,), generator=g)
+    pos[0] = S - 1
+    starts = (torch.rand(B, generator=g) * (pos + 1).float()).long()
+    starts[0] = 0
+    _attn_check(q, k, v, ks, vs, pos, starts, 1.13 / hd ** 0.5, splits=splits)
+
+
+@pytest.mark.parametrize("int8", [False, True])
+@pytest.mark.parametrize("W,hd,G", [(128, 128, 5), (256, 64, 8), (1024, 128, 4), (100, 128, 4), (64, 64, 8),
+                                    (100, 64, 8)])
+@pytest.mark.parametrize("splits", [1, 4])
+def test_ring_wraparound(int8, W, hd, G, splits):
+    """reference: tests/test_math_kernels.py:55-70 (positions before, at and past the wrap; left pad past window start)."""
+    B = 12
+    q, k, v, ks, vs = attn_case(B, 1, G, hd, W, int8, seed=1)
+    pos = torch.tensor([0, 5, W - 2, W - 1, W, W + 1, 2 * W + 7, 3 * W - 1, 5 * W + 3, W + 10, 4 * W, 7])
+    starts = torch.tensor([0, 2, 0, 3, 0, 4, 0, 2 * W + 5, 0, 30, 4 * W - 3, 7])
+    _attn_check(q, k, v, ks, vs, pos, starts, 0.1, window=W, splits=splits)
+
+
+@pytest.mark.parametrize("int8,hd,G", [(False, 128, 4), (True, 64, 8)])
+def test_window_smaller_than_cache(int8, hd, G):
+    """Sliding window on a non-ring cache; reference: tests/test_math_kernels.py:73-82."""
+    B, S, W = 6, 500, 64
+    q, k, v, ks, vs = attn_case(B, 1, G, hd, S, int8, seed=2)
+    pos = torch.tensor([10, 63, 64, 200, 499, 300])
+    starts = torch.tensor([0, 0, 1, 180, 0, 290])
+    _attn_check(q, k, v, ks, vs, pos, starts, 0.1, window=W, ring=False, splits=2)
+
+
+def test_matches_sdpa_fp16():
+    """Kernel vs torch SDPA with an additive mask (the model's formulation); reference: test_math_kernels.py:85-98."""
+    from ultraviolet_amd.kernels import decode_attention
+    B, G, hd, S = 32, 5, 128, 2048
+    q, k, v, _, _ = attn_case(B, 1, G, hd, S, False, seed=3)
+    g = torch.Generator().manual_seed(3)
+    pos = torch.randint(S // 2, S, (B,), generator=g)
+    starts = torch.randint(0, 50, (B,), generator=g)
+    t = torch.arange(S)[None]
+    bias = torch.zeros(B, S).masked_fill(~((t <= pos[:, None]) & (t >= starts[:, None])), float("-inf"))
+    bias = bias[:, None, None].expand(B, 1, G, S)
+    z = torch.nn.functional.scaled_dot_product_attention(q.float().view(B, 1, G, hd), k.float(), v.float(),
+                                                         attn_mask=bias, scale=0.1)
+    out = decode_attention(q.to(DEV), k.to(DEV), v.to(DEV), pos.to(DEV), starts.to(DEV), 0.1)
+    torch.testing.assert_close(out.float().cpu().view_as(z), z, atol=2e-3, rtol=2e-3)
+
+
+@pytest.mark.parametrize("hd,G,KH", [(128, 4, 2), (64, 8, 1), (64, 4, 2)])
+def test_non_contiguous_global_slice(hd, G, KH):
+    """cache[:, :, :g_len] views: strides must be honoured; reference: tests/test_math_kernels.py:101-112."""
+    B, S = 5, 512
+    q, k, v, ks, vs = attn_case(B, KH, G, hd, S, True, seed=4)
+    pos = torch.tensor([0, 100, 255, 17, 200])
+    starts = torch.tensor([0, 3, 0, 17, 150])
+    _attn_check(q, k, v, ks, vs, pos, starts, 0.1, splits=2, kview=256)
+
+
+def test_int32_positions_and_empty_rows():
+    from ultraviolet_amd.kernels import decode_attention
+    B, S = 7, 256
+    q, k, v, ks, vs = attn_case(B, 1, 8, 64, S, True, seed=5, dtype=torch.bfloat16)
+    pos = torch.tensor([0, 1, 31, 32, 33, 255, 128], dtype=torch.int32)
+    starts = torch.tensor([0, 1, 0, 32, 0, 200, 129], dtype=torch.int32)  # last row: start > pos -> no valid key
+    d = lambda t: t.to(DEV)
+    out = decode_attention(d(q), d(k), d(v), d(pos), d(starts), 0.14125, k_scale=d(ks), v_scale=d(vs), num_splits=2,
+                           out_fp32=True)
+    da = _oracle()[0]
+    ref = da.decode_attention_ref(to_np(q)[:6], to_np(k)[:6], to_np(v)[:6], to_np(pos)[:6], to_np(starts)[:6], 0.14125,
+                                  k_scale=to_np(ks)[:6], v_scale=to_np(vs)[:6])
+    o = to_np(out)
+    np.testing.assert_allclose(o[:6], ref, atol=2e-3, rtol=2e-3)
+    assert (o[6] == 0).all()
+
+
+def test_stale_nonfinite_scales_outside_range_are_ignored():
+    """Slots outside lo..pos may hold anything (caches are never cleared on refill: reference model.py:883-884)."""
+    from ultraviolet_amd.kernels import decode_attention
+    B, S = 4, 128
+    q, k, v, ks, vs = attn_case(B, 1, 8, 64, S, True, seed=6)
+    pos = torch.tensor([40, 77, 5, 100])
+    starts = torch.tensor([3, 70, 0, 64])
+    ks2, vs2 = ks.clone(), vs.clone()
+    for b in range(B):
+        bad = torch.ones(S, dtype=torch.bool)
+        bad[starts[b]:pos[b] + 1] = False
+        ks2[b, 0, bad] = float("nan")
+        vs2[b, 0, bad] = float("inf")
+    d = lambda t: t.to(DEV)
+    for sp in (1, 3):
+        out = decode_attention(d(q), d(k), d(v), d(pos), d(starts), 0.1, k_scale=d(ks2), v_scale=d(vs2), num_splits=sp,
+                               out_fp32=True)
+        ref = _oracle()[0].decode_attention_ref(to_np(q), to_np(k), to_np(v), to_np(pos), to_np(starts), 0.1,
+                                                k_scale=to_np(ks), v_scale=to_np(vs))
+        np.testing.assert_allclose(to_np(out), ref, atol=2e-3, rtol=2e-3)
+
+
+def test_config2_shape_relative_error():
+    """BASELINE config 2: 256 rows, 8 heads x 64, KH = 1, contexts U[64, 1024], bf16 q, int8 KV, scale 0.14125.
+    Bar: 2e-3 max relative error on the fp32-accumulation output, relative error of a (row, head) output vector being
+    max_d |out - ref| / max_d |ref|; plus the reference's elementwise atol = rtol = 2e-3."""
+    from ultraviolet_amd.kernels import decode_attention
+    B, S = 256, 1024
+    q, k, v, ks, vs = attn_case(B, 1, 8, 64, S, True, seed=0, dtype=torch.bfloat16)
+    rng = np.random.default_rng(0)
+    n = rng.integers(64, 1025, size=B)
+    pos = torch.from_numpy(n - 1)
+    starts = torch.zeros(B, dtype=torch.long)
+    d = lambda t: t.to(DEV)
+    ref = _oracle()[0].decode_attention_ref(to_np(q), to_np(k), to_np(v), to_np(pos), to_np(starts), 0.14125,
+                                            k_scale=to_np(ks), v_scale=to_np(vs))
+    for sp in (1, 2, None):
+        out = to_np(decode_attention(d(q), d(k), d(v), d(pos), d(starts), 0.14125, k_scale=d(ks), v_scale=d(vs),
+                                     num_splits=sp, out_fp32=True))
+        rel = np.abs(out - ref).max(-1) / np.abs(ref).max(-1)
+        assert rel.max() < 2e-3, rel.max()
+        np.testing.assert_allclose(out, ref, atol=2e-3, rtol=2e-3)
+
+
+# ------------------------------------------------------------------------------------------------ quantizer
+def _all_patterns(dtype):
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(dtype)
+    return x[torch.isfinite(x.float())]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hd", [64, 128, 16, 48])
+def test_quantize_bit_exact_all_patterns(dtype, hd):
+    """Every finite fp16 / bf16 bit pattern appears as an element, against rows whose absmax sweeps every pattern."""
+    from ultraviolet_amd.kernels import quantize_kv
+    kq = _oracle()[2]
+    vals = _all_patterns(dtype)
+    g = torch.Generator().manual_seed(hd)
+    n = vals.numel()
+    rows = (n + hd - 1) // hd * 4
+    idx = torch.randint(0, n, (rows, hd), generator=g)
+    idx.view(-1)[:n] = torch.arange(n)
+    x = vals[idx]
+    # scale rows so the absmax also sweeps magnitudes: keep some rows as is, shrink others
+    mags = vals[torch.randint(0, n, (rows, 1), generator=g)].float().abs().clamp(max=6e4)
+    x2 = torch.where(x.float().abs() <= mags, x, torch.zeros_like(x))
+    x = torch.cat([x, x2])
+    q, s = quantize_kv(x.to(DEV))
+    rq, rs = kq.quantize_kv(to_np(x))
+    assert np.array_equal(to_np(q), rq)
+    assert np.array_equal(to_np(s).view(np.uint16), rs.view(np.uint16))
+
+
+def test_quantize_fp32_rows_and_zero_row():
+    from ultraviolet_amd.kernels import dequantize_kv, quantize_kv
+    kq = _oracle()[2]
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 3, 128, generator=g) * 3
+    x[0, 0] = 0
+    x[1, 1] = 1e-9       # scale underflows fp16 -> s = 0, codes +-127
+    x[2, 2, 5] = 7e4     # absmax/127 fine
+    q, s = quantize_kv(x.to(DEV))
+    rq, rs = kq.quantize_kv(x.numpy())
+    assert np.array_equal(to_np(q), rq) and np.array_equal(to_np(s).view(np.uint16), rs.view(np.uint16))
+    assert (to_np(q)[0, 0] == 0).all()
+    # reference bound, tests/test_math_kernels.py:115-121
+    xh = x.half()
+    q, s = quantize_kv(xh.to(DEV))
+    err = (dequantize_kv(q, s).float().cpu() - xh.float()).abs()
+    assert err.max() <= (s.float().cpu().unsqueeze(-1) * 0.5 + 1e-3).max()
+
+
+def test_kv_write_flat_index():
+    """reference: tests/test_math_kernels.py:122-128 (idx = [3, 31, 32, 55])."""
+    from ultraviolet_amd.kernels import dequantize_kv, kv_write
+    kq = _oracle()[2]
+    g = torch.Generator().manual_seed(0)
+    cache = torch.zeros(4, 1, 16, 128, dtype=torch.int8)
+    sc = torch.zeros(4, 1, 16, dtype=torch.half)
+    idx = torch.tensor([0 * 16 + 3, 1 * 16 + 15, 2 * 16 + 0, 3 * 16 + 7])
+    xv = torch.randn(4, 128, generator=g).half()
+    c_d, s_d = cache.to(DEV), sc.to(DEV)
+    kv_write(c_d, s_d, idx.to(DEV), xv.to(DEV))
+    rc, rs = cache.numpy().copy(), sc.numpy().copy()
+    kq.kv_write(rc, rs, idx.numpy(), to_np(xv))
+    assert np.array_equal(to_np(c_d), rc) and np.array_equal(to_np(s_d).view(np.uint16), rs.view(np.uint16))
+    back = dequantize_kv(c_d.view(-1, 128)[idx.to(DEV)], s_d.view(-1)[idx.to(DEV)])
+    torch.testing.assert_close(back.float().cpu(), xv.float(), atol=0.03, rtol=0.03)
+    # unquantized cache
+    c16 = torch.zeros(4, 1, 16, 128, dtype=torch.half, device=DEV)
+    kv_write(c16, None, idx.to(DEV), xv.to(DEV))
+    assert torch.equal(c16.view(-1, 128)[idx.to(DEV)].cpu(), xv)
+
+
+@pytest.mark.parametrize("ring", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_kv_append_matches_oracle_writes(ring, dtype):
+    """Fused K+V append == two oracle kv_write calls at (b*K+h)*S + pos (or pos % S)."""
+    from ultraviolet_amd.kernels import kv_append
+    kq = _oracle()[2]
+    B, K, S, hd = 37, 2, 48, 64
+    g = torch.Generator().manual_seed(3)
+    kc = torch.randint(-127, 128, (B, K, S, hd), generator=g, dtype=torch.int8)
+    vc = torch.randint(-127, 128, (B, K, S, hd), generator=g, dtype=torch.int8)
+    ksc = torch.rand(B, K, S, generator=g).half()
+    vsc = torch.rand(B, K, S, generator=g).half()
+    k = torch.randn(B, K, hd, generator=g).to(dtype)
+    v = torch.randn(B, K, hd, generator=g).to(dtype)
+    pos = torch.randint(0, 5 * S if ring else S, (B,), generator=g)
+    d = lambda t: t.to(DEV)
+    kcd, vcd, ksd, vsd = d(kc), d(vc), d(ksc), d(vsc)
+    kv_append(d(k), d(v), kcd, vcd, ksd, vsd, d(pos), ring=ring)
+    rk, rv, rks, rvs = kc.numpy().copy(), vc.numpy().copy(), ksc.numpy().copy(), vsc.numpy().copy()
+    ix = kq.decode_flat_index(pos.numpy(), K, S, ring)
+    kq.kv_write(rk, rks, ix, to_np(k).reshape(-1, hd))
+    kq.kv_write(rv, rvs, ix, to_np(v).reshape(-1, hd))
+    assert np.array_equal(to_np(kcd), rk) and np.array_equal(to_np(vcd), rv)
+    assert np.array_equal(to_np(ksd).view(np.uint16), rks.view(np.uint16))
+    assert np.array_equal(to_np(vsd).view(np.uint16), rvs.view(np.uint16))
+
+
+def test_kv_write_rows_prefill():
+    """reference semantics of kv_write_rows (kv_quant.py:39-54): partial rows, ring slots."""
+    from ultraviolet_amd.kernels import kv_write_rows
+    kq = _oracle()[2]
+    B, K, S, hd, T = 6, 1, 16, 64, 21
+    g = torch.Generator().manual_seed(4)
+    cache = torch.randint(-5, 5, (B, K, S, hd), generator=g, dtype=torch.int8)
+    sc = torch.rand(B, K, S, generator=g).half()
+    new = torch.randn(3, K, T, hd, generator=g).half()
+    rows = torch.tensor([4, 0, 3])
+    lo = T - S
+    slots = torch.arange(lo, T) % S
+    cd, sd = cache.to(DEV), sc.to(DEV)
+    kv_write_rows(cd, sd, new[:, :, lo:].to(DEV), slots.to(DEV), rows.to(DEV))
+    rc, rs = cache.numpy().copy(), sc.numpy().copy()
+    kq.kv_write_rows(rc, rs, to_np(new[:, :, lo:]), slots.numpy(), rows.numpy())
+    assert np.array_equal(to_np(cd), rc) and np.array_equal(to_np(sd).view(np.uint16), rs.view(np.uint16))
+
+
+# ------------------------------------------------------------------------------------------------ sampler
+SC = (23.0, 5.0, 7.5)
+
+
+@pytest.mark.parametrize("T", [1.0, 0.8])
+@pytest.mark.parametrize("dtype,V", [(torch.float16, 16384), (torch.bfloat16, 32768)])
+def test_sampler_matches_ref(T, dtype, V):
+    """reference: tests/test_perf_fz.py:96-119: token is the inverse-CDF draw of the exact (fp64) softmax up to fp32
+    summation rounding; mostly the same token as the flat-cumsum oracle; log-probs match log_softmax."""
+    from ultraviolet_amd.kernels.fused_sample import fused_sample
+    fs = _oracle()[1]
+    g = torch.Generator().manual_seed(0)
+    B = 1024
+    x = (torch.randn(B, V, generator=g) * torch.rand(B, 1, generator=g) * 8).to(dtype)
+    u = torch.rand(B, generator=g)
+    t, lp = fused_sample(x.to(DEV), u.to(DEV), SC, T)
+    t, lp = t.cpu(), lp.cpu()
+    tr, lpr = fs.fused_sample_ref(to_np(x), u.numpy(), SC, T)
+    assert t.dtype == torch.int64 and t.min() >= 0 and t.max() < V
+    assert (t.numpy() == tr).mean() > 0.99
+    z = torch.from_numpy(fs.softcap(to_np(x), SC)).double()
+    e = torch.exp((z - SC[0]) / T)
+    cs = e.cumsum(-1)
+    S = cs[:, -1]
+    tgt = (1.0 - u.double()) * S
+    hi = cs.gather(1, t[:, None])[:, 0]
+    lo = hi - e.gather(1, t[:, None])[:, 0]
+    tol = 1e-5 * S
+    assert ((tgt >= lo - tol) & (tgt <= hi + tol)).all()
+    ls = torch.log_softmax(z / T, -1).gather(1, t[:, None])[:, 0]
+    assert (lp.double() - ls).abs().max() < 2e-5
+
+
+def test_sampler_edges():
+    """reference: tests/test_perf_fz.py:66-71."""
+    from ultraviolet_amd.kernels.fused_sample import fused_sample
+    x = torch.full((2, 512), -1e4)
+    x[:, 40] = 10.0
+    tok, lp = fused_sample(x.to(DEV), torch.tensor([0.0, 1.0 - 2 ** -24]).to(DEV), SC, 1.0)
+    assert tok.max() < 512 and tok.min() >= 0 and torch.isfinite(lp).all()
+
+
+def test_sampler_distribution_chi2():
+    """reference: tests/test_perf_fz.py:122-134."""
+    from ultraviolet_amd.kernels.fused_sample import fused_sample
+    fs = _oracle()[1]
+    g = torch.Generator().manual_seed(1)
+    V, n = 4096, 1 << 17
+    for scale in (2.0, 12.0):
+        x = (torch.randn(V, generator=g) * scale).half()
+        p = torch.softmax(torch.from_numpy(fs.softcap(to_np(x), SC)).double(), -1)
+        u = torch.rand(n, generator=g)
+        t, _ = fused_sample(x[None].expand(n, V).contiguous().to(DEV), u.to(DEV), SC, 1.0)
+        cnt = torch.bincount(t.cpu(), minlength=V).double()
+        e = p * n
+        big = e >= 5
+        obs = torch.cat([cnt[big], cnt[~big].sum()[None]])
+        ex = torch.cat([e[big], e[~big].sum()[None]])
+        chi = ((obs - ex) ** 2 / ex).sum()
+        df = int(big.sum())
+        pval = float(torch.special.gammaincc(torch.tensor(df / 2, dtype=torch.float64), chi / 2))
+        assert pval > 1e-3
+
+
+def test_sampler_seeded_philox_and_greedy():
+    from ultraviolet_amd.kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
+    _, fs, _, ph = _oracle()
+    g = torch.Generator().manual_seed(2)
+    B, V = 300, 2048
+    x = (torch.randn(B, V, generator=g) * 4).bfloat16()
+    req = torch.randint(0, 2 ** 40, (B,), generator=g)
+    ti = torch.randint(0, 4096, (B,), generator=g)
+    seed = 0x1234_5678_9ABC_DEF0
+    t1, lp1, u1 = fused_sample_seeded(x.to(DEV), seed, req.to(DEV), ti.to(DEV), SC, 1.0, return_u=True)
+    uref = ph.request_uniform(seed, req.numpy(), ti.numpy())
+    assert np.array_equal(u1.cpu().numpy(), uref)            # Philox stream is bit-exact
+    t2, lp2 = fused_sample(x.to(DEV), torch.from_numpy(uref).to(DEV), SC, 1.0)
+    assert torch.equal(t1, t2) and torch.equal(lp1, lp2)
+    tg, lpg = greedy_sample(x.to(DEV), SC)
+    z = fs.softcap(to_np(x), SC)
+    assert np.array_equal(tg.cpu().numpy(), np.argmax(to_np(x), -1))
+    ref = torch.log_softmax(torch.from_numpy(z).double(), -1).gather(1, tg.cpu()[:, None])[:, 0]
+    assert (lpg.cpu().double() - ref).abs().max() < 2e-5
+
+
+def test_error_paths_are_loud():
+    from ultraviolet_amd import _lib as L
+    from ultraviolet_amd.kernels import decode_attention, quantize_kv
+    with pytest.raises(L.UvmiError):
+        quantize_kv(torch.zeros(4, 64))  # CPU tensor: no fallback
+    q = torch.zeros(2, 8, 64, device=DEV)  # fp32 q is not supported
+    kc = torch.zeros(2, 1, 64, 64, dtype=torch.int8, device=DEV)
+    sc = torch.zeros(2, 1, 64, dtype=torch.half, device=DEV)
+    p = torch.zeros(2, dtype=torch.long, device=DEV)
+    with pytest.raises(L.UvmiError):
+        decode_attention(q, kc, kc, p, p, 0.1, k_scale=sc, v_scale=sc)

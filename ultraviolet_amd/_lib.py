@@ -1,0 +1,109 @@
+"""ctypes binding of libuvmi.so (declarations: include/uvmi.h).  There is no CPU fallback: if the library has not
+been built, or a call fails, an exception is raised."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libuvmi.so")
+
+F16, BF16, F32, I8, I32, I64 = 0, 1, 2, 3, 4, 5
+_DT = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32, torch.int8: I8, torch.int32: I32,
+       torch.int64: I64}
+
+
+class UvmiError(RuntimeError):
+    pass
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise UvmiError(f"dtype {dt} is not supported by libuvmi") from None
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("q_dtype", C.c_int), ("sqb", C.c_int64), ("sqh", C.c_int64),
+                ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("kv_dtype", C.c_int),
+                ("skb", C.c_int64), ("skh", C.c_int64), ("sks", C.c_int64),
+                ("svb", C.c_int64), ("svh", C.c_int64), ("svs", C.c_int64),
+                ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+                ("ssb", C.c_int64), ("ssh", C.c_int64), ("stb", C.c_int64), ("sth", C.c_int64),
+                ("pos", C.c_void_p), ("starts", C.c_void_p), ("idx_dtype", C.c_int),
+                ("out", C.c_void_p), ("out_dtype", C.c_int), ("sob", C.c_int64), ("soh", C.c_int64),
+                ("B", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("S", C.c_int), ("hd", C.c_int),
+                ("scale", C.c_float), ("window", C.c_int), ("ring", C.c_int), ("num_splits", C.c_int),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
+class KvAppendArgs(C.Structure):
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("x_dtype", C.c_int), ("sxb", C.c_int64), ("sxh", C.c_int64),
+                ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+                ("scb", C.c_int64), ("sch", C.c_int64), ("scs", C.c_int64),
+                ("k_scale", C.c_void_p), ("v_scale", C.c_void_p), ("ssb", C.c_int64), ("ssh", C.c_int64),
+                ("pos", C.c_void_p), ("idx_dtype", C.c_int), ("rows", C.c_void_p),
+                ("B", C.c_int), ("KH", C.c_int), ("S", C.c_int), ("hd", C.c_int), ("ring", C.c_int)]
+
+
+class SampleArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("x_dtype", C.c_int), ("stride", C.c_int64), ("u", C.c_void_p),
+                ("seed", C.c_uint64), ("req_id", C.c_void_p), ("tok_idx", C.c_void_p),
+                ("tok", C.c_void_p), ("logp", C.c_void_p), ("u_out", C.c_void_p),
+                ("B", C.c_int), ("V", C.c_int),
+                ("cap_a", C.c_float), ("cap_b", C.c_float), ("cap_c", C.c_float), ("temperature", C.c_float)]
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Load libuvmi.so once.  Raises UvmiError when it is missing (build it with
+    `python -m ultraviolet_amd.csrc.build`)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise UvmiError(f"{LIB_PATH} not found: run `python -m ultraviolet_amd.csrc.build` (no CPU fallback)")
+        L = C.CDLL(LIB_PATH)
+        L.uvmi_last_error.restype = C.c_char_p
+        L.uvmi_decode_attn_workspace_bytes.restype = C.c_size_t
+        L.uvmi_decode_attn_workspace_bytes.argtypes = [C.c_int] * 5
+        L.uvmi_default_splits.argtypes = [C.c_int64, C.c_int, C.c_int]
+        L.uvmi_decode_attn.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+        L.uvmi_decode_attn_path.argtypes = [C.POINTER(AttnArgs)]
+        L.uvmi_quantize_rows.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int64, C.c_void_p, C.c_void_p,
+                                         C.c_void_p]
+        L.uvmi_dequantize_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+        L.uvmi_kv_write.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                    C.c_int64, C.c_int, C.c_int64, C.c_void_p]
+        L.uvmi_kv_append.argtypes = [C.POINTER(KvAppendArgs), C.c_void_p]
+        L.uvmi_fused_sample.argtypes = [C.POINTER(SampleArgs), C.c_void_p]
+        L.uvmi_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+        L.uvmi_philox4x32_10.restype = None
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().uvmi_last_error().decode(errors="replace")
+        raise UvmiError(f"{what} failed ({rc}): {msg}")
+
+
+def stream_ptr(t: torch.Tensor) -> int:
+    """HIP stream torch is currently launching on for t's device."""
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_cuda(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise UvmiError("libuvmi kernels need device tensors (there is no CPU path)")
+
+
+EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_rows", "uvmi_dequantize_rows",
+           "uvmi_kv_write", "uvmi_kv_append", "uvmi_decode_attn", "uvmi_decode_attn_workspace_bytes",
+           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10"]

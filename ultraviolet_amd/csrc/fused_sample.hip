@@ -1,0 +1,247 @@
+// Fused softcap + categorical draw (inverse CDF, one uniform per row) + behaviour log-prob, and greedy argmax.
+//
+// Contract (ultraviolet/kernels/fused_sample.py:31-77 of the reference): with z = a*sigmoid((x+b)/c) and
+// e = exp((z-a)/T) in (exp(-a/T), 1] (the softcap bounds z, so there is no max pass), S = sum(e),
+// target = (1-u)*S; the token is the first index whose running sum reaches target (clamped to V-1) and
+// logp = (z_tok - a)/T - log S.  The running sum is hierarchical here (512-element chunks, then lanes, then the
+// lane's 8 elements), so the token equals the flat-cumsum one up to fp32 summation order.
+//
+// e is evaluated as exp2(-(a/T)*log2(e) / (1 + exp2(t*log2(e)))), t = (x+b)/c: algebraically the same as above
+// (z - a = -a*sigmoid(-t)) without the cancellation of z - a near the cap.
+//
+// One workgroup of 256 threads per row streams the row once (HBM-bound: 2 B per logit for bf16/fp16), keeps only
+// the 64 chunk sums in LDS, then one wave re-reads the chosen 1 KB chunk (cache-hot).  When u is not supplied it is
+// drawn from Philox4x32-10 keyed by the seed with counter (token index, request id lo, request id hi, "SAMP"), so a
+// request's stream does not depend on the slot it occupies.
+#include "common.h"
+
+namespace uvmi {
+
+constexpr int CHUNK = 512;          // elements per wave pass: 64 lanes x 8
+constexpr uint32_t DOMAIN_SAMPLE = 0x53414D50u;
+
+__host__ __device__ inline void philox4x32_10(const uint32_t c_in[4], const uint32_t k_in[2], uint32_t out[4]) {
+  uint32_t c0 = c_in[0], c1 = c_in[1], c2 = c_in[2], c3 = c_in[3], k0 = k_in[0], k1 = k_in[1];
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+struct SampleParams {
+  const void* x; int64_t stride; const float* u; uint64_t seed; const int64_t* req_id; const int64_t* tok_idx;
+  int64_t* tok; float* logp; float* u_out;
+  int V;
+  float inv_c_l2, b_over_c_l2;  // t*log2(e) = x*inv_c_l2 + b_over_c_l2
+  float neg_a_over_t_l2;        // -(a/T)*log2(e)
+  float neg_a_over_t;           // -(a/T)
+  float cap_a, cap_b, cap_c, inv_c;
+};
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* row, int i, float (&o)[8]) {  // elements 8i .. 8i+7
+  if (DT == UVMI_F32) {
+    const float4 a = ((const float4*)row)[2 * i], b = ((const float4*)row)[2 * i + 1];
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  } else {
+    const uint4 w = ((const uint4*)row)[i];
+    const uint32_t r[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      if (DT == UVMI_BF16) {
+        o[2 * j] = __uint_as_float(r[j] << 16);
+        o[2 * j + 1] = __uint_as_float(r[j] & 0xffff0000u);
+      } else {
+        o[2 * j] = half_bits_to_float(r[j] & 0xffff);
+        o[2 * j + 1] = half_bits_to_float(r[j] >> 16);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ float e_of(float x, const SampleParams& P) {
+  const float E = __builtin_amdgcn_exp2f(fmaf(x, P.inv_c_l2, P.b_over_c_l2));  // exp(t), may be +inf (then e = 1)
+  return __builtin_amdgcn_exp2f(P.neg_a_over_t_l2 * __builtin_amdgcn_rcpf(1.0f + E));
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void sample_kernel(SampleParams P) {
+  __shared__ float csum[64 + 4];
+  __shared__ int sh_chunk;
+  __shared__ float sh_before, sh_total, sh_target;
+  const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const char* xr = (const char*)P.x + (int64_t)row * P.stride * (DT == UVMI_F32 ? 4 : 2);
+  const int nchunks = P.V / CHUNK;  // host guarantees V % 512 == 0 and nchunks <= 64
+  for (int c = wave; c < nchunks; c += 4) {
+    float v[8];
+    load8<DT>(xr, c * 64 + lane, v);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) s += e_of(v[j], P);
+    s = wave_sum(s);
+    if (lane == 0) csum[c] = s;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  // ---- wave 0: pick the chunk, then the lane, then the element
+  float mine = lane < nchunks ? csum[lane] : 0.f;
+  float incl = mine;  // inclusive scan over chunks in lane order
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float t = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += t;
+  }
+  const float S = __shfl(incl, 63, 64);
+  float u;
+  if (P.u) {
+    u = P.u[row];
+  } else {
+    const uint64_t rid = (uint64_t)P.req_id[row], ti = (uint64_t)P.tok_idx[row];
+    const uint32_t ctr[4] = {(uint32_t)ti, (uint32_t)rid, (uint32_t)(rid >> 32), DOMAIN_SAMPLE};
+    const uint32_t key[2] = {(uint32_t)P.seed, (uint32_t)(P.seed >> 32)};
+    uint32_t o[4];
+    philox4x32_10(ctr, key, o);
+    u = (float)(o[0] >> 8) * 5.9604644775390625e-08f;  // 2^-24
+  }
+  const float target = (1.0f - u) * S;
+  const unsigned long long below = __ballot(lane < nchunks && incl < target);
+  int ck = __popcll(below);  // first chunk whose inclusive sum reaches target
+  if (ck > nchunks - 1) ck = nchunks - 1;
+  const float before = ck > 0 ? __shfl(incl, ck - 1, 64) : 0.f;
+  float v[8], e[8];
+  load8<DT>(xr, ck * 64 + lane, v);
+  float ls = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    e[j] = e_of(v[j], P);
+    ls += e[j];
+  }
+  float linc = ls;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float t = __shfl_up(linc, o, 64);
+    if (lane >= o) linc += t;
+  }
+  linc += before;
+  const unsigned long long lb = __ballot(linc < target);
+  int ln = __popcll(lb);
+  if (ln > 63) ln = 63;
+  // every lane recomputes the winner lane's walk from broadcast values (uniform control flow)
+  float run = ln > 0 ? __shfl(linc, ln - 1, 64) : before;
+  int jsel = 7;
+  bool found = false;
+  float xsel = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const float ej = __shfl(e[j], ln, 64), xj = __shfl(v[j], ln, 64);
+    run += ej;
+    if (!found && run >= target) { found = true; jsel = j; xsel = xj; }
+    if (j == 7 && !found) xsel = xj;
+  }
+  if (lane == 0) {
+    const int tok = ck * CHUNK + ln * 8 + jsel;
+    P.tok[row] = tok;
+    // logp = (z_tok - a)/T - log S, with (z - a)/T = -(a/T) / (1 + exp(t))
+    const float E = __builtin_amdgcn_exp2f(fmaf(xsel, P.inv_c_l2, P.b_over_c_l2));
+    P.logp[row] = P.neg_a_over_t * __builtin_amdgcn_rcpf(1.0f + E) - __logf(S);
+    if (P.u_out) P.u_out[row] = u;
+  }
+}
+
+// Greedy: argmax of the raw head output (the softcap is strictly increasing, so argmax z = argmax x), first maximal
+// index; logp = log softmax(z)[tok] at T = 1.
+template <int DT>
+__global__ __launch_bounds__(256) void argmax_kernel(SampleParams P) {
+  __shared__ float smax[4];
+  __shared__ int sidx[4];
+  __shared__ float ssum[4];
+  const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const char* xr = (const char*)P.x + (int64_t)row * P.stride * (DT == UVMI_F32 ? 4 : 2);
+  const int nvec = P.V / 8;
+  float best = -INFINITY, esum = 0.f;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < nvec; i += 256) {
+    float v[8];
+    load8<DT>(xr, i, v);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      if (v[j] > best) { best = v[j]; bi = i * 8 + j; }
+      // softmax(z) with T = 1: e = exp(z - a)
+      const float E = __builtin_amdgcn_exp2f(fmaf(v[j], P.inv_c_l2, P.b_over_c_l2));
+      esum += __builtin_amdgcn_exp2f(-P.cap_a * 1.4426950408889634f * __builtin_amdgcn_rcpf(1.0f + E));
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+  }
+  esum = wave_sum(esum);
+  if (lane == 0) { smax[wave] = best; sidx[wave] = bi; ssum[wave] = esum; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float tot = 0.f;
+    for (int w = 0; w < 4; w++) {
+      tot += ssum[w];
+      if (smax[w] > best || (smax[w] == best && sidx[w] < bi)) { best = smax[w]; bi = sidx[w]; }
+    }
+    P.tok[row] = bi;
+    const float E = __builtin_amdgcn_exp2f(fmaf(best, P.inv_c_l2, P.b_over_c_l2));
+    P.logp[row] = -P.cap_a * __builtin_amdgcn_rcpf(1.0f + E) - __logf(tot);
+    if (P.u_out) P.u_out[row] = 0.f;
+  }
+}
+
+}  // namespace uvmi
+
+using namespace uvmi;
+
+extern "C" void uvmi_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) { philox4x32_10(ctr, key, out); }
+
+extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
+  UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_fused_sample: null args");
+  UVMI_REQUIRE(a->x && a->tok && a->logp, UVMI_EINVAL, "uvmi_fused_sample: null pointer");
+  UVMI_REQUIRE(is_float_dtype(a->x_dtype), UVMI_EINVAL, "uvmi_fused_sample: x_dtype must be a float type");
+  UVMI_REQUIRE(a->B >= 0 && a->V > 0 && a->stride >= a->V, UVMI_EINVAL, "uvmi_fused_sample: bad sizes");
+  UVMI_REQUIRE(a->V % CHUNK == 0 && a->V / CHUNK <= 64, UVMI_EUNSUPPORTED,
+               "uvmi_fused_sample: V=%d must be a multiple of 512 and at most 32768", a->V);
+  UVMI_REQUIRE(a->cap_c != 0.f, UVMI_EINVAL, "uvmi_fused_sample: softcap c must be non-zero");
+  const int eb = a->x_dtype == UVMI_F32 ? 4 : 2;
+  UVMI_REQUIRE(((uintptr_t)a->x % 16) == 0 && (a->stride * eb) % 16 == 0, UVMI_EUNSUPPORTED,
+               "uvmi_fused_sample: rows of x must be 16-byte aligned");
+  const bool greedy = !(a->temperature > 0.f);
+  if (!greedy) {
+    UVMI_REQUIRE(a->cap_a / a->temperature <= 80.0f, UVMI_EUNSUPPORTED, "uvmi_fused_sample: a/T = %g exceeds 80 (fp32 underflow)",
+                 (double)(a->cap_a / a->temperature));
+    UVMI_REQUIRE(a->u || (a->req_id && a->tok_idx), UVMI_EINVAL, "uvmi_fused_sample: need u or (req_id, tok_idx)");
+  }
+  if (a->B == 0) return UVMI_OK;
+  SampleParams P;
+  P.x = a->x; P.stride = a->stride; P.u = a->u; P.seed = a->seed; P.req_id = a->req_id; P.tok_idx = a->tok_idx;
+  P.tok = a->tok; P.logp = a->logp; P.u_out = a->u_out; P.V = a->V;
+  const float l2e = 1.4426950408889634f;
+  P.inv_c = 1.0f / a->cap_c;
+  P.inv_c_l2 = l2e / a->cap_c;
+  P.b_over_c_l2 = a->cap_b / a->cap_c * l2e;
+  const float T = greedy ? 1.0f : a->temperature;
+  P.neg_a_over_t = -a->cap_a / T;
+  P.neg_a_over_t_l2 = P.neg_a_over_t * l2e;
+  P.cap_a = a->cap_a; P.cap_b = a->cap_b; P.cap_c = a->cap_c;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(a->B), blk(256);
+#define UVMI_S(K)                                                                          \
+  do {                                                                                     \
+    if (a->x_dtype == UVMI_F16) hipLaunchKernelGGL((K<UVMI_F16>), grid, blk, 0, st, P);    \
+    else if (a->x_dtype == UVMI_BF16) hipLaunchKernelGGL((K<UVMI_BF16>), grid, blk, 0, st, P); \
+    else hipLaunchKernelGGL((K<UVMI_F32>), grid, blk, 0, st, P);                           \
+  } while (0)
+  if (greedy) UVMI_S(argmax_kernel); else UVMI_S(sample_kernel);
+#undef UVMI_S
+  UVMI_CHECK_LAUNCH("uvmi_fused_sample");
+  return UVMI_OK;
+}

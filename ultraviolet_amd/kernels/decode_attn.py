@@ -1,0 +1,115 @@
+"""Split-K single-query decode attention over a static, slot-indexed KV cache (MQA/GQA, ragged per-row positions,
+full-context or ring-buffer sliding-window caches, fp16/bf16 or int8 with per-token-per-head fp16 scales).
+
+Mirror of ultraviolet/kernels/decode_attn.py of the reference (`decode_attention`, `default_splits`, the
+`mathk::decode_attn` custom op); the kernels are in csrc/decode_attn.hip."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+from torch import Tensor
+
+from .. import _lib as L
+
+
+def default_splits(n_bk: int, ctx: int, device=None, min_chunk: int = 64, waves: int = 16) -> int:
+    """Splits per (row, kv head): enough wave64 work items for ~`waves` per compute unit, each chunk >= min_chunk keys
+    (reference: decode_attn.py:121-129, re-derived for 256 CUs)."""
+    if device is not None:
+        with torch.cuda.device(device):
+            cus = L.lib().uvmi_device_cus()
+    else:
+        cus = L.lib().uvmi_device_cus()
+    if cus <= 0:
+        raise L.UvmiError(L.lib().uvmi_last_error().decode())
+    want = -(-waves * cus // max(int(n_bk), 1))
+    return int(max(1, min(want, max(1, int(ctx) // min_chunk), 64)))
+
+
+def supported(q: Tensor, k_cache: Tensor) -> bool:
+    """True when the MFMA kernel serves this geometry (reference: decode_attn_cuda.supported,
+    decode_attn_cuda.py:265-270).  Other geometries run the generic kernel."""
+    H, hd = q.shape[-2], q.shape[-1]
+    G = H // k_cache.shape[1]
+    return bool(q.is_cuda and hd == 64 and 1 <= G <= 8 and k_cache.dtype == torch.int8
+                and q.dtype in (torch.float16, torch.bfloat16))
+
+
+def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out):
+    B, H, hd = q.shape
+    KH, S = k_cache.shape[1], k_cache.shape[2]
+    int8 = k_cache.dtype == torch.int8
+    assert q.stride(-1) == 1 and k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1 and out.stride(-1) == 1
+    if int8:
+        assert k_scale is not None and v_scale is not None and k_scale.stride(-1) == 1 and v_scale.stride(-1) == 1
+    assert pos.dtype == starts.dtype and pos.is_contiguous() and starts.is_contiguous()
+    ws, ws_bytes = None, 0
+    if num_splits > 1:
+        ws_bytes = L.lib().uvmi_decode_attn_workspace_bytes(B, H, KH, hd, num_splits)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    a = L.AttnArgs()
+    a.q, a.q_dtype, a.sqb, a.sqh = q.data_ptr(), L.dtype_code(q.dtype), q.stride(0), q.stride(1)
+    a.k_cache, a.v_cache, a.kv_dtype = k_cache.data_ptr(), v_cache.data_ptr(), L.dtype_code(k_cache.dtype)
+    a.skb, a.skh, a.sks = k_cache.stride(0), k_cache.stride(1), k_cache.stride(2)
+    a.svb, a.svh, a.svs = v_cache.stride(0), v_cache.stride(1), v_cache.stride(2)
+    if int8:
+        a.k_scale, a.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
+        a.ssb, a.ssh, a.stb, a.sth = k_scale.stride(0), k_scale.stride(1), v_scale.stride(0), v_scale.stride(1)
+    a.pos, a.starts, a.idx_dtype = pos.data_ptr(), starts.data_ptr(), L.dtype_code(pos.dtype)
+    a.out, a.out_dtype, a.sob, a.soh = out.data_ptr(), L.dtype_code(out.dtype), out.stride(0), out.stride(1)
+    a.B, a.H, a.KH, a.S, a.hd = B, H, KH, S, hd
+    a.scale, a.window, a.ring, a.num_splits = float(scale), int(window), int(bool(ring)), int(num_splits)
+    a.workspace, a.workspace_bytes = (ws.data_ptr() if ws is not None else None), ws_bytes
+    L.check(L.lib().uvmi_decode_attn(C.byref(a), L.stream_ptr(q)), "uvmi_decode_attn")
+    return out
+
+
+@torch.library.custom_op("uvmi::decode_attn", mutates_args=())
+def _decode_attn_op(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float,
+                    window: int, ring: bool, k_scale: Tensor | None, v_scale: Tensor | None, num_splits: int,
+                    out_fp32: bool) -> Tensor:
+    out = torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
+    return _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out)
+
+
+@_decode_attn_op.register_fake
+def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out_fp32):
+    return torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
+
+
+def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float, *,
+                     window: int = 0, ring: bool | None = None, k_scale: Tensor | None = None,
+                     v_scale: Tensor | None = None, ctx_hint: int | None = None, num_splits: int | None = None,
+                     block_n: int | None = None, num_warps: int = 1, backend: str = "auto",
+                     out_fp32: bool = False) -> Tensor:
+    """Single-query attention for every row of a static KV cache (reference: decode_attn.py:193-230).
+
+    q        (B, H, hd) fp16 or bf16 (any (B, 1, H, hd) view is accepted); H = K * G, query head h*G+g uses kv head h.
+    k_cache, v_cache  (B, K, S, hd) fp16/bf16, or int8 with k_scale / v_scale (B, K, S) fp16.
+    pos      (B,) int: position of the current (last) key, already written to the cache.  Keys attended:
+             positions max(starts[b], pos[b] - window + 1, 0) .. pos[b] (window 0 = unlimited).
+    starts   (B,) int: first valid (non-pad) position of each row.
+    ring     slot of position t is t % S (default: window > 0); else slot t (needs pos < S).
+    ctx_hint static upper bound on keys per row (e.g. g_len, or the window) for choosing num_splits.
+    block_n, num_warps, backend  accepted for signature compatibility; the HIP kernels choose their own tiling
+             ("hip" / "auto" / "cuda" / "triton" all run the HIP path).
+    out_fp32 return the fp32 result before rounding to q.dtype (for parity checks).
+    Returns (B, H, hd) in q.dtype.  Graph-capturable; registered as a torch custom op (opaque to torch.compile)."""
+    if q.dim() == 4:
+        q = q.reshape(q.size(0), q.size(-2), q.size(-1))
+    L.require_cuda(q, k_cache, v_cache, pos, starts)
+    B, H, hd = q.shape
+    KH, S = k_cache.shape[1], k_cache.shape[2]
+    if ring is None:
+        ring = window > 0
+    if num_splits is None:
+        ctx = ctx_hint or S
+        if window > 0:
+            ctx = min(ctx, window)
+        num_splits = default_splits(B * KH, ctx, q.device)
+    q = q.contiguous() if q.stride(-1) != 1 else q
+    if pos.dtype != starts.dtype:
+        starts = starts.to(pos.dtype)
+    return _decode_attn_op(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window),
+                           bool(ring), k_scale, v_scale, int(num_splits), bool(out_fp32))
