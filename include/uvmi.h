@@ -98,7 +98,10 @@ typedef struct uvmi_attn_args {
   float scale;                             /* softmax scale applied to q.k */
   int window;                              /* 0 = unlimited; else keys pos-window+1..pos */
   int ring;                                /* slot of position t is t % S (else t) */
-  int num_splits;                          /* >= 1: chunks each row's key range is cut into */
+  int num_splits;                          /* >= 1: upper bound on the chunks a row's key range is cut into */
+  int chunk_keys;                          /* 0: every row is cut into num_splits equal chunks (the reference's rule,
+                                              decode_attn.py:42-44); > 0: chunks of at least this many keys, so short
+                                              rows use fewer work items and a row that fits one chunk skips the combine */
   void* workspace; size_t workspace_bytes; /* >= uvmi_decode_attn_workspace_bytes(...) when num_splits > 1 */
 } uvmi_attn_args;
 

@@ -214,7 +214,7 @@ def test_quantize_fp32_rows_and_zero_row():
     assert np.array_equal(to_np(q), rq) and np.array_equal(to_np(s).view(np.uint16), rs.view(np.uint16))
     assert (to_np(q)[0, 0] == 0).all()
     # reference bound, tests/test_math_kernels.py:115-121
-    xh = x.half()
+    xh = x.clamp(-100, 100).half()  # 7e4 is not finite in fp16
     q, s = quantize_kv(xh.to(DEV))
     err = (dequantize_kv(q, s).float().cpu() - xh.float()).abs()
     assert err.max() <= (s.float().cpu().unsqueeze(-1) * 0.5 + 1e-3).max()
@@ -307,7 +307,10 @@ def test_sampler_matches_ref(T, dtype, V):
     t, lp = t.cpu(), lp.cpu()
     tr, lpr = fs.fused_sample_ref(to_np(x), u.numpy(), SC, T)
     assert t.dtype == torch.int64 and t.min() >= 0 and t.max() < V
-    assert (t.numpy() == tr).mean() > 0.99
+    # The oracle's flat sequential fp32 cumsum and the kernel's chunk / lane / element sums are different summation
+    # orders of the same masses, so tokens agree only up to fp32 summation error (which grows with V for the flat
+    # sum); the order-independent checks are agreement with the float64 inverse-CDF draw and its CDF interval.
+    assert (t.numpy() == tr).mean() > 0.9
     z = torch.from_numpy(fs.softcap(to_np(x), SC)).double()
     e = torch.exp((z - SC[0]) / T)
     cs = e.cumsum(-1)
@@ -317,6 +320,8 @@ def test_sampler_matches_ref(T, dtype, V):
     lo = hi - e.gather(1, t[:, None])[:, 0]
     tol = 1e-5 * S
     assert ((tgt >= lo - tol) & (tgt <= hi + tol)).all()
+    t64 = torch.searchsorted(cs, tgt[:, None]).squeeze(1).clamp_(max=V - 1)
+    assert (t == t64).float().mean() > 0.99
     ls = torch.log_softmax(z / T, -1).gather(1, t[:, None])[:, 0]
     assert (lp.double() - ls).abs().max() < 2e-5
 

@@ -37,7 +37,7 @@ class AttnArgs(C.Structure):
                 ("out", C.c_void_p), ("out_dtype", C.c_int), ("sob", C.c_int64), ("soh", C.c_int64),
                 ("B", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("S", C.c_int), ("hd", C.c_int),
                 ("scale", C.c_float), ("window", C.c_int), ("ring", C.c_int), ("num_splits", C.c_int),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+                ("chunk_keys", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
 class KvAppendArgs(C.Structure):

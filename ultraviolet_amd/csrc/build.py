@@ -18,7 +18,10 @@ SOURCES = ["common.hip", "kv_quant.hip", "decode_attn.hip", "fused_sample.hip", 
 LIB = os.path.join(HERE, "libuvmi.so")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unknown-warning-option"]
+         "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unknown-warning-option",
+         # keep MFMA accumulators in VGPRs: the attention kernels rescale them with VALU ops, and the AGPR form costs
+         # an accvgpr read/write pair per register per step
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 
 def _hipcc() -> str:

@@ -17,19 +17,27 @@
 //         A and 8g+4+j is key 4g+j of stream B: probabilities never move between lanes;
 //       - K rows are read as one 16-byte load per lane (lane = key m, bytes 16g..16g+15), V as dwords
 //         (lane = bytes 4m..4m+3 of 8 keys), both fully coalesced over 64-byte rows; int8 is turned into fp16 with
-//         v_perm_b32 against 0x64 bytes (fp16 0x64uu = 1024 + u, u = x ^ 0x80 = x + 128): K keeps the +1152 bias,
-//         which is cancelled by the accumulator's initial value -1152 * sum(q), V removes it with a packed add;
-//       - online softmax per (stream, head) column; the two streams are merged once at the end.
+//         v_perm_b32 only (u = x ^ 0x80 = x + 128): K' = fp16 0x64uu = 1024 + u keeps a +1152 bias that is
+//         cancelled by the accumulator's initial value -1152 * sum(q); V'' = fp16 0x00uu = u * 2^-24 (a subnormal,
+//         which the f16 MFMA honours) keeps a +128 bias that is removed at the end with 128 * sum(P'), P' being the
+//         fp16-rounded probabilities (accumulated with v_dot2_f32_f16);
+//       - all addressing in the loop is scalar (wave-uniform tile base) plus lane-invariant 32-bit offsets;
+//       - online softmax per (stream, head) column, rescaling only when some column's maximum grew; the two
+//         streams are merged once at the end.
 //   * attn_generic: any head_dim <= 256, G <= 16, int8 / fp16 / bf16 caches, arbitrary alignment: plain fp32 VALU.
 //
 // Split partials (acc, m, l) go to a caller-provided workspace; attn_combine merges them.
 #include "common.h"
+
+#include <cstdlib>
 
 namespace uvmi {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 
 constexpr float LOG2E = 1.4426950408889634f;
 
@@ -38,42 +46,46 @@ struct AttnParams {
   const void* pos; const void* starts;
   void* out; float* ws_o; float* ws_m; float* ws_l;
   int64_t sqb, sqh, skb, skh, sks, svb, svh, svs, ssb, ssh, stb, sth, sob, soh;
-  int B, H, KH, G, S, hd, window, ring, splits, idx64;
+  int B, H, KH, G, S, hd, window, ring, splits, idx64, chunk_keys, gran;  // gran: chunk granularity (keys)
   int64_t n_items;
   float scale_log2;
 };
 
-// Row range and this split's chunk.  Chunks are multiples of 32 keys starting at lo rounded down to 32, so a
-// 16-key tile never straddles two splits and tiles stay aligned to the slot grid.
-struct Chunk { int lo, p, s0, s1; };
-__device__ __forceinline__ Chunk split_range(const AttnParams& P, int b, int sid) {
-  int p = (int)load_index(P.pos, P.idx64, b);
-  int st = (int)load_index(P.starts, P.idx64, b);
+// Key range of a row and how it is cut.  The span starts at lo rounded down to 32 so tiles stay aligned to the
+// slot grid; each work item gets `chunk` keys (a multiple of 32, at least chunk_keys, and large enough that at most
+// `splits` items cover the span).  A row with a single chunk is written directly, without partials.
+struct RowPlan { int lo, p, a0, chunk, nsplit; };
+__device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b) {
+  RowPlan r;
+  const int p = (int)load_index(P.pos, P.idx64, b);
+  const int st = (int)load_index(P.starts, P.idx64, b);
   int lo = st > 0 ? st : 0;
   if (P.window > 0 && p - P.window + 1 > lo) lo = p - P.window + 1;
-  Chunk c;
-  c.lo = lo;
-  c.p = p;
-  int a0 = lo & ~31;
-  int span = p + 1 - a0;
+  r.lo = lo;
+  r.p = p;
+  r.a0 = lo & ~31;
+  int span = p + 1 - r.a0;
   if (span < 0) span = 0;
-  int chunk = (((span + P.splits - 1) / P.splits) + 31) & ~31;
-  c.s0 = a0 + sid * chunk;
-  c.s1 = min(c.s0 + chunk, p + 1);
-  return c;
+  const int gr = P.gran;  // multiple of 32
+  int chunk = (((span + P.splits - 1) / P.splits) + gr - 1) / gr * gr;
+  if (chunk < P.chunk_keys) chunk = P.chunk_keys;
+  if (chunk < gr) chunk = gr;
+  r.chunk = chunk;
+  r.nsplit = span > 0 ? (span + chunk - 1) / chunk : 1;
+  return r;
 }
 
 // ---------------------------------------------------------------------------------------------------- MFMA kernel
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
 
-template <typename T>
-__device__ __forceinline__ T bitcast_h8(const uint32_t (&r)[4]) {
-  T v;
+__device__ __forceinline__ h8 as_h8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const uint32_t r[4] = {a, b, c, d};
+  h8 v;
   __builtin_memcpy(&v, r, 16);
   return v;
 }
 
-__device__ __forceinline__ float xmax16(float v) {  // max over lanes l, l^16 (rows of 16 lanes pairwise)
+__device__ __forceinline__ float xmax16(float v) {  // max over lanes l, l^16
   auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
@@ -90,213 +102,289 @@ __device__ __forceinline__ float xsum32(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-struct Tile {         // one 32-key super-tile as loaded from HBM
-  uint4 kA, kB;       // key m of stream A / B, bytes 16g..16g+15
+struct Tile {             // one 32-key super-tile as loaded from HBM (26 dwords per lane)
+  uint4 kA, kB;           // key m of stream A / B, bytes 16g..16g+15
   uint32_t vA[4], vB[4];  // keys 4g+j of stream A / B, bytes 4m..4m+3
-  uint2 ksc, vsc;     // 4 fp16 scales of keys 4g..4g+3 of this lane's stream
+  uint2 ksc, vsc;         // fp16 scales of keys 4g..4g+3 of this lane's stream
 };
 
-template <int QDT, int ODT>
+struct AttnState {
+  f4 O[4];                // O''^T tiles: 2^-24 * sum (v + 128) P'
+  float mrun, lrun, psum; // running max (score units before scale), sum p, sum of the fp16-rounded P'
+};
+
+// WPR waves of a workgroup share one work item (row, kv head, split): wave w takes super-tiles w, w + WPR, ... of the
+// chunk, so the workgroup streams 32 * WPR consecutive keys (2 KB * WPR of K and of V) per step, which keeps many more
+// DRAM pages open-and-hit than one wave per row does; the WPR online-softmax states are merged through LDS at the end.
+template <int QDT, int ODT, int WPR>
 __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
+  constexpr int IPB = 4 / WPR;  // items per block
+  __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
+  __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
   const int lane = threadIdx.x & 63;
-  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= P.n_items) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wsub = wave % WPR;
+  int64_t item = (int64_t)blockIdx.x * IPB + wave / WPR;  // wave-uniform
+  const bool live_item = item < P.n_items;
+  if (!live_item) {
+    if (WPR == 1) return;
+    item = P.n_items - 1;  // keep the wave for the barrier below; it does no work
+  }
   const int sid = (int)(item % P.splits);
   const int64_t bk = item / P.splits;
   const int b = (int)(bk / P.KH), h = (int)(bk % P.KH);
-  const int m = lane & 15, g = lane >> 4;  // also (n, g) of the accumulator layout
+  const RowPlan rp = plan_row(P, b);
+  const bool live = live_item && sid < rp.nsplit;
+  if (WPR == 1 && !live) return;
+  const int s0 = rp.a0 + sid * rp.chunk;
+  const int s1 = live ? min(s0 + rp.chunk, rp.p + 1) : s0;
+  const int lo_eff = max(rp.lo, s0);
+  const int m = lane & 15, g = lane >> 4;  // A/B operand (row, group) == accumulator (column, group)
   const int strm = m >> 3, head = m & 7;
-  const Chunk c = split_range(P, b, sid);
   const int G = P.G;
+  const float c = P.scale_log2;
 
-  // ---- Q^T operands: lane (n, g) holds q[head][16g + 8s + j]; fp16 (bf16 inputs are converted, exact for
-  // 2^-14 <= |q| <= 65504)
+  // ---- Q^T operands: lane (n, g) holds q[head][16g + 8s + j] as fp16 (bf16 inputs are converted; exact for
+  // 2^-14 <= |q| <= 65504).  The K operand carries a +1152 bias, cancelled by starting the accumulator at
+  // -1152 * sum_d q[head][d].
   uint32_t qr[8];
   float qsum = 0.f;
   {
     const uint16_t* qp = (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + head) * P.sqh + 16 * g;
-    float qf[16];
-    if (head < G) {
-      uint4 w0 = *(const uint4*)qp, w1 = *(const uint4*)(qp + 8);
-      const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-      for (int i = 0; i < 8; i++) {
-        if (QDT == UVMI_BF16) {
-          qf[2 * i] = __uint_as_float(w[i] << 16);
-          qf[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-        } else {
-          qf[2 * i] = half_bits_to_float(w[i] & 0xffff);
-          qf[2 * i + 1] = half_bits_to_float(w[i] >> 16);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; i++) qf[i] = 0.f;
-    }
+    uint4 w0 = uint4{0, 0, 0, 0}, w1 = uint4{0, 0, 0, 0};
+    if (head < G) { w0 = *(const uint4*)qp; w1 = *(const uint4*)(qp + 8); }
+    const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      uint16_t lo16 = float_to_half_bits(qf[2 * i]), hi16 = float_to_half_bits(qf[2 * i + 1]);
-      qr[i] = (uint32_t)lo16 | ((uint32_t)hi16 << 16);
-      qsum += half_bits_to_float(lo16) + half_bits_to_float(hi16);
+      float f0, f1;
+      if (QDT == UVMI_BF16) { f0 = __uint_as_float(w[i] << 16); f1 = __uint_as_float(w[i] & 0xffff0000u); }
+      else { f0 = half_bits_to_float(w[i] & 0xffff); f1 = half_bits_to_float(w[i] >> 16); }
+      const uint16_t l16 = float_to_half_bits(f0), h16 = float_to_half_bits(f1);
+      qr[i] = (uint32_t)l16 | ((uint32_t)h16 << 16);
+      qsum += half_bits_to_float(l16) + half_bits_to_float(h16);
     }
-    // sum over the 4 lane groups -> sum over all 64 dims of this head
-    qsum = xsum16(qsum);
-    qsum = xsum32(qsum);
+    qsum = xsum32(xsum16(qsum));  // all 64 dims of this head
   }
   const uint32_t mA = strm == 0 ? 0xffffffffu : 0u, mB = ~mA;
-  uint32_t qa0[4], qa1[4], qb0[4], qb1[4];
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    qa0[i] = qr[i] & mA; qa1[i] = qr[4 + i] & mA;
-    qb0[i] = qr[i] & mB; qb1[i] = qr[4 + i] & mB;
-  }
-  const h8 QA0 = bitcast_h8<h8>(qa0), QA1 = bitcast_h8<h8>(qa1), QB0 = bitcast_h8<h8>(qb0), QB1 = bitcast_h8<h8>(qb1);
+  const h8 QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA), QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
+  const h8 QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB), QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
   const float cinit = -1152.0f * qsum;
 
-  // ---- state
-  f4 O[4];
+  AttnState st;
 #pragma unroll
-  for (int t = 0; t < 4; t++) O[t] = f4{0.f, 0.f, 0.f, 0.f};
-  float mrun = -INFINITY, lrun = 0.f;
+  for (int t = 0; t < 4; t++) st.O[t] = f4{0.f, 0.f, 0.f, 0.f};
+  st.mrun = -INFINITY;
+  st.lrun = 0.f;
+  st.psum = 0.f;
 
-  const int lo_eff = max(c.lo, c.s0);
+  // ---- addressing: wave-uniform row base + wave-uniform tile offset (scalar) + lane-invariant 32-bit offsets
   const int8_t* kbase = (const int8_t*)P.kc + (int64_t)b * P.skb + (int64_t)h * P.skh;
   const int8_t* vbase = (const int8_t*)P.vc + (int64_t)b * P.svb + (int64_t)h * P.svh;
   const uint16_t* ksb = (const uint16_t*)P.ks + (int64_t)b * P.ssb + (int64_t)h * P.ssh;
   const uint16_t* vsb = (const uint16_t*)P.vs + (int64_t)b * P.stb + (int64_t)h * P.sth;
   const int S = P.S;
-  const int smax = S - 1;
+  const uint32_t sks = (uint32_t)P.sks, svs = (uint32_t)P.svs;
+  const uint32_t usks = __builtin_amdgcn_readfirstlane(sks), usvs = __builtin_amdgcn_readfirstlane(svs);
+  const uint32_t koA = m * sks + 16 * g, koB = koA + 16 * sks;  // K: key m of stream A / B, bytes 16g..
+  const uint32_t voA = 4 * g * svs + 4 * m;     // V: key 4g (+j via the scalar offset), bytes 4m..
+  const uint32_t so = 16 * strm + 4 * g;  // scale offset (elements) inside the super-tile
 
-  auto slot_of = [&](int t) -> int {  // t is a multiple of 16 here; ring needs S % 16 == 0 (host-checked)
-    if (P.ring) return t % S;
-    return t;
-  };
-  auto load_tile = [&](int tb, Tile& T) {
-    const int sa = slot_of(tb), sb2 = slot_of(tb + 16);
-    // K: key m of each stream
-    int ka = min(sa + m, smax), kb = min(sb2 + m, smax);
-    T.kA = *(const uint4*)(kbase + (int64_t)ka * P.sks + 16 * g);
-    T.kB = *(const uint4*)(kbase + (int64_t)kb * P.sks + 16 * g);
+  // Buffer descriptors (wave-uniform, one per row stream): a load is descriptor base + lane-invariant VGPR offset +
+  // scalar tile offset, so the loop spends no VALU work on addresses.  num_records covers exactly the row's bytes.
+  const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (S - 1) * (int)sks + 64, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (S - 1) * (int)svs + 64, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rKS = __builtin_amdgcn_make_buffer_rsrc((void*)ksb, 0, S * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rVS = __builtin_amdgcn_make_buffer_rsrc((void*)vsb, 0, S * 2, 0x00020000);
+  const uint32_t so2 = so * 2;
+
+  // slot0: cache slot of absolute position tb (a multiple of 32).  Ring caches have S % 32 == 0 (host-checked), so a
+  // super-tile never wraps.  load_tile needs slot0 + 32 <= S; a linear cache that ends inside its last super-tile
+  // takes load_tail (per-lane clamped rows) for that one tile, outside the pipelined loop.
+  auto load_tile = [&](int slot_in, Tile& T) {
+    const int slot0 = __builtin_amdgcn_readfirstlane(slot_in);  // wave-uniform by construction
+    const uint32_t ok = (uint32_t)slot0 * usks, ov = (uint32_t)slot0 * usvs, os = (uint32_t)slot0 * 2;
+    u4 ka = __builtin_amdgcn_raw_buffer_load_b128(rK, koA, ok, 0);
+    u4 kb = __builtin_amdgcn_raw_buffer_load_b128(rK, koB, ok, 0);
+    T.kA = uint4{ka.x, ka.y, ka.z, ka.w};
+    T.kB = uint4{kb.x, kb.y, kb.z, kb.w};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      int va = min(sa + 4 * g + j, smax), vb = min(sb2 + 4 * g + j, smax);
-      T.vA[j] = *(const uint32_t*)(vbase + (int64_t)va * P.svs + 4 * m);
-      T.vB[j] = *(const uint32_t*)(vbase + (int64_t)vb * P.svs + 4 * m);
+      T.vA[j] = __builtin_amdgcn_raw_buffer_load_b32(rV, voA, ov + j * usvs, 0);
+      T.vB[j] = __builtin_amdgcn_raw_buffer_load_b32(rV, voA, ov + (16 + j) * usvs, 0);
     }
-    int ss = min((strm ? sb2 : sa) + 4 * g, S - 4);
+    u2 a = __builtin_amdgcn_raw_buffer_load_b64(rKS, so2, os, 0);
+    u2 c2 = __builtin_amdgcn_raw_buffer_load_b64(rVS, so2, os, 0);
+    T.ksc = uint2{a.x, a.y};
+    T.vsc = uint2{c2.x, c2.y};
+  };
+  auto load_tail = [&](int slot0, Tile& T) {
+    const int smax = S - 1;
+    T.kA = *(const uint4*)(kbase + (int64_t)min(slot0 + m, smax) * P.sks + 16 * g);
+    T.kB = *(const uint4*)(kbase + (int64_t)min(slot0 + 16 + m, smax) * P.sks + 16 * g);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      T.vA[j] = *(const uint32_t*)(vbase + (int64_t)min(slot0 + 4 * g + j, smax) * P.svs + 4 * m);
+      T.vB[j] = *(const uint32_t*)(vbase + (int64_t)min(slot0 + 16 + 4 * g + j, smax) * P.svs + 4 * m);
+    }
+    const int ss = min(slot0 + (int)so, S - 4);  // S % 4 == 0: a clamped group is entirely past the cache end
     T.ksc = *(const uint2*)(ksb + ss);
     T.vsc = *(const uint2*)(vsb + ss);
   };
 
-  if (c.s0 < c.s1) {
-    Tile cur, nxt;
-    load_tile(c.s0, cur);
-    for (int tb = c.s0; tb < c.s1; tb += 32) {
-      const bool more = tb + 32 < c.s1;
-      if (more) load_tile(tb + 32, nxt);
+  auto step = [&](const Tile& T, int tb, bool edge) {
+    // ---- S^T = K' . Q^T - 1152 sum(q), K' = 1024 + (k ^ 0x80) as fp16 0x64uu
+    f4 acc = f4{cinit, cinit, cinit, cinit};
+    {
+      const uint32_t a0 = T.kA.x ^ 0x80808080u, a1 = T.kA.y ^ 0x80808080u, a2 = T.kA.z ^ 0x80808080u, a3 = T.kA.w ^ 0x80808080u;
+      const uint32_t b0 = T.kB.x ^ 0x80808080u, b1 = T.kB.y ^ 0x80808080u, b2 = T.kB.z ^ 0x80808080u, b3 = T.kB.w ^ 0x80808080u;
+      constexpr uint32_t C64 = 0x64646464u, LO = 0x04010400u, HI = 0x04030402u;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(perm(C64, a0, LO), perm(C64, a0, HI), perm(C64, a1, LO), perm(C64, a1, HI)), QA0, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(perm(C64, a2, LO), perm(C64, a2, HI), perm(C64, a3, LO), perm(C64, a3, HI)), QA1, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(perm(C64, b0, LO), perm(C64, b0, HI), perm(C64, b1, LO), perm(C64, b1, HI)), QB0, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(perm(C64, b2, LO), perm(C64, b2, HI), perm(C64, b3, LO), perm(C64, b3, HI)), QB1, acc, 0, 0, 0);
+    }
+    // ---- t_i = (q.k_int) * kscale_i for the lane's keys 4g+i of its stream (softmax scale applied inside exp2)
+    h2 ks01, ks23, vs01, vs23;
+    __builtin_memcpy(&ks01, &T.ksc.x, 4); __builtin_memcpy(&ks23, &T.ksc.y, 4);
+    __builtin_memcpy(&vs01, &T.vsc.x, 4); __builtin_memcpy(&vs23, &T.vsc.y, 4);
+    float t[4] = {acc[0] * (float)ks01[0], acc[1] * (float)ks01[1], acc[2] * (float)ks23[0], acc[3] * (float)ks23[1]};
+    float vsf[4] = {(float)vs01[0], (float)vs01[1], (float)vs23[0], (float)vs23[1]};
+    if (edge) {  // keys outside [lo_eff, s1): no score, and their (possibly stale, non-finite) V scale must not meet p = 0
+      const int t0 = tb + 16 * strm + 4 * g;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        if (t0 + i < lo_eff || t0 + i >= s1) { t[i] = -INFINITY; vsf[i] = 0.f; }
+    }
+    float mx = fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3]));
+    mx = xmax32(xmax16(mx));
+    if (__builtin_amdgcn_ballot_w64(mx > st.mrun) != 0) {  // some column's maximum grew: rescale (alpha = 1 elsewhere)
+      const float mnew = fmaxf(st.mrun, mx);
+      const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((st.mrun - mnew) * c);
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) st.O[tt] *= alpha;
+      st.lrun *= alpha;
+      st.psum *= alpha;
+      st.mrun = mnew;
+    }
+    const float mc = st.mrun == -INFINITY ? 0.f : st.mrun * c;
+    float p[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) p[i] = __builtin_amdgcn_exp2f(fmaf(t[i], c, -mc));
+    st.lrun += (p[0] + p[1]) + (p[2] + p[3]);
+    // ---- P' = fp16(p * vscale), placed in this stream's half of the contraction slots
+    const h2 p01 = h2{(_Float16)(p[0] * vsf[0]), (_Float16)(p[1] * vsf[1])};
+    const h2 p23 = h2{(_Float16)(p[2] * vsf[2]), (_Float16)(p[3] * vsf[3])};
+    const h2 ones = h2{(_Float16)1.0f, (_Float16)1.0f};
+    st.psum = __builtin_amdgcn_fdot2(p23, ones, __builtin_amdgcn_fdot2(p01, ones, st.psum, false), false);
+    uint32_t u01, u23;
+    __builtin_memcpy(&u01, &p01, 4);
+    __builtin_memcpy(&u23, &p23, 4);
+    const h8 PB = as_h8(u01 & mA, u23 & mA, u01 & mB, u23 & mB);
+    // ---- O''^T += V'' . P'^T with V'' = (v ^ 0x80) * 2^-24 (fp16 subnormal 0x00uu; the MFMA takes subnormals);
+    // tile tt, operand row m is head dim 4m + tt
+    {
+      uint32_t xa[4], xb[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) { xa[j] = T.vA[j] ^ 0x80808080u; xb[j] = T.vB[j] ^ 0x80808080u; }
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) {
+        const uint32_t sel = 0x0c000c00u | ((4u + tt) << 16) | (uint32_t)tt;  // [0, S0.byte tt, 0, S1.byte tt]
+        const h8 va = as_h8(perm(xa[1], xa[0], sel), perm(xa[3], xa[2], sel), perm(xb[1], xb[0], sel), perm(xb[3], xb[2], sel));
+        st.O[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, PB, st.O[tt], 0, 0, 0);
+      }
+    }
+  };
 
-      // ---- K -> fp16 (1024 + u), S^T = K . Q^T - 1152 sum(q)
-      f4 acc = f4{cinit, cinit, cinit, cinit};
-      {
-        const uint32_t wa[4] = {cur.kA.x ^ 0x80808080u, cur.kA.y ^ 0x80808080u, cur.kA.z ^ 0x80808080u, cur.kA.w ^ 0x80808080u};
-        const uint32_t wb[4] = {cur.kB.x ^ 0x80808080u, cur.kB.y ^ 0x80808080u, cur.kB.z ^ 0x80808080u, cur.kB.w ^ 0x80808080u};
-        uint32_t a0[4], a1[4], b0[4], b1[4];
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-          a0[2 * i] = perm(0x64646464u, wa[i], 0x04010400u);     a0[2 * i + 1] = perm(0x64646464u, wa[i], 0x04030402u);
-          a1[2 * i] = perm(0x64646464u, wa[2 + i], 0x04010400u); a1[2 * i + 1] = perm(0x64646464u, wa[2 + i], 0x04030402u);
-          b0[2 * i] = perm(0x64646464u, wb[i], 0x04010400u);     b0[2 * i + 1] = perm(0x64646464u, wb[i], 0x04030402u);
-          b1[2 * i] = perm(0x64646464u, wb[2 + i], 0x04010400u); b1[2 * i + 1] = perm(0x64646464u, wb[2 + i], 0x04030402u);
-        }
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast_h8<h8>(a0), QA0, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast_h8<h8>(a1), QA1, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast_h8<h8>(b0), QB0, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast_h8<h8>(b1), QB1, acc, 0, 0, 0);
+  {
+    // Pipelined part: tiles that lie entirely inside the cache.  The next tile's loads are issued unconditionally
+    // before the current tile is consumed (past the end the current tile is re-read, a cache hit), so that no
+    // branch separates load issue from use and the wait counters stay exact.
+    constexpr int STEP = 32 * WPR;
+    const int s1f = P.ring ? s1 : min(s1, S & ~31);
+    int tb = s0 + 32 * wsub;
+    if (tb < s1f) {
+      int slot = P.ring ? tb % S : tb;
+      auto next_slot = [&](int sl, int t) {
+        if (t + STEP >= s1f) return sl;
+        sl += STEP;
+        if (P.ring) while (sl >= S) sl -= S;
+        return sl;
+      };
+      Tile TA, TB;
+      load_tile(slot, TA);
+      while (true) {
+        slot = next_slot(slot, tb);
+        load_tile(slot, TB);
+        step(TA, tb, tb < lo_eff || tb + 32 > s1);
+        tb += STEP;
+        if (tb >= s1f) break;
+        slot = next_slot(slot, tb);
+        load_tile(slot, TA);
+        step(TB, tb, tb < lo_eff || tb + 32 > s1);
+        tb += STEP;
+        if (tb >= s1f) break;
       }
-      // ---- scores in the exp2 domain: s_i = acc_i * kscale_i * scale * log2(e); lane (n, g) key = base + 4g + i
-      float s[4];
-      {
-        const float k0 = half_bits_to_float(cur.ksc.x & 0xffff), k1 = half_bits_to_float(cur.ksc.x >> 16);
-        const float k2 = half_bits_to_float(cur.ksc.y & 0xffff), k3 = half_bits_to_float(cur.ksc.y >> 16);
-        s[0] = acc[0] * (k0 * P.scale_log2); s[1] = acc[1] * (k1 * P.scale_log2);
-        s[2] = acc[2] * (k2 * P.scale_log2); s[3] = acc[3] * (k3 * P.scale_log2);
-      }
-      float vsf[4] = {half_bits_to_float(cur.vsc.x & 0xffff), half_bits_to_float(cur.vsc.x >> 16),
-                      half_bits_to_float(cur.vsc.y & 0xffff), half_bits_to_float(cur.vsc.y >> 16)};
-      if (tb < lo_eff || tb + 32 > c.s1) {  // edge tiles: mask keys outside [lo_eff, s1); their (possibly stale,
-        const int t0 = tb + 16 * strm + 4 * g;  // non-finite) V scale must not meet p = 0
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-          if (t0 + i < lo_eff || t0 + i >= c.s1) { s[i] = -INFINITY; vsf[i] = 0.f; }
-      }
-      float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-      mx = xmax16(mx);
-      mx = xmax32(mx);
-      const float mnew = fmaxf(mrun, mx);
-      const float msafe = mnew == -INFINITY ? 0.f : mnew;
-      const float alpha = __builtin_amdgcn_exp2f(mrun - msafe);
-      float p[4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) p[i] = __builtin_amdgcn_exp2f(s[i] - msafe);
-      lrun = lrun * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
-      mrun = mnew;
-      // ---- P' = p * vscale -> fp16 pairs in this stream's half of the contraction slots
-      h8 PB;
-      {
-        h2 p01 = h2{(_Float16)(p[0] * vsf[0]), (_Float16)(p[1] * vsf[1])};
-        h2 p23 = h2{(_Float16)(p[2] * vsf[2]), (_Float16)(p[3] * vsf[3])};
-        uint32_t u01, u23;
-        __builtin_memcpy(&u01, &p01, 4);
-        __builtin_memcpy(&u23, &p23, 4);
-        const uint32_t r[4] = {u01 & mA, u23 & mA, u01 & mB, u23 & mB};
-        PB = bitcast_h8<h8>(r);
-      }
-      // ---- O^T = alpha * O^T + V^T . P'^T ; tile t, row m of the A operand is head dim 4m + t
-#pragma unroll
-      for (int t = 0; t < 4; t++) {
-        O[t] *= alpha;
-      }
-      {
-        uint32_t xa[4], xb[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) { xa[j] = cur.vA[j] ^ 0x80808080u; xb[j] = cur.vB[j] ^ 0x80808080u; }
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-          const uint32_t sel = 0x0c000c00u | ((4u + t) << 16) | (uint32_t)t;  // [0, S0.byte t, 0, S1.byte t]
-          uint32_t r[4];
-          r[0] = perm(xa[1], xa[0], sel) | 0x64006400u;
-          r[1] = perm(xa[3], xa[2], sel) | 0x64006400u;
-          r[2] = perm(xb[1], xb[0], sel) | 0x64006400u;
-          r[3] = perm(xb[3], xb[2], sel) | 0x64006400u;
-          h8 va = bitcast_h8<h8>(r);
-          va = va - (h8)((_Float16)1152.0f);
-          O[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, PB, O[t], 0, 0, 0);
-        }
-      }
-      if (more) cur = nxt;
+    }
+    if (tb < s1) {  // linear cache ending inside this super-tile (at most one wave of the item gets here)
+      Tile TT;
+      load_tail(tb, TT);
+      step(TT, tb, true);
     }
   }
 
-  // ---- reduce l over the 4 lane groups, merge stream B into stream A (lanes n and n+8 of each 16-lane row)
-  lrun = xsum16(lrun);
-  lrun = xsum32(lrun);
-  const float m_o = __shfl_xor(mrun, 8, 64), l_o = __shfl_xor(lrun, 8, 64);
-  const float mm = fmaxf(mrun, m_o);
+  // ---- reduce l and sum P' over the 4 lane groups, merge stream B into stream A (lanes n and n^8), undo the bias
+  float lsum = xsum32(xsum16(st.lrun)), ps = xsum32(xsum16(st.psum));
+  const float m2 = st.mrun == -INFINITY ? -INFINITY : st.mrun * c;  // exp2 domain
+  const float m_o = __shfl_xor(m2, 8, 64), l_o = __shfl_xor(lsum, 8, 64), ps_o = __shfl_xor(ps, 8, 64);
+  const float mm = fmaxf(m2, m_o);
   const float ms = mm == -INFINITY ? 0.f : mm;
-  const float w_s = __builtin_amdgcn_exp2f(mrun - ms), w_o = __builtin_amdgcn_exp2f(m_o - ms);
-  const float lm = lrun * w_s + l_o * w_o;
+  const float w_s = __builtin_amdgcn_exp2f(m2 - ms), w_o = __builtin_amdgcn_exp2f(m_o - ms);
+  const float lm = lsum * w_s + l_o * w_o;
+  const float pm = 128.0f * (ps * w_s + ps_o * w_o);
+  const float w_s24 = w_s * 16777216.0f, w_o24 = w_o * 16777216.0f;
   float o[16];  // head dims 16g .. 16g+15: O[t][i] is dim 16g + 4i + t
 #pragma unroll
   for (int t = 0; t < 4; t++)
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const float mine = O[t][i];
+      const float mine = st.O[t][i];
       const float oth = __shfl_xor(mine, 8, 64);
-      o[4 * i + t] = mine * w_s + oth * w_o;
+      o[4 * i + t] = (mine * w_s24 + oth * w_o24) - pm;
     }
+  float mfin = mm, lfin = lm;
+  if (WPR > 1) {  // merge the WPR waves of this item through LDS; its first wave writes the result
+    if (strm == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) *(float4*)&sh_o[wave][head][16 * g + 4 * i] = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+      if (g == 0) { sh_ml[wave][head][0] = mm; sh_ml[wave][head][1] = lm; }
+    }
+    __syncthreads();
+    if (wsub != 0 || !live) return;
+    if (strm == 0) {
+      float mw[WPR];
+      float mall = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < WPR; w++) { mw[w] = sh_ml[wave + w][head][0]; mall = fmaxf(mall, mw[w]); }
+      const float msf = mall == -INFINITY ? 0.f : mall;
+      lfin = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; i++) o[i] = 0.f;
+#pragma unroll
+      for (int w = 0; w < WPR; w++) {
+        const float ww = __builtin_amdgcn_exp2f(mw[w] - msf);
+        lfin += ww * sh_ml[wave + w][head][1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const float4 x = *(const float4*)&sh_o[wave + w][head][16 * g + 4 * i];
+          o[4 * i] += ww * x.x; o[4 * i + 1] += ww * x.y; o[4 * i + 2] += ww * x.z; o[4 * i + 3] += ww * x.w;
+        }
+      }
+      mfin = mall;
+    }
+  }
   if (strm == 0 && head < G) {
-    if (P.splits == 1) {
-      const float inv = lm > 0.f ? 1.0f / lm : 0.f;
+    if (rp.nsplit == 1) {
+      const float inv = lfin > 0.f ? 1.0f / lfin : 0.f;
       const int64_t off = (int64_t)b * P.sob + (int64_t)(h * G + head) * P.soh + 16 * g;
       if (ODT == UVMI_F32) {
         float* op = (float*)P.out + off;
@@ -321,8 +409,8 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
 #pragma unroll
       for (int i = 0; i < 4; i++) *(float4*)(op + 4 * i) = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
       if (g == 0) {
-        P.ws_m[r] = mm;
-        P.ws_l[r] = lm;
+        P.ws_m[r] = mfin;
+        P.ws_l[r] = lfin;
       }
     }
   }
@@ -353,8 +441,13 @@ __global__ __launch_bounds__(64) void attn_generic(AttnParams P) {
     qs[i] = elem<QDT>::ld(P.q, (int64_t)b * P.sqb + (int64_t)(h * G + gi) * P.sqh + d);
   }
   __syncthreads();
-  const Chunk c = split_range(P, b, sid);
-  const int lo_eff = max(c.lo, c.s0);
+  const RowPlan rp = plan_row(P, b);
+  if (sid >= rp.nsplit) return;
+  struct { int s0, s1; } c;
+  c.s0 = rp.a0 + sid * rp.chunk;
+  c.s1 = min(c.s0 + rp.chunk, rp.p + 1);
+  const int lo_eff = max(rp.lo, c.s0);
+  const bool direct = rp.nsplit == 1;
   constexpr int MAXG = 16, MAXD = 4;  // hd <= 256
   float mrun[MAXG], lrun[MAXG], acc[MAXG][MAXD];
 #pragma unroll
@@ -427,7 +520,7 @@ __global__ __launch_bounds__(64) void attn_generic(AttnParams P) {
       for (int dj = 0; dj < MAXD; dj++) {
         const int d = lane + 64 * dj;
         if (d < hd) {
-          if (P.splits == 1) {
+          if (direct) {
             const float v = lrun[gi] > 0.f ? acc[gi][dj] / lrun[gi] : 0.f;
             elem<ODT>::st(P.out, (int64_t)b * P.sob + (int64_t)(h * G + gi) * P.soh + d, v);
           } else {
@@ -435,7 +528,7 @@ __global__ __launch_bounds__(64) void attn_generic(AttnParams P) {
           }
         }
       }
-      if (P.splits > 1 && lane == 0) {
+      if (!direct && lane == 0) {
         P.ws_m[item * G + gi] = mrun[gi];
         P.ws_l[item * G + gi] = lrun[gi];
       }
@@ -444,38 +537,41 @@ __global__ __launch_bounds__(64) void attn_generic(AttnParams P) {
 }
 
 // ---------------------------------------------------------------------------------------------------- combine
-// One wave per (row, kv head, query head): out = sum_s w_s o_s / sum_s w_s l_s, w_s = 2^(m_s - max m); empty splits
-// (m = -inf) get weight 0 (decode_attn.py:96-115 of the reference).
+// One wave per (row, kv head), all G query heads: out = sum_s w_s o_s / sum_s w_s l_s, w_s = 2^(m_s - max m); empty
+// splits (m = -inf) get weight 0 (decode_attn.py:96-115 of the reference).  Rows that fit one chunk were written by
+// the attention kernel and are skipped.
 template <int ODT>
 __global__ __launch_bounds__(256) void attn_combine(AttnParams P) {
   const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (bk * G + gi)
-  if (r >= (int64_t)P.B * P.KH * P.G) return;
-  const int64_t bk = r / P.G;
-  const int gi = (int)(r % P.G);
+  const int64_t bk = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (bk >= (int64_t)P.B * P.KH) return;
   const int b = (int)(bk / P.KH), h = (int)(bk % P.KH);
-  float mx = -INFINITY;
-  for (int s = 0; s < P.splits; s++) mx = fmaxf(mx, P.ws_m[(bk * P.splits + s) * P.G + gi]);
-  const float ms = mx == -INFINITY ? 0.f : mx;
-  float den = 0.f;
-  float num[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < P.splits; s++) {
-    const int64_t pr = (bk * P.splits + s) * P.G + gi;
-    const float m = P.ws_m[pr];
-    if (m == -INFINITY) continue;
-    const float w = exp2f(m - ms);
-    den += w * P.ws_l[pr];
+  const RowPlan rp = plan_row(P, b);
+  if (rp.nsplit <= 1) return;
+  for (int gi = 0; gi < P.G; gi++) {
+    float mx = -INFINITY;
+    for (int s = 0; s < rp.nsplit; s++) mx = fmaxf(mx, P.ws_m[(bk * P.splits + s) * P.G + gi]);
+    const float ms = mx == -INFINITY ? 0.f : mx;
+    float den = 0.f;
+    float num[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < rp.nsplit; s++) {
+      const int64_t pr = (bk * P.splits + s) * P.G + gi;
+      const float m = P.ws_m[pr];
+      if (m == -INFINITY) continue;
+      const float w = exp2f(m - ms);
+      den += w * P.ws_l[pr];
+#pragma unroll
+      for (int dj = 0; dj < 4; dj++) {
+        const int d = lane + 64 * dj;
+        if (d < P.hd) num[dj] += w * P.ws_o[pr * P.hd + d];
+      }
+    }
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
 #pragma unroll
     for (int dj = 0; dj < 4; dj++) {
       const int d = lane + 64 * dj;
-      if (d < P.hd) num[dj] += w * P.ws_o[pr * P.hd + d];
+      if (d < P.hd) elem<ODT>::st(P.out, (int64_t)b * P.sob + (int64_t)(h * P.G + gi) * P.soh + d, num[dj] * inv);
     }
-  }
-  const float inv = den > 0.f ? 1.0f / den : 0.f;
-#pragma unroll
-  for (int dj = 0; dj < 4; dj++) {
-    const int d = lane + 64 * dj;
-    if (d < P.hd) elem<ODT>::st(P.out, (int64_t)b * P.sob + (int64_t)(h * P.G + gi) * P.soh + d, num[dj] * inv);
   }
 }
 
@@ -493,7 +589,7 @@ static int check_common(const uvmi_attn_args* a) {
   UVMI_REQUIRE(a->kv_dtype != UVMI_I8 || (a->k_scale && a->v_scale), UVMI_EINVAL, "uvmi_decode_attn: int8 cache needs k_scale and v_scale");
   UVMI_REQUIRE(a->idx_dtype == UVMI_I64 || a->idx_dtype == UVMI_I32, UVMI_EINVAL, "uvmi_decode_attn: pos/starts must be I32 or I64");
   UVMI_REQUIRE(a->num_splits >= 1 && a->num_splits <= 1024, UVMI_EINVAL, "uvmi_decode_attn: num_splits=%d out of range", a->num_splits);
-  UVMI_REQUIRE(a->window >= 0, UVMI_EINVAL, "uvmi_decode_attn: negative window");
+  UVMI_REQUIRE(a->window >= 0 && a->chunk_keys >= 0, UVMI_EINVAL, "uvmi_decode_attn: negative window or chunk_keys");
   UVMI_REQUIRE(a->hd <= 256 && a->H / a->KH <= 16, UVMI_EUNSUPPORTED, "uvmi_decode_attn: head_dim %d / group %d beyond 256 / 16", a->hd,
                a->H / a->KH);
   return UVMI_OK;
@@ -502,7 +598,9 @@ static int check_common(const uvmi_attn_args* a) {
 static bool mfma_ok(const uvmi_attn_args* a) {
   const int G = a->H / a->KH;
   if (a->hd != 64 || a->kv_dtype != UVMI_I8 || G > 8) return false;
-  if (a->ring && (a->S % 16 != 0)) return false;
+  if (!(a->scale > 0.f)) return false;  // the running maximum is tracked before the (positive) softmax scale
+  if (a->ring && (a->S % 32 != 0)) return false;
+  if (a->sks > (1 << 20) || a->svs > (1 << 20) || a->sks < 0 || a->svs < 0) return false;  // 32-bit tile offsets
   if (a->S % 4 != 0 || a->S < 4) return false;
   auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
   if (!al(a->q, 16) || a->sqb % 8 || a->sqh % 8) return false;
@@ -529,9 +627,11 @@ extern "C" int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus) {
   if (n_cus <= 0) n_cus = uvmi_device_cus();
   if (n_cus <= 0) n_cus = 256;
   if (n_bk < 1) n_bk = 1;
-  // 16 resident waves per CU hide HBM latency with one 4 KB super-tile in flight each; chunks stay >= 64 keys
-  const int64_t want = (16LL * n_cus + n_bk - 1) / n_bk;
-  int64_t cap = ctx / 64;
+  // One workgroup (4 waves streaming interleaved tiles) per (row, kv head, split).  A row is only cut when there are
+  // fewer rows than compute units, and never into chunks shorter than 256 keys: the combine pass costs more than the
+  // imbalance it removes once every CU has a workgroup.
+  const int64_t want = (n_cus + n_bk - 1) / n_bk;
+  int64_t cap = ctx / 256;
   if (cap < 1) cap = 1;
   int64_t s = want < cap ? want : cap;
   if (s > 64) s = 64;
@@ -557,6 +657,8 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   P.ssb = a->ssb; P.ssh = a->ssh; P.stb = a->stb; P.sth = a->sth; P.sob = a->sob; P.soh = a->soh;
   P.B = a->B; P.H = a->H; P.KH = a->KH; P.G = a->H / a->KH; P.S = a->S; P.hd = a->hd;
   P.window = a->window; P.ring = a->ring ? 1 : 0; P.splits = a->num_splits; P.idx64 = a->idx_dtype == UVMI_I64;
+  P.chunk_keys = a->chunk_keys > 0 ? ((a->chunk_keys + 31) & ~31) : 0;
+  P.gran = 32;
   P.n_items = (int64_t)a->B * a->KH * a->num_splits;
   P.scale_log2 = a->scale * LOG2E;
   P.ws_o = P.ws_m = P.ws_l = nullptr;
@@ -572,9 +674,21 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   }
   UVMI_REQUIRE(P.n_items < (1LL << 31), UVMI_EUNSUPPORTED, "uvmi_decode_attn: too many work items");
   if (mfma_ok(a)) {
-    const dim3 grid((unsigned)((P.n_items + 3) / 4)), blk(256);
-#define UVMI_L(QD, OD) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD>), grid, blk, 0, st, P)
-    const int od = a->num_splits > 1 ? UVMI_F32 : a->out_dtype;  // partials are fp32; ODT only matters for splits == 1
+    // waves per work item: long rows are streamed by all 4 waves of a workgroup, short ones by 2 or 1
+    const int ctx = a->window > 0 && a->window < a->S ? a->window : a->S;
+    int wpr = ctx >= 512 ? 4 : (ctx >= 128 ? 2 : 1);
+    if (const char* e = getenv("UVMI_ATTN_WPR")) { const int v = atoi(e); if (v == 1 || v == 2 || v == 4) wpr = v; }
+    P.gran = 32 * wpr;
+    if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
+    const int ipb = 4 / wpr;
+    const dim3 grid((unsigned)((P.n_items + ipb - 1) / ipb)), blk(256);
+#define UVMI_L(QD, OD)                                                                         \
+  do {                                                                                         \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 4>), grid, blk, 0, st, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2>), grid, blk, 0, st, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1>), grid, blk, 0, st, P);               \
+  } while (0)
+    const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
     if (a->q_dtype == UVMI_F16) {
       if (od == UVMI_F16) UVMI_L(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(UVMI_F16, UVMI_BF16); else UVMI_L(UVMI_F16, UVMI_F32);
     } else {
@@ -584,7 +698,7 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   } else {
     const dim3 grid((unsigned)P.n_items), blk(64);
     const size_t sh = ((size_t)P.G * a->hd + (size_t)P.G * 64) * 4;
-    const int od = a->num_splits > 1 ? UVMI_F32 : a->out_dtype;
+    const int od = a->out_dtype;
 #define UVMI_L(QD, KD, OD) hipLaunchKernelGGL((attn_generic<QD, KD, OD>), grid, blk, sh, st, P)
 #define UVMI_LO(QD, KD) do { if (od == UVMI_F16) UVMI_L(QD, KD, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(QD, KD, UVMI_BF16); else UVMI_L(QD, KD, UVMI_F32); } while (0)
 #define UVMI_LK(QD) do { if (a->kv_dtype == UVMI_I8) UVMI_LO(QD, UVMI_I8); else if (a->kv_dtype == UVMI_F16) UVMI_LO(QD, UVMI_F16); else UVMI_LO(QD, UVMI_BF16); } while (0)
@@ -595,7 +709,7 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   }
   UVMI_CHECK_LAUNCH("uvmi_decode_attn");
   if (a->num_splits > 1) {
-    const int64_t rows = (int64_t)a->B * a->H;
+    const int64_t rows = (int64_t)a->B * a->KH;
     const dim3 grid((unsigned)((rows + 3) / 4)), blk(256);
     if (a->out_dtype == UVMI_F16) hipLaunchKernelGGL((attn_combine<UVMI_F16>), grid, blk, 0, st, P);
     else if (a->out_dtype == UVMI_BF16) hipLaunchKernelGGL((attn_combine<UVMI_BF16>), grid, blk, 0, st, P);

@@ -13,9 +13,10 @@ from torch import Tensor
 from .. import _lib as L
 
 
-def default_splits(n_bk: int, ctx: int, device=None, min_chunk: int = 64, waves: int = 16) -> int:
-    """Splits per (row, kv head): enough wave64 work items for ~`waves` per compute unit, each chunk >= min_chunk keys
-    (reference: decode_attn.py:121-129, re-derived for 256 CUs)."""
+def default_splits(n_bk: int, ctx: int, device=None, min_chunk: int = 256, waves: int = 1) -> int:
+    """Splits per (row, kv head) (reference: decode_attn.py:121-129, re-derived for MI355X).  Each (row, kv head,
+    split) is one workgroup whose 4 waves stream interleaved key tiles, so a row is only cut when there are fewer rows
+    than `waves` workgroups per compute unit, and never into chunks shorter than min_chunk keys."""
     if device is not None:
         with torch.cuda.device(device):
             cus = L.lib().uvmi_device_cus()
@@ -36,7 +37,7 @@ def supported(q: Tensor, k_cache: Tensor) -> bool:
                 and q.dtype in (torch.float16, torch.bfloat16))
 
 
-def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out):
+def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0):
     B, H, hd = q.shape
     KH, S = k_cache.shape[1], k_cache.shape[2]
     int8 = k_cache.dtype == torch.int8
@@ -60,6 +61,7 @@ def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_sc
     a.out, a.out_dtype, a.sob, a.soh = out.data_ptr(), L.dtype_code(out.dtype), out.stride(0), out.stride(1)
     a.B, a.H, a.KH, a.S, a.hd = B, H, KH, S, hd
     a.scale, a.window, a.ring, a.num_splits = float(scale), int(window), int(bool(ring)), int(num_splits)
+    a.chunk_keys = int(chunk_keys)
     a.workspace, a.workspace_bytes = (ws.data_ptr() if ws is not None else None), ws_bytes
     L.check(L.lib().uvmi_decode_attn(C.byref(a), L.stream_ptr(q)), "uvmi_decode_attn")
     return out
@@ -68,13 +70,13 @@ def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_sc
 @torch.library.custom_op("uvmi::decode_attn", mutates_args=())
 def _decode_attn_op(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float,
                     window: int, ring: bool, k_scale: Tensor | None, v_scale: Tensor | None, num_splits: int,
-                    out_fp32: bool) -> Tensor:
+                    out_fp32: bool, chunk_keys: int) -> Tensor:
     out = torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
-    return _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out)
+    return _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys)
 
 
 @_decode_attn_op.register_fake
-def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out_fp32):
+def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out_fp32, chunk_keys):
     return torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
 
 
@@ -82,7 +84,7 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
                      window: int = 0, ring: bool | None = None, k_scale: Tensor | None = None,
                      v_scale: Tensor | None = None, ctx_hint: int | None = None, num_splits: int | None = None,
                      block_n: int | None = None, num_warps: int = 1, backend: str = "auto",
-                     out_fp32: bool = False) -> Tensor:
+                     out_fp32: bool = False, chunk_keys: int = 0) -> Tensor:
     """Single-query attention for every row of a static KV cache (reference: decode_attn.py:193-230).
 
     q        (B, H, hd) fp16 or bf16 (any (B, 1, H, hd) view is accepted); H = K * G, query head h*G+g uses kv head h.
@@ -95,6 +97,8 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
     block_n, num_warps, backend  accepted for signature compatibility; the HIP kernels choose their own tiling
              ("hip" / "auto" / "cuda" / "triton" all run the HIP path).
     out_fp32 return the fp32 result before rounding to q.dtype (for parity checks).
+    chunk_keys  0: every row is cut into num_splits equal chunks (the reference's rule); > 0: chunks of at least this
+             many keys and at most num_splits of them per row, so short rows take fewer work items.
     Returns (B, H, hd) in q.dtype.  Graph-capturable; registered as a torch custom op (opaque to torch.compile)."""
     if q.dim() == 4:
         q = q.reshape(q.size(0), q.size(-2), q.size(-1))
@@ -112,4 +116,4 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
     if pos.dtype != starts.dtype:
         starts = starts.to(pos.dtype)
     return _decode_attn_op(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window),
-                           bool(ring), k_scale, v_scale, int(num_splits), bool(out_fp32))
+                           bool(ring), k_scale, v_scale, int(num_splits), bool(out_fp32), int(chunk_keys))
