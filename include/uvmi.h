@@ -86,7 +86,7 @@ int uvmi_kv_append(const uvmi_kv_append_args* a, void* stream);
 typedef struct uvmi_attn_args {
   const void* q; int q_dtype;              /* (B, H, hd) F16 or BF16, inner stride 1 */
   int64_t sqb, sqh;
-  const void* k_cache; const void* v_cache; int kv_dtype; /* (B, KH, S, hd) I8, F16 or BF16, inner stride 1 */
+  const void* k_cache; const void* v_cache; int kv_dtype; /* (B, KH, S, hd) I8, F16, BF16 or F32, inner stride 1 */
   int64_t skb, skh, sks, svb, svh, svs;
   const void* k_scale; const void* v_scale; /* (B, KH, S) fp16 when kv_dtype == I8, else NULL */
   int64_t ssb, ssh, stb, sth;
@@ -138,6 +138,57 @@ typedef struct uvmi_sample_args {
 int uvmi_fused_sample(const uvmi_sample_args* a, void* stream);
 /* Host-side Philox4x32-10 (Random123) for tests and host tooling: out[4] = philox(ctr[4], key[2]). */
 void uvmi_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Fused per-token kernels of the UV-50M step (everything between the GEMMs).  dtype is the activation type
+ * (F16 / BF16 / F32); weightless RMSNorm uses eps = machine epsilon of that type, as F.rms_norm(eps=None) does in
+ * the reference (ultraviolet/model.py:190-191).
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* x = rmsnorm(table[tok]); n = rmsnorm(x).  Replaces rms_norm_(self.embed(idx)) and the first block's pre-norm
+ * (ultraviolet/kernels/fast_decode.py:286, 305).  x_out may be NULL. */
+int uvmi_embed_norm(const void* table, int dtype, int64_t vocab, const int64_t* tok, int64_t rows, int d,
+                    void* x_out, void* n_out, void* stream);
+
+/* h = a*x + b*y; n = rmsnorm(h).  Replaces the residual lambdas of Block.finish followed by the next pre-norm
+ * (ultraviolet/model.py:567-571; fast_decode.py:305, 332).  h_out may be NULL. */
+int uvmi_add_norm(const void* x, const void* y, int dtype, float a, float b, int64_t rows, int d, void* h_out,
+                  void* n_out, void* stream);
+
+/* Attention.qkv after the fused QKV GEMM (ultraviolet/model.py:310-319) plus the decode-time cache append
+ * (fast_decode.py:291-294, 315-317) for n token rows: value-embedding gate on v, QK-norm, partial RoPE
+ * (half-split pairing) at pos[r], q written in q_dtype for the attention kernel, k / v optionally written
+ * unquantized (prefill attention, XSA) and quantized into the int8 cache at row rows[r], slot pos[r] (or
+ * pos[r] % S when ring; on a ring only positions > last_pos[r] - S are written).  head_dim 64. */
+typedef struct uvmi_qkv_post_args {
+  const void* qkv; int dtype;          /* (n, (H + 2 KH) * hd): q heads, then k heads, then v heads */
+  const void* xn;                      /* (n, d) normed block input (value-embedding gate reads xn[:, :ve_ch]) */
+  const void* ve_table;                /* (vocab, KH * hd) value-embedding table, same dtype; NULL if !has_ve */
+  const float* ve_gate;                /* (KH, ve_ch) fp32 */
+  const int64_t* tok;                  /* (n,) token ids (value-embedding rows) */
+  const int64_t* pos;                  /* (n,) absolute position of each token */
+  const int64_t* rows;                 /* (n,) cache row of each token; NULL = identity */
+  const int64_t* last_pos;             /* (n,) last position of the token's prompt, or NULL (decode rows) */
+  const float* inv_freq;               /* (n_pairs,) RoPE frequencies, fp32 */
+  void* q_out; int q_dtype;            /* (n, H, hd) F16 or BF16 */
+  void* k_out; void* v_out;            /* (n, KH, hd) in dtype, or NULL */
+  int8_t* k_cache; int8_t* v_cache;    /* (B, KH, S, hd) or NULL (no append) */
+  uint16_t* k_scale; uint16_t* v_scale;
+  int64_t scb, sch, scs, ssb, ssh;     /* cache / scale strides */
+  int64_t n, vocab;
+  int H, KH, hd, d, ve_ch, n_pairs, S, ring, has_ve, rope;
+} uvmi_qkv_post_args;
+int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream);
+
+/* Attention.post before the output projection (ultraviolet/model.py:321-333): XSA z -= xsa[h] (z . v_hat) v_hat with
+ * the unquantized current v (fp32), then z *= 2 sigmoid(gate_w[h] . xn[:gate_ch]).  xsa = tanh(alpha) (H,) fp32 or NULL;
+ * gate_w (H, gate_ch) fp32 or NULL.  z (n, H, hd) in z_dtype (F16 / BF16); out (n, H * hd) in dtype. */
+int uvmi_attn_post(const void* z, int z_dtype, const void* v, const void* xn, int dtype, const float* gate_w,
+                   const float* xsa, float xsa_eps, int64_t n, int H, int KH, int hd, int d, int gate_ch, void* out,
+                   void* stream);
+
+/* SwiGLU after the fused gate/up GEMM (ultraviolet/model.py:388-391): out[r, j] = silu(gu[r, j]) * gu[r, f + j]. */
+int uvmi_swiglu(const void* gu, int dtype, int64_t rows, int f, void* out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -57,6 +57,18 @@ class SampleArgs(C.Structure):
                 ("cap_a", C.c_float), ("cap_b", C.c_float), ("cap_c", C.c_float), ("temperature", C.c_float)]
 
 
+class QkvPostArgs(C.Structure):
+    _fields_ = [("qkv", C.c_void_p), ("dtype", C.c_int), ("xn", C.c_void_p), ("ve_table", C.c_void_p),
+                ("ve_gate", C.c_void_p), ("tok", C.c_void_p), ("pos", C.c_void_p), ("rows", C.c_void_p),
+                ("last_pos", C.c_void_p), ("inv_freq", C.c_void_p), ("q_out", C.c_void_p), ("q_dtype", C.c_int),
+                ("k_out", C.c_void_p), ("v_out", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+                ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+                ("scb", C.c_int64), ("sch", C.c_int64), ("scs", C.c_int64), ("ssb", C.c_int64), ("ssh", C.c_int64),
+                ("n", C.c_int64), ("vocab", C.c_int64),
+                ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int), ("d", C.c_int), ("ve_ch", C.c_int),
+                ("n_pairs", C.c_int), ("S", C.c_int), ("ring", C.c_int), ("has_ve", C.c_int), ("rope", C.c_int)]
+
+
 _lib = None
 
 
@@ -83,6 +95,14 @@ def lib() -> C.CDLL:
         L.uvmi_fused_sample.argtypes = [C.POINTER(SampleArgs), C.c_void_p]
         L.uvmi_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
         L.uvmi_philox4x32_10.restype = None
+        L.uvmi_embed_norm.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
+                                      C.c_void_p]
+        L.uvmi_add_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int64, C.c_int, C.c_void_p,
+                                    C.c_void_p, C.c_void_p]
+        L.uvmi_qkv_post.argtypes = [C.POINTER(QkvPostArgs), C.c_void_p]
+        L.uvmi_attn_post.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_float,
+                                     C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        L.uvmi_swiglu.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 
@@ -106,4 +126,5 @@ def require_cuda(*ts: torch.Tensor) -> None:
 
 EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_rows", "uvmi_dequantize_rows",
            "uvmi_kv_write", "uvmi_kv_append", "uvmi_decode_attn", "uvmi_decode_attn_workspace_bytes",
-           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10"]
+           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
+           "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu"]

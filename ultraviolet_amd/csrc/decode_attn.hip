@@ -422,6 +422,7 @@ template <int KVDT>
 __device__ __forceinline__ float kv_ld(const void* p, int64_t i) {
   if (KVDT == UVMI_I8) return (float)((const int8_t*)p)[i];
   if (KVDT == UVMI_F16) return half_bits_to_float(((const uint16_t*)p)[i]);
+  if (KVDT == UVMI_F32) return ((const float*)p)[i];
   return bf16_to_float(((const uint16_t*)p)[i]);
 }
 
@@ -584,8 +585,8 @@ static int check_common(const uvmi_attn_args* a) {
   UVMI_REQUIRE(a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16, UVMI_EUNSUPPORTED, "uvmi_decode_attn: q must be F16 or BF16");
   UVMI_REQUIRE(a->out_dtype == UVMI_F16 || a->out_dtype == UVMI_BF16 || a->out_dtype == UVMI_F32, UVMI_EUNSUPPORTED,
                "uvmi_decode_attn: out must be F16, BF16 or F32");
-  UVMI_REQUIRE(a->kv_dtype == UVMI_I8 || a->kv_dtype == UVMI_F16 || a->kv_dtype == UVMI_BF16, UVMI_EUNSUPPORTED,
-               "uvmi_decode_attn: cache must be I8, F16 or BF16");
+  UVMI_REQUIRE(a->kv_dtype == UVMI_I8 || a->kv_dtype == UVMI_F16 || a->kv_dtype == UVMI_BF16 || a->kv_dtype == UVMI_F32, UVMI_EUNSUPPORTED,
+               "uvmi_decode_attn: cache must be I8, F16, BF16 or F32");
   UVMI_REQUIRE(a->kv_dtype != UVMI_I8 || (a->k_scale && a->v_scale), UVMI_EINVAL, "uvmi_decode_attn: int8 cache needs k_scale and v_scale");
   UVMI_REQUIRE(a->idx_dtype == UVMI_I64 || a->idx_dtype == UVMI_I32, UVMI_EINVAL, "uvmi_decode_attn: pos/starts must be I32 or I64");
   UVMI_REQUIRE(a->num_splits >= 1 && a->num_splits <= 1024, UVMI_EINVAL, "uvmi_decode_attn: num_splits=%d out of range", a->num_splits);
@@ -701,7 +702,7 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
     const int od = a->out_dtype;
 #define UVMI_L(QD, KD, OD) hipLaunchKernelGGL((attn_generic<QD, KD, OD>), grid, blk, sh, st, P)
 #define UVMI_LO(QD, KD) do { if (od == UVMI_F16) UVMI_L(QD, KD, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(QD, KD, UVMI_BF16); else UVMI_L(QD, KD, UVMI_F32); } while (0)
-#define UVMI_LK(QD) do { if (a->kv_dtype == UVMI_I8) UVMI_LO(QD, UVMI_I8); else if (a->kv_dtype == UVMI_F16) UVMI_LO(QD, UVMI_F16); else UVMI_LO(QD, UVMI_BF16); } while (0)
+#define UVMI_LK(QD) do { if (a->kv_dtype == UVMI_I8) UVMI_LO(QD, UVMI_I8); else if (a->kv_dtype == UVMI_F16) UVMI_LO(QD, UVMI_F16); else if (a->kv_dtype == UVMI_F32) UVMI_LO(QD, UVMI_F32); else UVMI_LO(QD, UVMI_BF16); } while (0)
     if (a->q_dtype == UVMI_F16) UVMI_LK(UVMI_F16); else UVMI_LK(UVMI_BF16);
 #undef UVMI_LK
 #undef UVMI_LO

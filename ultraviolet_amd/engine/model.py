@@ -1,0 +1,271 @@
+"""UV-50M forward for inference on the HIP kernels: int8 KV state, one decode step for a ragged batch, packed prefill.
+
+Mirrors ultraviolet/kernels/fast_decode.py of the reference (KernelDecodeState :21-57, decode_step_fast :272-334,
+_prefill_packed / prefill_packed_host :117-269) and the layer math of ultraviolet/model.py (Attention.qkv / post
+:302-335, Block.finish :567-571, MathLM.logits :824-827).  The GEMMs are torch (hipBLASLt) calls on preallocated
+buffers; everything between them is one fused HIP kernel per stage, and K/V go straight into the int8 cache.
+One decode step is a fixed launch sequence with no host synchronisation: it reads per-row positions on the device, so
+a single captured graph serves every context length (the reference needs one graph per 1024-token bucket,
+model.py:1099-1100)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from .. import _lib as L
+from ..kernels.decode_attn import decode_attention
+from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
+from .config import UVConfig
+from .weights import UVWeights
+
+
+class KVState:
+    """Slot-indexed int8 KV cache (reference: KernelDecodeState, fast_decode.py:21-57): per layer k, v (B, K, S, hd) int8
+    and k_scale, v_scale (B, K, S) fp16 with S = max_len on global layers and min(window, max_len) on local (ring)
+    layers; pos / starts (B,) int64 on the device.  pos is the next position to write."""
+
+    def __init__(self, cfg: UVConfig, B: int, max_len: int, device="cuda"):
+        self.cfg, self.B, self.max_len = cfg, B, max_len
+        self.local_len = min(cfg.window, max_len)
+        dev = torch.device(device)
+        self.k, self.v, self.k_scale, self.v_scale = [], [], [], []
+        for l in range(cfg.n_layers):
+            S = max_len if cfg.is_global(l) else self.local_len
+            shp = (B, cfg.n_kv_heads, S, cfg.head_dim)
+            self.k.append(torch.zeros(shp, dtype=torch.int8, device=dev))
+            self.v.append(torch.zeros(shp, dtype=torch.int8, device=dev))
+            self.k_scale.append(torch.zeros(shp[:3], dtype=torch.float16, device=dev))
+            self.v_scale.append(torch.zeros(shp[:3], dtype=torch.float16, device=dev))
+        self.pos = torch.zeros(B, dtype=torch.long, device=dev)
+        self.starts = torch.zeros(B, dtype=torch.long, device=dev)
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.k + self.v + self.k_scale + self.v_scale)
+
+
+def kv_bytes_per_seq(cfg: UVConfig, ctx: int) -> int:
+    """int8 cache bytes of one sequence at context ctx (reference: fast_decode.py:64-67)."""
+    per_pos = 2 * cfg.n_kv_heads * (cfg.head_dim + 2)
+    return sum(per_pos * (ctx if cfg.is_global(l) else min(ctx, cfg.window)) for l in range(cfg.n_layers))
+
+
+class UVEngine:
+    def __init__(self, weights: UVWeights, max_tokens: int):
+        """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens)."""
+        self.w, self.cfg = weights, weights.cfg
+        cfg, dt, dev = self.cfg, weights.dtype, weights.device
+        assert cfg.head_dim == 64, "the fused kernels are written for head_dim 64"
+        self.dtype, self.device, self.max_tokens = dt, dev, max_tokens
+        self.dt_code = L.dtype_code(dt)
+        self.q_dtype = torch.bfloat16 if dt == torch.bfloat16 else torch.float16
+        n, d, H, K, hd, f = max_tokens, cfg.d_model, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_ff
+        e = lambda *s, dtype=dt: torch.empty(*s, dtype=dtype, device=dev)
+        self.buf = dict(x=e(n, d), xn=e(n, d), h=e(n, d), qkv=e(n, (H + 2 * K) * hd), q=e(n, H, hd, dtype=self.q_dtype),
+                        k=e(n, K, hd), v=e(n, K, hd), zg=e(n, H * hd), a=e(n, d), gu=e(n, 2 * f), act=e(n, f), m=e(n, d))
+        L.lib()  # fail now if the library is missing
+
+    # ------------------------------------------------------------------------------------------------ kernels
+    def _embed_norm(self, tok: Tensor, n: int):
+        b = self.buf
+        rc = L.lib().uvmi_embed_norm(self.w.embed.data_ptr(), self.dt_code, self.cfg.vocab_size, tok.data_ptr(), n,
+                                     self.cfg.d_model, b["x"].data_ptr(), b["xn"].data_ptr(), L.stream_ptr(tok))
+        L.check(rc, "uvmi_embed_norm")
+
+    def _add_norm(self, x: Tensor, y: Tensor, a: float, bb: float, n: int, h_out: Tensor | None, n_out: Tensor):
+        rc = L.lib().uvmi_add_norm(x.data_ptr(), y.data_ptr(), self.dt_code, a, bb, n, self.cfg.d_model,
+                                   None if h_out is None else h_out.data_ptr(), n_out.data_ptr(), L.stream_ptr(x))
+        L.check(rc, "uvmi_add_norm")
+
+    def _qkv_post(self, l: int, tok: Tensor, pos: Tensor, rows: Tensor | None, last_pos: Tensor | None, st: KVState | None,
+                  n: int, write_cache: bool = True):
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        glob = cfg.is_global(l)
+        a = L.QkvPostArgs()
+        a.qkv, a.dtype, a.xn = b["qkv"].data_ptr(), self.dt_code, b["xn"].data_ptr()
+        has_ve = cfg.has_ve(l)
+        if has_ve:
+            a.ve_table, a.ve_gate, a.tok = self.w.value_embed.data_ptr(), W["ve_gate"].data_ptr(), tok.data_ptr()
+        a.pos = pos.data_ptr()
+        a.rows = None if rows is None else rows.data_ptr()
+        a.last_pos = None if last_pos is None else last_pos.data_ptr()
+        a.inv_freq = self.w.inv_freq.data_ptr()
+        a.q_out, a.q_dtype = b["q"].data_ptr(), L.dtype_code(self.q_dtype)
+        a.k_out, a.v_out = b["k"].data_ptr(), b["v"].data_ptr()
+        if st is not None and write_cache:
+            kc, ks = st.k[l], st.k_scale[l]
+            a.k_cache, a.v_cache, a.k_scale, a.v_scale = kc.data_ptr(), st.v[l].data_ptr(), ks.data_ptr(), st.v_scale[l].data_ptr()
+            a.scb, a.sch, a.scs, a.ssb, a.ssh = kc.stride(0), kc.stride(1), kc.stride(2), ks.stride(0), ks.stride(1)
+            a.S = kc.size(2)
+        a.n, a.vocab = n, cfg.vocab_size
+        a.H, a.KH, a.hd, a.d, a.ve_ch, a.n_pairs = cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_model, cfg.ve_gate_channels, cfg.n_pairs
+        a.ring, a.has_ve = int(not glob), int(has_ve)
+        a.rope = int(((not glob) or cfg.global_rope) and cfg.n_pairs > 0)
+        L.check(L.lib().uvmi_qkv_post(C.byref(a), L.stream_ptr(pos)), "uvmi_qkv_post")
+
+    def _attn_post(self, l: int, z: Tensor, n: int):
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        rc = L.lib().uvmi_attn_post(z.data_ptr(), L.dtype_code(z.dtype), b["v"].data_ptr(), b["xn"].data_ptr(), self.dt_code,
+                                    None if W["attn_gate"] is None else W["attn_gate"].data_ptr(),
+                                    None if W["xsa"] is None else W["xsa"].data_ptr(), float(cfg.xsa_eps), n, cfg.n_heads,
+                                    cfg.n_kv_heads, cfg.head_dim, cfg.d_model, cfg.gate_ch, b["zg"].data_ptr(), L.stream_ptr(z))
+        L.check(rc, "uvmi_attn_post")
+
+    def _swiglu(self, n: int):
+        b = self.buf
+        rc = L.lib().uvmi_swiglu(b["gu"].data_ptr(), self.dt_code, n, self.cfg.d_ff, b["act"].data_ptr(), L.stream_ptr(b["gu"]))
+        L.check(rc, "uvmi_swiglu")
+
+    # ------------------------------------------------------------------------------------------------ trunk
+    def _trunk(self, tok: Tensor, pos: Tensor, n: int, attn, rows=None, last_pos=None, st: KVState | None = None) -> Tensor:
+        """n token rows through all layers; attn(l, q (n, H, hd)) -> z (n, H, hd) runs after K/V of the layer have been
+        appended to the cache and written unquantized to buf k / v.  Returns the final normed hidden (n, d) (a buffer)."""
+        cfg, b = self.cfg, self.buf
+        assert n <= self.max_tokens
+        self._embed_norm(tok, n)
+        x, xn = b["x"][:n], b["xn"][:n]
+        for l, W in enumerate(self.w.layers):
+            torch.mm(xn, W["wqkv"].t(), out=b["qkv"][:n])
+            self._qkv_post(l, tok, pos, rows, last_pos, st, n)
+            z = attn(l, b["q"][:n])
+            self._attn_post(l, z, n)
+            torch.mm(b["zg"][:n], W["wo"].t(), out=b["a"][:n])
+            # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
+            self._add_norm(x, b["a"][:n], W["resid_attn"], W["post_attn"], n, b["h"], b["xn"])
+            torch.mm(xn, W["gu"].t(), out=b["gu"][:n])
+            self._swiglu(n)
+            torch.mm(b["act"][:n], W["down"].t(), out=b["m"][:n])
+            # x = resid_mlp * h + post_mlp * m ; xn = rmsnorm(x) (next block's pre-norm, or the final norm)
+            self._add_norm(b["h"][:n], b["m"][:n], W["resid_mlp"], W["post_mlp"], n, b["x"], b["xn"])
+        return xn
+
+    def head(self, hidden: Tensor) -> Tensor:
+        """Raw tied-head output (n, V) in the activation dtype: the GEMM MathLM.logits runs before .float() and the
+        softcap (model.py:824-827); the sampler applies the softcap."""
+        return torch.mm(hidden, self.w.embed.t())
+
+    def logits(self, hidden: Tensor) -> Tensor:
+        a, bb, c = self.cfg.softcap
+        return a * torch.sigmoid((self.head(hidden).float() + bb) / c)
+
+    # ------------------------------------------------------------------------------------------------ decode
+    @torch.no_grad()
+    def decode_step(self, tok: Tensor, st: KVState, num_splits: dict | None = None) -> Tensor:
+        """One token for all B rows at per-row st.pos (reference: decode_step_fast, fast_decode.py:272-334): append K/V
+        at pos first, attend lo..pos, then st.pos += 1.  Returns the final normed hidden (B, d)."""
+        cfg = self.cfg
+        B = tok.numel()
+        pos, starts = st.pos, st.starts
+        ns = num_splits or {}
+
+        def attn(l, q):
+            if cfg.is_global(l):
+                return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0, ring=False,
+                                        k_scale=st.k_scale[l], v_scale=st.v_scale[l], num_splits=ns.get("global"))
+            return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=cfg.window, ring=True,
+                                    k_scale=st.k_scale[l], v_scale=st.v_scale[l], num_splits=ns.get("local"))
+
+        h = self._trunk(tok, pos, B, attn, st=st)
+        st.pos.add_(1)
+        return h
+
+    # ------------------------------------------------------------------------------------------------ prefill
+    @torch.no_grad()
+    def prefill(self, prompts: list[list[int]], rows: list[int], st: KVState, left_pad: bool = True) -> Tensor:
+        """Packed prefill of whole prompts into cache rows `rows` (reference: prefill_packed_host, fast_decode.py:210-269):
+        the real tokens of all prompts run back to back through the trunk with causal (and, on local layers, windowed)
+        attention over their own unquantized K/V; only the cache write quantises.  left_pad keeps the reference's
+        positions (token j of a prompt of length n sits at T - n + j, T = longest prompt of the call) so the cache
+        layout equals the reference's; left_pad=False starts every prompt at position 0.  Sets st.pos / st.starts of the
+        rows and returns the final normed hidden of each prompt's last token (len(prompts), d)."""
+        cfg, dev = self.cfg, self.device
+        lens = np.fromiter((len(p) for p in prompts), dtype=np.int64, count=len(prompts))
+        assert lens.min() > 0
+        T = int(lens.max())
+        assert T <= st.max_len
+        starts = (T - lens) if left_pad else np.zeros_like(lens)
+        cu = np.zeros(len(prompts) + 1, dtype=np.int64)
+        cu[1:] = np.cumsum(lens)
+        N = int(cu[-1])
+        assert N <= self.max_tokens, f"{N} prefill tokens exceed the engine's max_tokens {self.max_tokens}"
+        x = np.fromiter((t for p in prompts for t in p), dtype=np.int64, count=N)
+        seg = np.repeat(np.arange(len(prompts), dtype=np.int64), lens)
+        idx = np.arange(N, dtype=np.int64)
+        pos = idx - cu[:-1][seg] + starts[seg]
+        rows_np = np.asarray(rows, dtype=np.int64)
+        tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+        tok_t, pos_t, row_t = tt(x), tt(pos), tt(rows_np[seg])
+        last_t = tt((starts + lens - 1)[seg])
+        pidx_t, pstart_t = tt(idx), tt(cu[:-1][seg])   # packed index of each token and of its segment's first token
+        K, hd, b = cfg.n_kv_heads, cfg.head_dim, self.buf
+
+        def attn(l, q):
+            # every packed token is a "row" whose cache is the packed unquantized K / V of this call (batch stride 0)
+            kp = b["k"][:N].transpose(0, 1).unsqueeze(0).expand(N, K, N, hd)
+            vp = b["v"][:N].transpose(0, 1).unsqueeze(0).expand(N, K, N, hd)
+            w = 0 if cfg.is_global(l) else cfg.window
+            return decode_attention(q, kp, vp, pidx_t, pstart_t, cfg.attn_scale, window=w, ring=False, num_splits=1)
+
+        h = self._trunk(tok_t, pos_t, N, attn, rows=row_t, last_pos=last_t, st=st)
+        rt = tt(rows_np)
+        st.starts[rt] = tt(starts)
+        st.pos[rt] = tt(starts + lens)
+        return h.index_select(0, tt(cu[1:] - 1))
+
+    # ------------------------------------------------------------------------------------------------ generation
+    @torch.no_grad()
+    def generate(self, prompts: list[list[int]], max_new: int, temperature: float = 0.0, seed: int = 0,
+                 max_len: int | None = None, use_graph: bool = False, return_logp: bool = False):
+        """Static-batch generation (reference: generate, model.py:1228-1263): packed prefill of all prompts, then
+        lockstep decode.  temperature <= 0: greedy.  Otherwise the fused sampler with Philox uniforms keyed by
+        (seed, request = prompt index, token index)."""
+        cfg, dev = self.cfg, self.device
+        B = len(prompts)
+        T = max(len(p) for p in prompts)
+        st = KVState(cfg, B, max_len or (T + max_new), dev)
+        req = torch.arange(B, dtype=torch.long, device=dev)
+        ti = torch.zeros(B, dtype=torch.long, device=dev)
+
+        def draw(hidden):
+            xh = self.head(hidden)
+            if temperature <= 0:
+                return greedy_sample(xh, cfg.softcap)
+            return fused_sample_seeded(xh, seed, req, ti, cfg.softcap, temperature)
+
+        tok, lp = draw(self.prefill(prompts, list(range(B)), st))
+        toks, lps = [tok.clone()], [lp.clone()]
+        cur = tok.clone()
+        graph = None
+
+        def step():
+            ti.add_(1)
+            t, l_ = draw(self.decode_step(cur, st))
+            cur.copy_(t)
+            lpbuf.copy_(l_)
+
+        lpbuf = torch.zeros(B, dtype=torch.float32, device=dev)
+        for i in range(max_new - 1):
+            if use_graph:
+                if graph is None:
+                    pos0, ti0, cur0 = st.pos.clone(), ti.clone(), cur.clone()
+                    s = torch.cuda.Stream()
+                    s.wait_stream(torch.cuda.current_stream())
+                    with torch.cuda.stream(s):
+                        step()
+                    torch.cuda.current_stream().wait_stream(s)
+                    st.pos.copy_(pos0); ti.copy_(ti0); cur.copy_(cur0)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        step()
+                    st.pos.copy_(pos0); ti.copy_(ti0); cur.copy_(cur0)
+                graph.replay()
+            else:
+                step()
+            toks.append(cur.clone())
+            lps.append(lpbuf.clone())
+        out = torch.stack(toks, 1).tolist()
+        if return_logp:
+            return out, torch.stack(lps, 1).cpu().numpy()
+        return out
