@@ -92,6 +92,9 @@ typedef struct uvmi_attn_args {
   int64_t ssb, ssh, stb, sth;
   const void* pos; const void* starts; int idx_dtype; /* (B,) I64 or I32: position of the current key (already
                                                          written) and first valid position of each row */
+  const void* rows;                        /* optional (B,) cache row of each query row (same idx_dtype): lets a compacted
+                                              batch of active slots address a larger cache; rows[b] < 0 marks a padding
+                                              row (no keys, zero output); NULL = identity */
   void* out; int out_dtype;                /* (B, H, hd) F16 / BF16 / F32, inner stride 1 */
   int64_t sob, soh;
   int B, H, KH, S, hd;
@@ -141,19 +144,20 @@ void uvmi_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t o
 
 /* ------------------------------------------------------------------------------------------------------------
  * Fused per-token kernels of the UV-50M step (everything between the GEMMs).  dtype is the activation type
- * (F16 / BF16 / F32); weightless RMSNorm uses eps = machine epsilon of that type, as F.rms_norm(eps=None) does in
- * the reference (ultraviolet/model.py:190-191).
+ * (F16 / BF16 / F32).  eps is the RMSNorm epsilon: the reference calls F.rms_norm(x, eps=None)
+ * (ultraviolet/model.py:190-191), whose default depends on the torch release (machine epsilon of the input dtype or of
+ * fp32), so the caller passes the value its torch uses.
  * ---------------------------------------------------------------------------------------------------------- */
 
 /* x = rmsnorm(table[tok]); n = rmsnorm(x).  Replaces rms_norm_(self.embed(idx)) and the first block's pre-norm
  * (ultraviolet/kernels/fast_decode.py:286, 305).  x_out may be NULL. */
-int uvmi_embed_norm(const void* table, int dtype, int64_t vocab, const int64_t* tok, int64_t rows, int d,
+int uvmi_embed_norm(const void* table, int dtype, int64_t vocab, const int64_t* tok, int64_t rows, int d, float eps,
                     void* x_out, void* n_out, void* stream);
 
 /* h = a*x + b*y; n = rmsnorm(h).  Replaces the residual lambdas of Block.finish followed by the next pre-norm
  * (ultraviolet/model.py:567-571; fast_decode.py:305, 332).  h_out may be NULL. */
-int uvmi_add_norm(const void* x, const void* y, int dtype, float a, float b, int64_t rows, int d, void* h_out,
-                  void* n_out, void* stream);
+int uvmi_add_norm(const void* x, const void* y, int dtype, float a, float b, int64_t rows, int d, float eps,
+                  void* h_out, void* n_out, void* stream);
 
 /* Attention.qkv after the fused QKV GEMM (ultraviolet/model.py:310-319) plus the decode-time cache append
  * (fast_decode.py:291-294, 315-317) for n token rows: value-embedding gate on v, QK-norm, partial RoPE
@@ -177,6 +181,7 @@ typedef struct uvmi_qkv_post_args {
   int64_t scb, sch, scs, ssb, ssh;     /* cache / scale strides */
   int64_t n, vocab;
   int H, KH, hd, d, ve_ch, n_pairs, S, ring, has_ve, rope;
+  float eps;                           /* QK-norm epsilon */
 } uvmi_qkv_post_args;
 int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream);
 
@@ -189,6 +194,41 @@ int uvmi_attn_post(const void* z, int z_dtype, const void* v, const void* xn, in
 
 /* SwiGLU after the fused gate/up GEMM (ultraviolet/model.py:388-391): out[r, j] = silu(gu[r, j]) * gu[r, f + j]. */
 int uvmi_swiglu(const void* gu, int dtype, int64_t rows, int f, void* out, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * On-device continuous batching: the slot table of generate_continuous (ultraviolet/model.py:1283-1350) and
+ * StreamGen (scripts/rl_stream.py:55-146) kept in device memory.  All arrays are caller-owned.
+ * ---------------------------------------------------------------------------------------------------------- */
+typedef struct uvmi_sched_state {
+  int64_t* slot_req;    /* (B,) request id bound to the slot, -1 = free */
+  int64_t* slot_cnt;    /* (B,) tokens generated so far (the token drawn from the prefill counts) */
+  int64_t* slot_limit;  /* (B,) length limit of the request */
+  int64_t* slot_tok;    /* (B,) last sampled token = input of the next step */
+  int64_t* pos;         /* (B,) next position to write (the KV state's pos) */
+  int64_t* starts;      /* (B,) first valid position (the KV state's starts) */
+  int32_t* out_tok;     /* (B, max_new) generated tokens per slot */
+  float* out_lp;        /* (B, max_new) behaviour log-probs, or NULL */
+  int64_t* done_req; int64_t* done_slot; int64_t* done_cnt; /* (done_cap,) completion records, appended in arrival order */
+  int32_t* counters;    /* [0] active slots at the last compact, [1] completion records written, [2] bucket overflow flag */
+  int64_t max_new; int64_t eos_id; /* eos_id < 0: none */
+  int B; int done_cap;
+} uvmi_sched_state;
+
+/* List the active slots (ascending) and gather their token, position, start, request id and token index into dense
+ * arrays of length n_bucket; rows past the active count get slot -1 and zeros.  Replaces the host loop over rows of
+ * rl_stream.py:105-124 and the device-built index tensors of fast_decode.py:126-134. */
+int uvmi_sched_compact(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c,
+                       int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, void* stream);
+/* Scatter sampled tokens / log-probs into the slots' output rows, advance count and position, retire rows on EOS,
+ * length limit or (retire_p > 0) a Philox Bernoulli draw keyed by (seed, request, token index), park retired rows at
+ * position 0 and append completion records.  Replaces buf.scatter_ / cnt.add_ and the harvest test of
+ * rl_stream.py:120-143, model.py:1321-1350. */
+int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const int64_t* act_slot, const int64_t* new_tok,
+                      const float* new_lp, float retire_p, uint64_t seed, void* stream);
+/* Bind n freshly prefilled requests to slots and record their first sampled token (model.py:1306-1313,
+ * rl_stream.py:86-92). */
+int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, const int64_t* req_ids,
+                     const int64_t* limits, const int64_t* first_tok, const float* first_lp, void* stream);
 
 #ifdef __cplusplus
 }

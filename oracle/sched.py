@@ -1,0 +1,71 @@
+"""Continuous-batching slot bookkeeping, pure-Python simulator (checker only; see oracle/__init__.py).
+
+Restates the slot logic of the reference's host loops (generate_continuous, ultraviolet/model.py:1283-1350; StreamGen,
+scripts/rl_stream.py:66-146) at per-step granularity, which is what the device-side table does: the token drawn from
+the prefill is token 0 of a request (model.py:1306-1313); a row finishes when its count reaches its limit or it emits
+EOS, inclusive (rl_stream.py:131-138); finished rows are parked at position 0 (model.py:1345-1350); the output column is
+clamped to the buffer width (rl_stream.py:122).  The reference tests a row only every check_every steps and discards
+what it decoded past the end; retiring at the exact step returns the same rows.
+
+Pinned by: the invariants of the reference's tests (every request returned once, rows EOS-terminated or exactly limit
+long: tests/test_rl_stream.py:82-94) and brute-force comparison with a straight-line per-request loop in
+tests/test_oracle_sched.py.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import philox
+
+
+class SlotTable:
+    def __init__(self, B: int, max_new: int, eos_id: int | None = None):
+        self.B, self.max_new, self.eos = B, max_new, -1 if eos_id is None else int(eos_id)
+        self.req = np.full(B, -1, np.int64)
+        self.cnt = np.zeros(B, np.int64)
+        self.limit = np.zeros(B, np.int64)
+        self.tok = np.zeros(B, np.int64)
+        self.pos = np.zeros(B, np.int64)
+        self.starts = np.zeros(B, np.int64)
+        self.out_tok = np.zeros((B, max_new), np.int32)
+        self.out_lp = np.zeros((B, max_new), np.float32)
+        self.done: list[tuple[int, int, int]] = []   # (request, slot, count)
+
+    def _finish(self, slot, req, cnt):
+        self.done.append((int(req), int(slot), int(cnt)))
+        self.req[slot] = -1
+        self.pos[slot] = 0
+        self.starts[slot] = 0
+
+    def admit(self, slots, req_ids, limits, first_tok, first_lp, pos, starts):
+        for i, s in enumerate(slots):
+            self.req[s], self.limit[s], self.tok[s], self.cnt[s] = req_ids[i], limits[i], first_tok[i], 1
+            self.pos[s], self.starts[s] = pos[i], starts[i]
+            self.out_tok[s, 0], self.out_lp[s, 0] = first_tok[i], first_lp[i]
+            if limits[i] <= 1 or (self.eos >= 0 and first_tok[i] == self.eos):
+                self._finish(s, req_ids[i], 1)
+
+    def compact(self, n_bucket: int):
+        act = np.nonzero(self.req >= 0)[0]
+        n = min(len(act), n_bucket)
+        out = {k: np.zeros(n_bucket, np.int64) for k in ("tok", "pos", "starts", "req", "cnt")}
+        slot = np.full(n_bucket, -1, np.int64)
+        slot[:n] = act[:n]
+        for k, src in (("tok", self.tok), ("pos", self.pos), ("starts", self.starts), ("req", self.req), ("cnt", self.cnt)):
+            out[k][:n] = src[act[:n]]
+        return slot, out, len(act)
+
+    def commit(self, act_slot, new_tok, new_lp, retire_p: float = 0.0, seed: int = 0):
+        for i, s in enumerate(act_slot):
+            if s < 0:
+                continue
+            c = int(self.cnt[s])
+            col = min(c, self.max_new - 1)
+            self.out_tok[s, col], self.out_lp[s, col] = new_tok[i], new_lp[i]
+            self.cnt[s], self.tok[s] = c + 1, new_tok[i]
+            self.pos[s] += 1
+            fin = c + 1 >= self.limit[s] or (self.eos >= 0 and new_tok[i] == self.eos)
+            if not fin and retire_p > 0:
+                fin = float(philox.request_uniform(seed, int(self.req[s]), c, philox.DOMAIN_RETIRE)) < np.float32(retire_p)
+            if fin:
+                self._finish(s, self.req[s], c + 1)

@@ -1,0 +1,159 @@
+"""GPU parity of the UV-50M engine (fused kernels + attention + sampler through the C ABI) against the torch-CPU oracle
+that is itself pinned by golden vectors from the reference.  Restates tests/test_math_kernels.py:152-189 and
+tests/test_math_model.py:303-323 of the reference."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _setup(name="uv-test", dtype=torch.float32, seed=0, perturb=0.06, **over):
+    from oracle.model import OracleModel
+    from ultraviolet_amd.engine import UVEngine, UVWeights, make_config, random_params
+    cfg = make_config(name, **over)
+    params = random_params(cfg, seed, perturb=perturb)
+    eng = UVEngine(UVWeights(cfg, params, dtype, DEV), max_tokens=2048)
+    return cfg, params, eng, OracleModel
+
+
+def _prompts(cfg, lens, seed=0):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(1, cfg.vocab_size, size=int(n)).tolist() for n in lens]
+
+
+def _teacher_forced(eng, prompts, cont, max_len):
+    from ultraviolet_amd.engine import KVState
+    B = len(prompts)
+    st = KVState(eng.cfg, B, max_len, DEV)
+    outs = [eng.logits(eng.prefill(prompts, list(range(B)), st)).cpu()]
+    for t in range(cont.shape[1]):
+        outs.append(eng.logits(eng.decode_step(torch.as_tensor(cont[:, t]).to(DEV), st)).cpu())
+    torch.cuda.synchronize()
+    return torch.stack(outs, 1).numpy(), st
+
+
+def _oracle_teacher_forced(m, prompts, cont, max_len):
+    from oracle.model import OracleState
+    B = len(prompts)
+    st = OracleState(m.cfg, B, max_len)
+    outs = [m.logits(m.prefill(prompts, list(range(B)), st)).numpy()]
+    for t in range(cont.shape[1]):
+        outs.append(m.logits(m.decode_step(cont[:, t], st)).numpy())
+    return np.stack(outs, 1), st
+
+
+def test_fp32_engine_matches_oracle_logits_and_cache():
+    """Through ring wrap (window 16) and left padding: logits close, int8 cache bytes and scales equal up to isolated
+    rounding ties, positions exact."""
+    cfg, params, eng, OracleModel = _setup(window=16)
+    prompts = _prompts(cfg, (5, 12, 9, 20, 1, 17))
+    cont = np.random.default_rng(1).integers(1, cfg.vocab_size, size=(6, 30))
+    lg, st = _teacher_forced(eng, prompts, cont, 64)
+    ref, ost = _oracle_teacher_forced(OracleModel(cfg, params, torch.float32), prompts, cont, 64)
+    assert np.isfinite(lg).all()
+    assert np.abs(lg - ref).max() < 2e-2                      # fp16 q in the attention kernel, fp16 P
+    assert (lg.argmax(-1) == ref.argmax(-1)).mean() > 0.98
+    assert np.array_equal(st.pos.cpu().numpy(), ost.pos) and np.array_equal(st.starts.cpu().numpy(), ost.starts)
+    nb = nd = 0
+    for l in range(cfg.n_layers):
+        for mine, o in ((st.k[l], ost.k[l]), (st.v[l], ost.v[l])):
+            # only slots a real token was written to are comparable (the oracle's padded prefill also writes pad slots)
+            d = np.abs(mine.cpu().numpy().astype(np.int32) - o.astype(np.int32))
+            valid = np.zeros(d.shape[:3], bool)
+            S = d.shape[2]
+            for b in range(d.shape[0]):
+                for t in range(int(ost.starts[b]), int(ost.pos[b])):
+                    if cfg.is_global(l) or t >= int(ost.pos[b]) - S:
+                        valid[b, :, t if cfg.is_global(l) else t % S] = True
+            nb += int(valid.sum()) * d.shape[3]
+            nd += int((d[valid] != 0).sum())
+            assert d[valid].max() <= 2
+    # deeper layers see activations that differ at the 1e-3 level (fp16 q and P in the attention kernel), which moves
+    # codes near a rounding boundary by one step; the quantizer itself is checked bit-exactly on identical inputs in
+    # test_gpu_kernels.py and on layer 0 below
+    assert nd < 0.15 * nb, (nd, nb)
+
+
+def test_first_layer_cache_is_bit_exact():
+    """Layer 0 sees only embedding -> norm -> QKV GEMM -> QK-norm / RoPE before the quantizer; with fp32 GEMMs its int8
+    bytes and fp16 scales must equal the oracle's almost everywhere (GEMM summation order can flip a tie)."""
+    cfg, params, eng, OracleModel = _setup(window=16)
+    prompts = _prompts(cfg, (16, 16, 16, 16), seed=3)
+    cont = np.random.default_rng(4).integers(1, cfg.vocab_size, size=(4, 8))
+    _, st = _teacher_forced(eng, prompts, cont, 32)
+    _, ost = _oracle_teacher_forced(OracleModel(cfg, params, torch.float32), prompts, cont, 32)
+    k = st.k[0].cpu().numpy()
+    assert (k != ost.k[0]).mean() < 2e-3
+    assert (st.k_scale[0].cpu().numpy().view(np.uint16) != ost.ks[0].view(np.uint16)).mean() < 2e-2
+
+
+@pytest.mark.parametrize("name,over", [("uv-test", dict(window=16)), ("uv-50m-alpha", dict())])
+def test_greedy_64_tokens_identical_fp32(name, over):
+    """BASELINE config 1 shape: 8 prompts, lengths U[32, 128], greedy 64 new tokens, int8 KV: identical token streams
+    (fp32 activations on the GPU vs the fp32 CPU oracle)."""
+    cfg, params, eng, OracleModel = _setup(name, perturb=0.06, **over)
+    rng = np.random.default_rng(0)
+    lens = rng.integers(32, 129, size=8)
+    prompts = [rng.integers(1, cfg.vocab_size, size=int(n)).tolist() for n in lens]
+    out = np.array(eng.generate(prompts, 64, temperature=0.0))
+    ref, lgs, _ = OracleModel(cfg, params, torch.float32).generate_greedy(prompts, 64, return_logits=True)
+    assert len(np.unique(ref)) > 8                                  # the stream is not one repeated token
+    # A stream may only leave the oracle's at a step where the oracle's own top-2 logits are closer than the numeric
+    # noise of the GPU path (fp16 q and P in the attention kernel, a different GEMM summation order): ~2e-3.
+    identical = 0
+    for b in range(len(prompts)):
+        d = np.nonzero(out[b] != ref[b])[0]
+        if len(d) == 0:
+            identical += 1
+            continue
+        t = int(d[0])
+        top2 = np.sort(lgs[b, t])[-2:]
+        assert top2[1] - top2[0] < 2e-3, f"row {b} diverges at step {t} with top-2 logit gap {top2[1] - top2[0]:.2e}"
+    assert identical >= len(prompts) - 2, identical
+
+
+def test_bf16_engine_close_to_oracle():
+    """reference bar for the int8 kernel path vs its SDPA path: max |logit diff| < 0.25, argmax agreement > 0.9
+    (tests/test_math_kernels.py:170-172)."""
+    cfg, params, eng, OracleModel = _setup(dtype=torch.bfloat16, window=16)
+    prompts = _prompts(cfg, (5, 12, 9, 20, 3, 17))
+    cont = np.random.default_rng(1).integers(1, cfg.vocab_size, size=(6, 30))
+    lg, _ = _teacher_forced(eng, prompts, cont, 64)
+    ref, _ = _oracle_teacher_forced(OracleModel(cfg, params, torch.bfloat16), prompts, cont, 64)
+    assert np.isfinite(lg).all()
+    assert np.abs(lg - ref).max() < 0.25
+    assert (lg.argmax(-1) == ref.argmax(-1)).mean() > 0.9
+
+
+def test_graph_replay_matches_eager_and_seeded_sampling_is_reproducible():
+    """One captured graph serves every step (positions are read on the device); replays equal eager
+    (reference: tests/test_math_kernels.py:176-189).  Seeded sampling does not depend on graph vs eager."""
+    cfg, params, eng, _ = _setup(dtype=torch.bfloat16, window=16)
+    prompts = _prompts(cfg, (6, 3, 4, 9), seed=5)
+    a = eng.generate(prompts, 40, temperature=0.0, use_graph=False)
+    b = eng.generate(prompts, 40, temperature=0.0, use_graph=True)
+    assert a == b
+    s1, lp1 = eng.generate(prompts, 40, temperature=1.0, seed=11, use_graph=False, return_logp=True)
+    s2, lp2 = eng.generate(prompts, 40, temperature=1.0, seed=11, use_graph=True, return_logp=True)
+    s3 = eng.generate(prompts, 40, temperature=1.0, seed=12)
+    assert s1 == s2 and np.array_equal(lp1, lp2) and s1 != s3
+    assert np.isfinite(lp1).all() and (lp1 <= 1e-6).all()
+
+
+def test_prefill_left_pad_vs_zero_start_positions():
+    """Starting every prompt at position 0 instead of left-padding changes cache slots but not the logits
+    (RoPE is relative, global layers have no positions)."""
+    from ultraviolet_amd.engine import KVState
+    cfg, params, eng, _ = _setup(window=16)
+    prompts = _prompts(cfg, (7, 19, 2), seed=6)
+    st1, st2 = KVState(cfg, 3, 64, DEV), KVState(cfg, 3, 64, DEV)
+    l1 = eng.logits(eng.prefill(prompts, [0, 1, 2], st1, left_pad=True))
+    l2 = eng.logits(eng.prefill(prompts, [2, 0, 1], st2, left_pad=False))
+    assert (l1 - l2).abs().max() < 2e-3
+    assert st2.starts.tolist() == [0, 0, 0] and sorted(st2.pos.tolist()) == [2, 7, 19]
+    tok = torch.tensor([5, 6, 7], device=DEV)
+    d1 = eng.logits(eng.decode_step(tok, st1))
+    d2 = eng.logits(eng.decode_step(tok[[1, 2, 0]], st2))
+    assert (d1 - d2[[2, 0, 1]]).abs().max() < 5e-2   # keys are rotated, hence quantized, at different absolute positions

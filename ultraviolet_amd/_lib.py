@@ -33,7 +33,7 @@ class AttnArgs(C.Structure):
                 ("svb", C.c_int64), ("svh", C.c_int64), ("svs", C.c_int64),
                 ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
                 ("ssb", C.c_int64), ("ssh", C.c_int64), ("stb", C.c_int64), ("sth", C.c_int64),
-                ("pos", C.c_void_p), ("starts", C.c_void_p), ("idx_dtype", C.c_int),
+                ("pos", C.c_void_p), ("starts", C.c_void_p), ("idx_dtype", C.c_int), ("rows", C.c_void_p),
                 ("out", C.c_void_p), ("out_dtype", C.c_int), ("sob", C.c_int64), ("soh", C.c_int64),
                 ("B", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("S", C.c_int), ("hd", C.c_int),
                 ("scale", C.c_float), ("window", C.c_int), ("ring", C.c_int), ("num_splits", C.c_int),
@@ -66,7 +66,15 @@ class QkvPostArgs(C.Structure):
                 ("scb", C.c_int64), ("sch", C.c_int64), ("scs", C.c_int64), ("ssb", C.c_int64), ("ssh", C.c_int64),
                 ("n", C.c_int64), ("vocab", C.c_int64),
                 ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int), ("d", C.c_int), ("ve_ch", C.c_int),
-                ("n_pairs", C.c_int), ("S", C.c_int), ("ring", C.c_int), ("has_ve", C.c_int), ("rope", C.c_int)]
+                ("n_pairs", C.c_int), ("S", C.c_int), ("ring", C.c_int), ("has_ve", C.c_int), ("rope", C.c_int),
+                ("eps", C.c_float)]
+
+
+class SchedState(C.Structure):
+    _fields_ = [("slot_req", C.c_void_p), ("slot_cnt", C.c_void_p), ("slot_limit", C.c_void_p), ("slot_tok", C.c_void_p),
+                ("pos", C.c_void_p), ("starts", C.c_void_p), ("out_tok", C.c_void_p), ("out_lp", C.c_void_p),
+                ("done_req", C.c_void_p), ("done_slot", C.c_void_p), ("done_cnt", C.c_void_p), ("counters", C.c_void_p),
+                ("max_new", C.c_int64), ("eos_id", C.c_int64), ("B", C.c_int), ("done_cap", C.c_int)]
 
 
 _lib = None
@@ -95,14 +103,19 @@ def lib() -> C.CDLL:
         L.uvmi_fused_sample.argtypes = [C.POINTER(SampleArgs), C.c_void_p]
         L.uvmi_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
         L.uvmi_philox4x32_10.restype = None
-        L.uvmi_embed_norm.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
-                                      C.c_void_p]
-        L.uvmi_add_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int64, C.c_int, C.c_void_p,
-                                    C.c_void_p, C.c_void_p]
+        L.uvmi_embed_norm.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_void_p,
+                                      C.c_void_p, C.c_void_p]
+        L.uvmi_add_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_int64, C.c_int, C.c_float,
+                                    C.c_void_p, C.c_void_p, C.c_void_p]
         L.uvmi_qkv_post.argtypes = [C.POINTER(QkvPostArgs), C.c_void_p]
         L.uvmi_attn_post.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_float,
                                      C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         L.uvmi_swiglu.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
+        L.uvmi_sched_compact.argtypes = [C.POINTER(SchedState), C.c_int] + [C.c_void_p] * 7
+        L.uvmi_sched_commit.argtypes = [C.POINTER(SchedState), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_uint64,
+                                        C.c_void_p]
+        L.uvmi_sched_admit.argtypes = [C.POINTER(SchedState), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_void_p]
         _lib = L
     return _lib
 
@@ -127,4 +140,5 @@ def require_cuda(*ts: torch.Tensor) -> None:
 EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_rows", "uvmi_dequantize_rows",
            "uvmi_kv_write", "uvmi_kv_append", "uvmi_decode_attn", "uvmi_decode_attn_workspace_bytes",
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
-           "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu"]
+           "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu",
+           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit"]

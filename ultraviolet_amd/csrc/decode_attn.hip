@@ -43,7 +43,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 struct AttnParams {
   const void* q; const void* kc; const void* vc; const void* ks; const void* vs;
-  const void* pos; const void* starts;
+  const void* pos; const void* starts; const void* rows;
   void* out; float* ws_o; float* ws_m; float* ws_l;
   int64_t sqb, sqh, skb, skh, sks, svb, svh, svs, ssb, ssh, stb, sth, sob, soh;
   int B, H, KH, G, S, hd, window, ring, splits, idx64, chunk_keys, gran;  // gran: chunk granularity (keys)
@@ -57,8 +57,9 @@ struct AttnParams {
 struct RowPlan { int lo, p, a0, chunk, nsplit; };
 __device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b) {
   RowPlan r;
-  const int p = (int)load_index(P.pos, P.idx64, b);
+  int p = (int)load_index(P.pos, P.idx64, b);
   const int st = (int)load_index(P.starts, P.idx64, b);
+  if (P.rows && load_index(P.rows, P.idx64, b) < 0) p = -1;  // padding row of a compacted batch: no keys, output zeros
   int lo = st > 0 ? st : 0;
   if (P.window > 0 && p - P.window + 1 > lo) lo = p - P.window + 1;
   r.lo = lo;
@@ -178,10 +179,12 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   st.psum = 0.f;
 
   // ---- addressing: wave-uniform row base + wave-uniform tile offset (scalar) + lane-invariant 32-bit offsets
-  const int8_t* kbase = (const int8_t*)P.kc + (int64_t)b * P.skb + (int64_t)h * P.skh;
-  const int8_t* vbase = (const int8_t*)P.vc + (int64_t)b * P.svb + (int64_t)h * P.svh;
-  const uint16_t* ksb = (const uint16_t*)P.ks + (int64_t)b * P.ssb + (int64_t)h * P.ssh;
-  const uint16_t* vsb = (const uint16_t*)P.vs + (int64_t)b * P.stb + (int64_t)h * P.sth;
+  int64_t cb = P.rows ? load_index(P.rows, P.idx64, b) : (int64_t)b;  // cache row of this query row
+  if (cb < 0) cb = 0;                                                 // (dead rows have no keys; keep addresses valid)
+  const int8_t* kbase = (const int8_t*)P.kc + cb * P.skb + (int64_t)h * P.skh;
+  const int8_t* vbase = (const int8_t*)P.vc + cb * P.svb + (int64_t)h * P.svh;
+  const uint16_t* ksb = (const uint16_t*)P.ks + cb * P.ssb + (int64_t)h * P.ssh;
+  const uint16_t* vsb = (const uint16_t*)P.vs + cb * P.stb + (int64_t)h * P.sth;
   const int S = P.S;
   const uint32_t sks = (uint32_t)P.sks, svs = (uint32_t)P.svs;
   const uint32_t usks = __builtin_amdgcn_readfirstlane(sks), usvs = __builtin_amdgcn_readfirstlane(svs);
@@ -458,8 +461,10 @@ __global__ __launch_bounds__(64) void attn_generic(AttnParams P) {
 #pragma unroll
     for (int j = 0; j < MAXD; j++) acc[gi][j] = 0.f;
   }
-  const int64_t kb0 = (int64_t)b * P.skb + (int64_t)h * P.skh, vb0 = (int64_t)b * P.svb + (int64_t)h * P.svh;
-  const int64_t ks0 = (int64_t)b * P.ssb + (int64_t)h * P.ssh, vs0 = (int64_t)b * P.stb + (int64_t)h * P.sth;
+  int64_t cb = P.rows ? load_index(P.rows, P.idx64, b) : (int64_t)b;
+  if (cb < 0) cb = 0;
+  const int64_t kb0 = cb * P.skb + (int64_t)h * P.skh, vb0 = cb * P.svb + (int64_t)h * P.svh;
+  const int64_t ks0 = cb * P.ssb + (int64_t)h * P.ssh, vs0 = cb * P.stb + (int64_t)h * P.sth;
   for (int tb = lo_eff; tb < c.s1; tb += 64) {
     const int t = tb + lane;
     const bool valid = t < c.s1;
@@ -653,7 +658,7 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   AttnParams P;
   P.q = a->q; P.kc = a->k_cache; P.vc = a->v_cache; P.ks = a->k_scale; P.vs = a->v_scale;
-  P.pos = a->pos; P.starts = a->starts; P.out = a->out;
+  P.pos = a->pos; P.starts = a->starts; P.rows = a->rows; P.out = a->out;
   P.sqb = a->sqb; P.sqh = a->sqh; P.skb = a->skb; P.skh = a->skh; P.sks = a->sks; P.svb = a->svb; P.svh = a->svh; P.svs = a->svs;
   P.ssb = a->ssb; P.ssh = a->ssh; P.stb = a->stb; P.sth = a->sth; P.sob = a->sob; P.soh = a->soh;
   P.B = a->B; P.H = a->H; P.KH = a->KH; P.G = a->H / a->KH; P.S = a->S; P.hd = a->hd;

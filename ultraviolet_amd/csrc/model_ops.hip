@@ -1,8 +1,9 @@
 // Fused per-token kernels of the UV-50M decode / prefill step: everything between the GEMMs.
 //
 // One wave64 per token row.  All arithmetic is fp32; values are rounded to the activation type T (fp16 / bf16 / fp32)
-// where the next GEMM reads them.  Weightless RMSNorm uses eps = machine epsilon of T, which is what
-// torch.nn.functional.rms_norm(x, eps=None) does in the reference (ultraviolet/model.py:190-191).
+// where the next GEMM reads them.  Weightless RMSNorm takes its eps from the caller: the reference calls
+// torch.nn.functional.rms_norm(x, eps=None) (ultraviolet/model.py:190-191), whose default has been the machine epsilon
+// of the input dtype in some torch releases and of fp32 in others, so the host passes what its torch does.
 //
 //   embed_norm   x = rmsnorm(E[tok]); n = rmsnorm(x)                                    (fast_decode.py:286, 305)
 //   add_norm     h = a*x + b*y; n = rmsnorm(h)          residual lambdas + pre-norm     (model.py:567-571)
@@ -24,17 +25,13 @@ template <> __device__ __forceinline__ float round_t<UVMI_F32>(float v) { return
 template <> __device__ __forceinline__ float round_t<UVMI_F16>(float v) { return (float)(half_t)v; }
 template <> __device__ __forceinline__ float round_t<UVMI_BF16>(float v) { return bf16_to_float(float_to_bf16(v)); }
 
-template <int DT> __host__ __device__ constexpr float eps_t() {
-  return DT == UVMI_F32 ? 1.1920928955078125e-07f : (DT == UVMI_F16 ? 9.765625e-04f : 7.8125e-03f);
-}
-
 // ------------------------------------------------------------------------------------------------ embed / residual
 // MODE 0: src = E[tok[r]] ; x = rmsnorm(src)        MODE 1: x = a*xin + b*yin
 // then n = rmsnorm(x) (of the rounded x).  d <= 64 * 2 * NP.
 template <int DT, int MODE>
 __global__ __launch_bounds__(256) void norm_kernel(const void* __restrict__ xin, const void* __restrict__ yin,
                                                    const int64_t* __restrict__ tok, int64_t vocab, float a, float b,
-                                                   void* __restrict__ xout, void* __restrict__ nout, int64_t rows, int d) {
+                                                   void* __restrict__ xout, void* __restrict__ nout, int64_t rows, int d, float eps) {
   constexpr int NP = 16;  // pairs per lane: d <= 2048
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -63,7 +60,7 @@ __global__ __launch_bounds__(256) void norm_kernel(const void* __restrict__ xin,
     }
   }
   if (MODE == 0) {
-    const float rs = rsqrtf(wave_sum(ss) / (float)d + eps_t<DT>());
+    const float rs = rsqrtf(wave_sum(ss) / (float)d + eps);
     ss = 0.f;
 #pragma unroll
     for (int i = 0; i < NP; i++) {
@@ -71,7 +68,7 @@ __global__ __launch_bounds__(256) void norm_kernel(const void* __restrict__ xin,
       ss += v0[i] * v0[i] + v1[i] * v1[i];
     }
   }
-  const float rn = rsqrtf(wave_sum(ss) / (float)d + eps_t<DT>());
+  const float rn = rsqrtf(wave_sum(ss) / (float)d + eps);
 #pragma unroll
   for (int i = 0; i < NP; i++) {
     const int pidx = lane + 64 * i;
@@ -92,6 +89,7 @@ struct QkvArgs {
   int64_t scb, sch, scs, ssb, ssh;
   int64_t n, vocab;
   int H, KH, d, ve_ch, n_pairs, S, ring, has_ve, rope, q_dt;
+  float eps;
 };
 
 __device__ __forceinline__ void store_q(void* p, int dt, int64_t i, float v) {
@@ -115,7 +113,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
     sn = round_t<DT>(sinf(th));
   }
   auto norm_rope = [&](float x) -> float {  // QK-norm over the 64 lanes, then partial RoPE (half-split pairing)
-    const float rs = rsqrtf(wave_sum(x * x) * (1.0f / 64.0f) + eps_t<DT>());
+    const float rs = rsqrtf(wave_sum(x * x) * (1.0f / 64.0f) + A.eps);
     const float xn = round_t<DT>(x * rs);
     if (!A.rope) return xn;
     const float other = __shfl_xor(xn, A.n_pairs, 64);  // lane d <-> d + n_pairs (n_pairs is a power of two)
@@ -223,24 +221,24 @@ static void dispatch_dt(int dt, F&& f) {
   else f(std::integral_constant<int, UVMI_F32>{});
 }
 
-extern "C" int uvmi_embed_norm(const void* table, int dtype, int64_t vocab, const int64_t* tok, int64_t rows, int d, void* x_out,
-                               void* n_out, void* stream) {
+extern "C" int uvmi_embed_norm(const void* table, int dtype, int64_t vocab, const int64_t* tok, int64_t rows, int d, float eps,
+                               void* x_out, void* n_out, void* stream) {
   UVMI_REQUIRE(table && tok && n_out, UVMI_EINVAL, "uvmi_embed_norm: null pointer");
   UVMI_REQUIRE(is_float_dtype(dtype) && rows >= 0 && d > 0 && d % 2 == 0 && d <= 2048 && vocab > 0, UVMI_EINVAL, "uvmi_embed_norm: bad arguments");
   if (rows == 0) return UVMI_OK;
   const dim3 grid((unsigned)((rows + 3) / 4)), blk(256);
-  dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((norm_kernel<decltype(DT)::value, 0>), grid, blk, 0, (hipStream_t)stream, table, nullptr, tok, vocab, 0.f, 0.f, x_out, n_out, rows, d); });
+  dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((norm_kernel<decltype(DT)::value, 0>), grid, blk, 0, (hipStream_t)stream, table, nullptr, tok, vocab, 0.f, 0.f, x_out, n_out, rows, d, eps); });
   UVMI_CHECK_LAUNCH("uvmi_embed_norm");
   return UVMI_OK;
 }
 
-extern "C" int uvmi_add_norm(const void* x, const void* y, int dtype, float a, float b, int64_t rows, int d, void* h_out, void* n_out,
-                             void* stream) {
+extern "C" int uvmi_add_norm(const void* x, const void* y, int dtype, float a, float b, int64_t rows, int d, float eps, void* h_out,
+                             void* n_out, void* stream) {
   UVMI_REQUIRE(x && y && n_out, UVMI_EINVAL, "uvmi_add_norm: null pointer");
   UVMI_REQUIRE(is_float_dtype(dtype) && rows >= 0 && d > 0 && d % 2 == 0 && d <= 2048, UVMI_EINVAL, "uvmi_add_norm: bad arguments");
   if (rows == 0) return UVMI_OK;
   const dim3 grid((unsigned)((rows + 3) / 4)), blk(256);
-  dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((norm_kernel<decltype(DT)::value, 1>), grid, blk, 0, (hipStream_t)stream, x, y, nullptr, 0, a, b, h_out, n_out, rows, d); });
+  dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((norm_kernel<decltype(DT)::value, 1>), grid, blk, 0, (hipStream_t)stream, x, y, nullptr, 0, a, b, h_out, n_out, rows, d, eps); });
   UVMI_CHECK_LAUNCH("uvmi_add_norm");
   return UVMI_OK;
 }
@@ -263,7 +261,7 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   A.k_cache = a->k_cache; A.v_cache = a->v_cache; A.k_scale = a->k_scale; A.v_scale = a->v_scale;
   A.scb = a->scb; A.sch = a->sch; A.scs = a->scs; A.ssb = a->ssb; A.ssh = a->ssh; A.n = a->n; A.vocab = a->vocab;
   A.H = a->H; A.KH = a->KH; A.d = a->d; A.ve_ch = a->ve_ch; A.n_pairs = a->n_pairs; A.S = a->S; A.ring = a->ring; A.has_ve = a->has_ve;
-  A.rope = a->rope; A.q_dt = a->q_dtype;
+  A.rope = a->rope; A.q_dt = a->q_dtype; A.eps = a->eps;
   const dim3 grid((unsigned)((a->n + 3) / 4)), blk(256);
   dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
   UVMI_CHECK_LAUNCH("uvmi_qkv_post");

@@ -1,0 +1,174 @@
+// On-device continuous-batching bookkeeping: the slot table of the reference's host loop
+// (generate_continuous, ultraviolet/model.py:1283-1350; StreamGen, scripts/rl_stream.py:55-146) kept in HBM and
+// advanced by two tiny kernels per decode step, so a step needs no host synchronisation:
+//
+//   sched_compact  scan the slot table, list the active slots first (ascending), gather their token / position /
+//                  request id / token index into dense arrays of a fixed bucket length (padding rows get slot -1);
+//   sched_commit   scatter the sampled token and its log-prob into the slot's output row, advance count and position,
+//                  retire on EOS / length limit / seeded Bernoulli(p), park retired rows at position 0 and append a
+//                  completion record for the host to harvest asynchronously.
+//
+// Both are integer bookkeeping on <= a few thousand slots: latency-bound, one workgroup / one thread per row.
+#include "common.h"
+
+namespace uvmi {
+
+constexpr uint32_t DOMAIN_RETIRE = 0x52455452u;
+
+__device__ inline void philox_round10(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c[0], p1 = (uint64_t)0xCD9E8D57u * c[2];
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0, n1 = (uint32_t)p1, n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1, n3 = (uint32_t)p0;
+    c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+}
+
+// One workgroup of 1024 threads; slots are handled in tiles of 1024 with a running base (ordered compaction).
+__global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, int64_t* tok_c,
+                                                             int64_t* pos_c, int64_t* starts_c, int64_t* req_c, int64_t* cnt_c) {
+  __shared__ int wsum[16];
+  __shared__ int base_sh;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) base_sh = 0;
+  __syncthreads();
+  for (int t0 = 0; t0 < S.B; t0 += 1024) {
+    const int slot = t0 + tid;
+    const bool act = slot < S.B && S.slot_req[slot] >= 0;
+    const unsigned long long bal = __ballot(act);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wsum[wave] = __popcll(bal);
+    __syncthreads();
+    int woff = 0;
+    for (int w = 0; w < wave; w++) woff += wsum[w];
+    const int base = base_sh;
+    if (act) {
+      const int i = base + woff + before;
+      if (i < n_bucket) {
+        act_slot[i] = slot;
+        tok_c[i] = S.slot_tok[slot];
+        pos_c[i] = S.pos[slot];
+        starts_c[i] = S.starts[slot];
+        req_c[i] = S.slot_req[slot];
+        cnt_c[i] = S.slot_cnt[slot];
+      }
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int tot = 0;
+      for (int w = 0; w < 16; w++) tot += wsum[w];
+      base_sh = base + tot;
+    }
+    __syncthreads();
+  }
+  const int n_act = base_sh;
+  for (int i = n_act + tid; i < n_bucket; i += 1024) {
+    act_slot[i] = -1; tok_c[i] = 0; pos_c[i] = 0; starts_c[i] = 0; req_c[i] = 0; cnt_c[i] = 0;
+  }
+  if (tid == 0) {
+    S.counters[0] = n_act;                              // active slots seen by this step
+    if (n_act > n_bucket) S.counters[2] = 1;            // bucket too small: the overflow slots idle this step
+  }
+}
+
+__global__ __launch_bounds__(256) void sched_commit_kernel(uvmi_sched_state S, int n_bucket, const int64_t* act_slot,
+                                                           const int64_t* new_tok, const float* new_lp, float retire_p, uint64_t seed) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_bucket) return;
+  const int64_t slot = act_slot[i];
+  if (slot < 0) return;
+  const int64_t tok = new_tok[i];
+  const int64_t c = S.slot_cnt[slot];
+  const int64_t col = c < S.max_new ? c : S.max_new - 1;   // clamp like the reference's buffers (rl_stream.py:122)
+  S.out_tok[slot * S.max_new + col] = (int32_t)tok;
+  if (S.out_lp) S.out_lp[slot * S.max_new + col] = new_lp ? new_lp[i] : 0.f;
+  S.slot_cnt[slot] = c + 1;
+  S.slot_tok[slot] = tok;
+  S.pos[slot] += 1;
+  bool fin = (c + 1 >= S.slot_limit[slot]) || (S.eos_id >= 0 && tok == S.eos_id);
+  const int64_t req = S.slot_req[slot];
+  if (!fin && retire_p > 0.f) {
+    uint32_t ctr[4] = {(uint32_t)c, (uint32_t)req, (uint32_t)((uint64_t)req >> 32), DOMAIN_RETIRE};
+    philox_round10(ctr, (uint32_t)seed, (uint32_t)(seed >> 32));
+    fin = (float)(ctr[0] >> 8) * 5.9604644775390625e-08f < retire_p;
+  }
+  if (fin) {
+    const int k = atomicAdd(&S.counters[1], 1) % S.done_cap;  // ring: the host must poll before done_cap more rows finish
+    S.done_req[k] = req;
+    S.done_slot[k] = slot;
+    S.done_cnt[k] = c + 1;
+    S.slot_req[slot] = -1;
+    S.pos[slot] = 0;      // parked: never overruns the cache (model.py:1345-1350)
+    S.starts[slot] = 0;
+  }
+}
+
+// Admission after a prefill: bind request ids to slots and record the first sampled token (it counts as token 0 of
+// the request: model.py:1306-1313, rl_stream.py:86-92).  pos / starts were set by the prefill.
+__global__ __launch_bounds__(256) void sched_admit_kernel(uvmi_sched_state S, int n, const int64_t* slots, const int64_t* req_ids,
+                                                          const int64_t* limits, const int64_t* first_tok, const float* first_lp) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int64_t slot = slots[i];
+  if (slot < 0 || slot >= S.B) return;
+  S.slot_req[slot] = req_ids[i];
+  S.slot_limit[slot] = limits[i];
+  S.slot_tok[slot] = first_tok[i];
+  S.slot_cnt[slot] = 1;
+  S.out_tok[slot * S.max_new] = (int32_t)first_tok[i];
+  if (S.out_lp) S.out_lp[slot * S.max_new] = first_lp ? first_lp[i] : 0.f;
+  const bool fin = limits[i] <= 1 || (S.eos_id >= 0 && first_tok[i] == S.eos_id);
+  if (fin) {
+    const int k = atomicAdd(&S.counters[1], 1) % S.done_cap;
+    S.done_req[k] = req_ids[i]; S.done_slot[k] = slot; S.done_cnt[k] = 1;
+    S.slot_req[slot] = -1;
+    S.pos[slot] = 0;
+    S.starts[slot] = 0;
+  }
+}
+
+static int check_state(const uvmi_sched_state* s, const char* who) {
+  UVMI_REQUIRE(s, UVMI_EINVAL, "%s: null state", who);
+  UVMI_REQUIRE(s->slot_req && s->slot_cnt && s->slot_limit && s->slot_tok && s->pos && s->starts && s->out_tok && s->counters &&
+                   s->done_req && s->done_slot && s->done_cnt, UVMI_EINVAL, "%s: null pointer in state", who);
+  UVMI_REQUIRE(s->B > 0 && s->B <= (1 << 20) && s->max_new > 0 && s->done_cap > 0, UVMI_EINVAL, "%s: bad sizes", who);
+  return UVMI_OK;
+}
+
+}  // namespace uvmi
+
+using namespace uvmi;
+
+extern "C" int uvmi_sched_compact(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c,
+                                  int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, void* stream) {
+  int rc = check_state(s, "uvmi_sched_compact");
+  if (rc) return rc;
+  UVMI_REQUIRE(n_bucket > 0 && act_slot && tok_c && pos_c && starts_c && req_c && cnt_c, UVMI_EINVAL, "uvmi_sched_compact: bad arguments");
+  hipLaunchKernelGGL(sched_compact_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, *s, n_bucket, act_slot, tok_c, pos_c, starts_c, req_c, cnt_c);
+  UVMI_CHECK_LAUNCH("uvmi_sched_compact");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const int64_t* act_slot, const int64_t* new_tok,
+                                 const float* new_lp, float retire_p, uint64_t seed, void* stream) {
+  int rc = check_state(s, "uvmi_sched_commit");
+  if (rc) return rc;
+  UVMI_REQUIRE(n_bucket > 0 && act_slot && new_tok, UVMI_EINVAL, "uvmi_sched_commit: bad arguments");
+  hipLaunchKernelGGL(sched_commit_kernel, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket, act_slot, new_tok,
+                     new_lp, retire_p, seed);
+  UVMI_CHECK_LAUNCH("uvmi_sched_commit");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, const int64_t* req_ids, const int64_t* limits,
+                                const int64_t* first_tok, const float* first_lp, void* stream) {
+  int rc = check_state(s, "uvmi_sched_admit");
+  if (rc) return rc;
+  UVMI_REQUIRE(n >= 0 && (n == 0 || (slots && req_ids && limits && first_tok)), UVMI_EINVAL, "uvmi_sched_admit: bad arguments");
+  if (n == 0) return UVMI_OK;
+  hipLaunchKernelGGL(sched_admit_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n, slots, req_ids, limits, first_tok, first_lp);
+  UVMI_CHECK_LAUNCH("uvmi_sched_admit");
+  return UVMI_OK;
+}

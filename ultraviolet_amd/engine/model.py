@@ -52,6 +52,17 @@ def kv_bytes_per_seq(cfg: UVConfig, ctx: int) -> int:
     return sum(per_pos * (ctx if cfg.is_global(l) else min(ctx, cfg.window)) for l in range(cfg.n_layers))
 
 
+def rms_norm_eps(dtype: torch.dtype) -> float:
+    """eps that torch.nn.functional.rms_norm(x, eps=None) uses for this dtype in the installed torch (the reference relies
+    on that default, model.py:190-191): machine epsilon of the dtype in some releases, of fp32 in others.  Probed once on
+    the CPU with a vector small enough that the two candidates give clearly different results."""
+    x = torch.full((8,), 2.0 ** -6, dtype=dtype)
+    y = float(torch.nn.functional.rms_norm(x, (8,)).float()[0])
+    cands = [float(torch.finfo(dtype).eps), float(torch.finfo(torch.float32).eps)]
+    refs = [2.0 ** -6 / (2.0 ** -12 + e) ** 0.5 for e in cands]
+    return cands[int(np.argmin([abs(y - r) for r in refs]))]
+
+
 class UVEngine:
     def __init__(self, weights: UVWeights, max_tokens: int):
         """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens)."""
@@ -60,6 +71,7 @@ class UVEngine:
         assert cfg.head_dim == 64, "the fused kernels are written for head_dim 64"
         self.dtype, self.device, self.max_tokens = dt, dev, max_tokens
         self.dt_code = L.dtype_code(dt)
+        self.eps = rms_norm_eps(dt)
         self.q_dtype = torch.bfloat16 if dt == torch.bfloat16 else torch.float16
         n, d, H, K, hd, f = max_tokens, cfg.d_model, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_ff
         e = lambda *s, dtype=dt: torch.empty(*s, dtype=dtype, device=dev)
@@ -71,11 +83,11 @@ class UVEngine:
     def _embed_norm(self, tok: Tensor, n: int):
         b = self.buf
         rc = L.lib().uvmi_embed_norm(self.w.embed.data_ptr(), self.dt_code, self.cfg.vocab_size, tok.data_ptr(), n,
-                                     self.cfg.d_model, b["x"].data_ptr(), b["xn"].data_ptr(), L.stream_ptr(tok))
+                                     self.cfg.d_model, self.eps, b["x"].data_ptr(), b["xn"].data_ptr(), L.stream_ptr(tok))
         L.check(rc, "uvmi_embed_norm")
 
     def _add_norm(self, x: Tensor, y: Tensor, a: float, bb: float, n: int, h_out: Tensor | None, n_out: Tensor):
-        rc = L.lib().uvmi_add_norm(x.data_ptr(), y.data_ptr(), self.dt_code, a, bb, n, self.cfg.d_model,
+        rc = L.lib().uvmi_add_norm(x.data_ptr(), y.data_ptr(), self.dt_code, a, bb, n, self.cfg.d_model, self.eps,
                                    None if h_out is None else h_out.data_ptr(), n_out.data_ptr(), L.stream_ptr(x))
         L.check(rc, "uvmi_add_norm")
 
@@ -103,6 +115,7 @@ class UVEngine:
         a.H, a.KH, a.hd, a.d, a.ve_ch, a.n_pairs = cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_model, cfg.ve_gate_channels, cfg.n_pairs
         a.ring, a.has_ve = int(not glob), int(has_ve)
         a.rope = int(((not glob) or cfg.global_rope) and cfg.n_pairs > 0)
+        a.eps = self.eps
         L.check(L.lib().uvmi_qkv_post(C.byref(a), L.stream_ptr(pos)), "uvmi_qkv_post")
 
     def _attn_post(self, l: int, z: Tensor, n: int):

@@ -1,0 +1,227 @@
+"""Continuous-batching rollout driver on the device-side slot table.
+
+Mirrors the reference's StreamGen (scripts/rl_stream.py:39-154: add / chunk / n_active / n_outstanding / drop_queued,
+results as (meta, tokens, behaviour log-probs, start_version)) and generate_continuous (ultraviolet/model.py:1266-1354),
+with the per-step bookkeeping moved to the GPU:
+
+  * the slot table (request id, count, limit, current token, position, output rows) lives in HBM (csrc/sched.hip);
+  * each decode step is compact -> trunk over the active rows only -> head GEMM -> fused sampler -> commit, captured
+    once per bucket of active-row counts and replayed; no step reads anything back to the host;
+  * the host only polls a completion ring every `check_every` steps (one small copy), harvests finished rows and
+    prefills queued requests into the freed slots.
+
+Sampling is keyed by (seed, request id, token index), so a request's tokens do not depend on the slot it lands in or on
+when it is admitted; the reference's torch.rand stream (perf.py:595) has no such property."""
+from __future__ import annotations
+
+import collections
+import ctypes as C
+
+import numpy as np
+import torch
+
+from .. import _lib as L
+from ..kernels.decode_attn import decode_attention
+from ..kernels.fused_sample import fused_sample_seeded, greedy_sample
+from .model import KVState, UVEngine
+
+
+class Rollout:
+    def __init__(self, engine: UVEngine, slots: int, max_prompt: int, max_new: int, temperature: float = 1.0,
+                 seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
+                 use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False):
+        self.e, self.cfg = engine, engine.cfg
+        self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
+        self.T, self.seed, self.eos = float(temperature), int(seed), eos_id
+        self.ce, self.bucket, self.use_graph = check_every, bucket, use_graph
+        self.retire_p, self.left_pad = float(retire_p), left_pad
+        dev = engine.device
+        self.dev = dev
+        assert slots <= engine.max_tokens
+        self.st = KVState(self.cfg, slots, max_prompt + max_new + 1, dev)
+        z = lambda *s, dt=torch.long: torch.zeros(*s, dtype=dt, device=dev)
+        self.slot_req = torch.full((slots,), -1, dtype=torch.long, device=dev)
+        self.slot_cnt, self.slot_limit, self.slot_tok = z(slots), z(slots), z(slots)
+        self.out_tok = z(slots, max_new, dt=torch.int32)
+        self.out_lp = z(slots, max_new, dt=torch.float32)
+        self.done_cap = 2 * slots
+        self.done_req, self.done_slot, self.done_cnt = z(self.done_cap), z(self.done_cap), z(self.done_cap)
+        self.counters = z(4, dt=torch.int32)
+        s = L.SchedState()
+        s.slot_req, s.slot_cnt, s.slot_limit, s.slot_tok = (t.data_ptr() for t in (self.slot_req, self.slot_cnt, self.slot_limit, self.slot_tok))
+        s.pos, s.starts = self.st.pos.data_ptr(), self.st.starts.data_ptr()
+        s.out_tok, s.out_lp = self.out_tok.data_ptr(), self.out_lp.data_ptr()
+        s.done_req, s.done_slot, s.done_cnt, s.counters = (t.data_ptr() for t in (self.done_req, self.done_slot, self.done_cnt, self.counters))
+        s.max_new, s.eos_id, s.B, s.done_cap = max_new, -1 if eos_id is None else int(eos_id), slots, self.done_cap
+        self.sched = s
+        # dense per-step arrays (bucket length <= slots)
+        self.act, self.tok_c, self.pos_c, self.starts_c, self.req_c, self.cnt_c = (z(slots) for _ in range(6))
+        self.new_tok, self.new_lp = z(slots), z(slots, dt=torch.float32)
+        self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        self.queue = collections.deque()
+        self.meta: dict[int, tuple] = {}          # request id -> (meta, start_version)
+        self.free = list(range(slots))[::-1]
+        self.next_req = 0
+        self.n_active_host = 0                    # upper bound on active slots (exact after each poll / admit)
+        self.done_seen = 0
+        self.version = 0
+        self.n_decode_steps = 0
+        self.n_tokens = 0
+
+    # ------------------------------------------------------------------------------------------------ requests
+    def add(self, prompt_ids, meta, limit: int | None = None):
+        assert 0 < len(prompt_ids) <= self.max_prompt, "prompt longer than max_prompt"
+        self.queue.append((list(prompt_ids), meta, self.max_new if limit is None else min(int(limit), self.max_new)))
+
+    def n_active(self) -> int:
+        return self.B - len(self.free)
+
+    def n_outstanding(self) -> int:
+        return len(self.queue) + self.n_active()
+
+    def drop_queued(self, pred) -> int:
+        keep = [x for x in self.queue if not pred(x[1])]
+        n = len(self.queue) - len(keep)
+        self.queue = collections.deque(keep)
+        return n
+
+    # ------------------------------------------------------------------------------------------------ admission
+    @torch.no_grad()
+    def _admit(self):
+        """Prefill queued requests into free slots (FIFO), in calls of at most engine.max_tokens packed tokens."""
+        e = self.e
+        while self.queue and self.free:
+            batch, ntok = [], 0
+            while self.queue and len(batch) < len(self.free) and ntok + len(self.queue[0][0]) <= e.max_tokens:
+                it = self.queue.popleft()
+                batch.append(it)
+                ntok += len(it[0])
+            if not batch:
+                raise RuntimeError("a queued prompt exceeds the engine's max_tokens")
+            slots = [self.free.pop() for _ in batch]
+            reqs = list(range(self.next_req, self.next_req + len(batch)))
+            self.next_req += len(batch)
+            h = e.prefill([b[0] for b in batch], slots, self.st, left_pad=self.left_pad)
+            x = e.head(h)
+            tt = lambda a: torch.as_tensor(a, dtype=torch.long, device=self.dev)
+            req_t = tt(reqs)
+            if self.T > 0:
+                tok, lp = fused_sample_seeded(x, self.seed, req_t, torch.zeros_like(req_t), self.cfg.softcap, self.T)
+            else:
+                tok, lp = greedy_sample(x, self.cfg.softcap)
+            slot_t, lim_t = tt(slots), tt([b[2] for b in batch])   # named: they must outlive the launch call
+            rc = L.lib().uvmi_sched_admit(C.byref(self.sched), len(batch), slot_t.data_ptr(), req_t.data_ptr(), lim_t.data_ptr(),
+                                          tok.data_ptr(), lp.data_ptr(), L.stream_ptr(tok))
+            L.check(rc, "uvmi_sched_admit")
+            for r, b in zip(reqs, batch):
+                self.meta[r] = (b[1], self.version)
+            self.n_active_host += len(batch)
+
+    # ------------------------------------------------------------------------------------------------ decode
+    def _step_body(self, n: int):
+        e, cfg, st = self.e, self.cfg, self.st
+        lib = L.lib()
+        sp = L.stream_ptr(self.act)
+        L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                       self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
+        act, pos, starts = self.act[:n], self.pos_c[:n], self.starts_c[:n]
+
+        def attn(l, q):
+            if cfg.is_global(l):
+                return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0, ring=False,
+                                        k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=act, num_splits=1)
+            return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=cfg.window, ring=True,
+                                    k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=act, num_splits=1)
+
+        h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st)
+        x = e.head(h)
+        if self.T > 0:
+            tok, lp = fused_sample_seeded(x, self.seed, self.req_c[:n], self.cnt_c[:n], cfg.softcap, self.T)
+        else:
+            tok, lp = greedy_sample(x, cfg.softcap)
+        self.new_tok[:n].copy_(tok)
+        self.new_lp[:n].copy_(lp)
+        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
+                                      self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
+
+    def bucket_for(self, n_active: int) -> int:
+        return min(self.B, max(self.bucket, -(-n_active // self.bucket) * self.bucket))
+
+    @torch.no_grad()
+    def step(self):
+        """One decode step for every active slot (graph replay of the bucket that covers the active count)."""
+        n = self.bucket_for(self.n_active_host)
+        if not self.use_graph:
+            self._step_body(n)
+        else:
+            g = self.graphs.get(n)
+            if g is None:
+                # Capture without running: a captured step mutates the slot table, so nothing is executed until replay.
+                # The kernels and GEMM shapes for this bucket are warmed up on a scratch copy of the mutable state.
+                keep = [t.clone() for t in self._mutable()]
+                s = torch.cuda.Stream()
+                s.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(s):
+                    self._step_body(n)
+                torch.cuda.current_stream().wait_stream(s)
+                torch.cuda.synchronize()
+                for t, k in zip(self._mutable(), keep):
+                    t.copy_(k)
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    self._step_body(n)
+                self.graphs[n] = g
+            g.replay()
+        self.n_decode_steps += 1
+
+    def _mutable(self):
+        """State a decode step writes.  The KV cache is left out on purpose: the warm-up step writes K/V at the current
+        positions, and the real replay rewrites exactly those slots with identical inputs (as in model.py:1126-1127)."""
+        return [self.slot_req, self.slot_cnt, self.slot_limit, self.slot_tok, self.st.pos, self.st.starts, self.out_tok, self.out_lp,
+                self.done_req, self.done_slot, self.done_cnt, self.counters]
+
+    # ------------------------------------------------------------------------------------------------ harvest
+    @torch.no_grad()
+    def poll(self):
+        """Read the completion ring (one small device->host copy), return finished requests as
+        (meta, tokens, logp float32 array, start_version) and free their slots."""
+        cnt = self.counters.cpu().numpy()
+        n_done = int(cnt[1])
+        if cnt[2]:
+            raise RuntimeError("active slots exceeded the captured bucket (host bound on active slots was wrong)")
+        out = []
+        if n_done > self.done_seen:
+            assert n_done - self.done_seen <= self.done_cap, "completion ring overflow: poll more often"
+            ix = torch.arange(self.done_seen, n_done, device=self.dev) % self.done_cap
+            reqs, slots, cnts = (t.index_select(0, ix).cpu().numpy() for t in (self.done_req, self.done_slot, self.done_cnt))
+            order = np.argsort(reqs, kind="stable")   # arrival order inside one step is not deterministic: sort by request
+            reqs, slots, cnts = reqs[order], slots[order], cnts[order]
+            st = torch.as_tensor(slots, device=self.dev)
+            toks, lps = self.out_tok.index_select(0, st).cpu().numpy(), self.out_lp.index_select(0, st).cpu().numpy()
+            for j, (r, s_, c) in enumerate(zip(reqs, slots, cnts)):
+                c = min(int(c), self.max_new)
+                meta, v0 = self.meta.pop(int(r))
+                out.append((meta, toks[j, :c].tolist(), lps[j, :c].copy(), v0))
+                self.n_tokens += c
+                self.free.append(int(s_))
+            self.done_seen = n_done
+        self.n_active_host = self.n_active()
+        return out
+
+    def chunk(self):
+        """Fill idle slots from the queue, decode check_every steps, harvest (reference: StreamGen.chunk)."""
+        if self.queue and self.free:
+            self._admit()
+        if self.n_active() == 0:
+            return []
+        for _ in range(self.ce):
+            self.step()
+        return self.poll()
+
+    def run(self, max_chunks: int = 1 << 30):
+        res = []
+        for _ in range(max_chunks):
+            if self.n_outstanding() == 0:
+                break
+            res += self.chunk()
+        return res

@@ -37,7 +37,7 @@ def supported(q: Tensor, k_cache: Tensor) -> bool:
                 and q.dtype in (torch.float16, torch.bfloat16))
 
 
-def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0):
+def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0, rows=None):
     B, H, hd = q.shape
     KH, S = k_cache.shape[1], k_cache.shape[2]
     int8 = k_cache.dtype == torch.int8
@@ -58,6 +58,9 @@ def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_sc
         a.k_scale, a.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
         a.ssb, a.ssh, a.stb, a.sth = k_scale.stride(0), k_scale.stride(1), v_scale.stride(0), v_scale.stride(1)
     a.pos, a.starts, a.idx_dtype = pos.data_ptr(), starts.data_ptr(), L.dtype_code(pos.dtype)
+    if rows is not None:
+        assert rows.dtype == pos.dtype and rows.is_contiguous() and rows.numel() == B
+        a.rows = rows.data_ptr()
     a.out, a.out_dtype, a.sob, a.soh = out.data_ptr(), L.dtype_code(out.dtype), out.stride(0), out.stride(1)
     a.B, a.H, a.KH, a.S, a.hd = B, H, KH, S, hd
     a.scale, a.window, a.ring, a.num_splits = float(scale), int(window), int(bool(ring)), int(num_splits)
@@ -70,13 +73,13 @@ def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_sc
 @torch.library.custom_op("uvmi::decode_attn", mutates_args=())
 def _decode_attn_op(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float,
                     window: int, ring: bool, k_scale: Tensor | None, v_scale: Tensor | None, num_splits: int,
-                    out_fp32: bool, chunk_keys: int) -> Tensor:
+                    out_fp32: bool, chunk_keys: int, rows: Tensor | None) -> Tensor:
     out = torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
-    return _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys)
+    return _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys, rows)
 
 
 @_decode_attn_op.register_fake
-def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out_fp32, chunk_keys):
+def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out_fp32, chunk_keys, rows):
     return torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
 
 
@@ -84,7 +87,7 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
                      window: int = 0, ring: bool | None = None, k_scale: Tensor | None = None,
                      v_scale: Tensor | None = None, ctx_hint: int | None = None, num_splits: int | None = None,
                      block_n: int | None = None, num_warps: int = 1, backend: str = "auto",
-                     out_fp32: bool = False, chunk_keys: int = 0) -> Tensor:
+                     out_fp32: bool = False, chunk_keys: int = 0, rows: Tensor | None = None) -> Tensor:
     """Single-query attention for every row of a static KV cache (reference: decode_attn.py:193-230).
 
     q        (B, H, hd) fp16 or bf16 (any (B, 1, H, hd) view is accepted); H = K * G, query head h*G+g uses kv head h.
@@ -97,6 +100,8 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
     block_n, num_warps, backend  accepted for signature compatibility; the HIP kernels choose their own tiling
              ("hip" / "auto" / "cuda" / "triton" all run the HIP path).
     out_fp32 return the fp32 result before rounding to q.dtype (for parity checks).
+    rows     optional (B,) cache row of each query row (a compacted batch of active slots over a larger cache; a negative
+             entry marks a padding row, which gets zeros).
     chunk_keys  0: every row is cut into num_splits equal chunks (the reference's rule); > 0: chunks of at least this
              many keys and at most num_splits of them per row, so short rows take fewer work items.
     Returns (B, H, hd) in q.dtype.  Graph-capturable; registered as a torch custom op (opaque to torch.compile)."""
@@ -107,6 +112,8 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
     KH, S = k_cache.shape[1], k_cache.shape[2]
     if ring is None:
         ring = window > 0
+    if rows is not None:
+        rows = rows.to(pos.dtype).contiguous()
     if num_splits is None:
         ctx = ctx_hint or S
         if window > 0:
@@ -116,4 +123,4 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
     if pos.dtype != starts.dtype:
         starts = starts.to(pos.dtype)
     return _decode_attn_op(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window),
-                           bool(ring), k_scale, v_scale, int(num_splits), bool(out_fp32), int(chunk_keys))
+                           bool(ring), k_scale, v_scale, int(num_splits), bool(out_fp32), int(chunk_keys), rows)
