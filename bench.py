@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the UV-50M decode hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c2]
+
+Workload c5 (default; BASELINE.json configs[4], the configuration the metric is quoted on): GRPO-shaped rollout,
+256 prompts x group 8 = 2048 concurrent sequences, prompt lengths U{64..256} shared inside a group, T = 1.0 with seeded
+Philox sampling, per-sequence stop length min(Geom(1/600), 2048), random-init (perturbed) UV-50M in bf16 with an int8
+KV cache.  All prompts are prefilled (untimed, reported separately), W decode steps run untimed, then exactly K decode
+steps of the rollout are timed; a step is compact -> 10-layer trunk over the active rows -> tied head -> fused sampler ->
+commit, replayed from a captured graph, with the inputs resident in HBM.  value = tokens generated in the timed steps /
+seconds.
+
+After the timed region the same steps are replayed eagerly with HIP events around every decode-attention call of a
+subsample of steps (torch's current stream is the stream the kernels are launched on) to get the attention kernel's
+average launch duration and algorithmic bytes (132 B per attended key + q/out + positions) for the roofline object.
+The cpu_baseline object times this repo's CPU restatement of the reference path (oracle/, kind "port") on a bounded
+sample of the same workload on the host cores.
+
+Workload c2 (BASELINE.json configs[1]) times the single-layer ragged int8-KV attention op alone.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _c5_requests(cfg, n_prompts=256, group=8, seed=0):
+    rng = np.random.default_rng(seed)
+    prompts, limits = [], []
+    for _ in range(n_prompts):
+        n = int(rng.integers(64, 257))
+        p = rng.integers(1, cfg.vocab_size, size=n).tolist()
+        for _ in range(group):
+            prompts.append(p)
+            limits.append(int(min(rng.geometric(1.0 / 600.0), 2048)))
+    return prompts, limits
+
+
+def _attn_bytes(pos, starts, window, B, H=8, hd=64):
+    lo = np.maximum(starts, 0)
+    if window:
+        lo = np.maximum(lo, pos - window + 1)
+    n = np.maximum(pos - lo + 1, 0)
+    return 132 * int(n.sum()) + 4 * B * H * hd + 16 * B
+
+
+def bench_c5(args):
+    from ultraviolet_amd.engine import UVEngine, UVWeights, make_config
+    from ultraviolet_amd.engine.rollout import Rollout
+    dev = "cuda:0"
+    cfg = make_config("uv-50m-alpha")
+    weights = UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02)
+    eng = UVEngine(weights, max_tokens=16384)
+    prompts, limits = _c5_requests(cfg)
+    n_seq = len(prompts)
+
+    def make_rollout(use_graph):
+        g = Rollout(eng, slots=n_seq, max_prompt=256, max_new=2048, temperature=1.0, seed=0, eos_id=None, check_every=16,
+                    bucket=128, use_graph=use_graph)
+        for i, (p, l) in enumerate(zip(prompts, limits)):
+            g.add(p, i, limit=l)
+        return g
+
+    g = make_rollout(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    g._admit()
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    prefill_tokens = sum(len(p) for p in prompts)
+    g.precapture()
+    total_steps = max(limits) - 1
+    W = min(args.warmup, total_steps - 1)
+    K = min(args.steps, total_steps - W) if args.steps > 0 else total_steps - W
+
+    def run_steps(gg, n):
+        done = 0
+        while done < n:
+            m = min(gg.ce, n - done)
+            for _ in range(m):
+                gg.step()
+            done += m
+            gg.poll()
+
+    run_steps(g, W)
+    torch.cuda.synchronize()
+    tok0 = int(g.slot_cnt[g.slot_req >= 0].sum()) + g.n_tokens
+    active0 = g.n_active()
+    t0 = time.perf_counter()
+    run_steps(g, K)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    tok1 = int(g.slot_cnt[g.slot_req >= 0].sum()) + g.n_tokens
+    gen = tok1 - tok0
+    value = gen / dt
+
+    # ---- roofline of the dominant kernel: replay the same steps eagerly with events around the attention calls
+    roof = roofline_c5(make_rollout, eng, cfg, W, K)
+    cpu = cpu_baseline_c5(cfg, prompts, limits)
+    out = {
+        "metric": "decode tok/s, UV-50M ragged batch 2048", "value": round(value, 1), "unit": "tok/s", "n_gpus": 1,
+        "steps": K, "warmup": W, "ms_per_step": round(dt * 1e3 / K, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C5 GRPO rollout: 256 prompts x 8 = 2048 sequences, prompts U{64..256}, T=1.0 Philox seed 0, "
+                               "stop min(Geom(1/600), 2048), UV-50M (10L d640 8x64 MQA, vocab 32768) bf16, int8 KV",
+                   "slots": n_seq, "active_at_start": active0, "active_at_end": g.n_active(), "tokens_timed": gen,
+                   "prefill_tokens": prefill_tokens, "prefill_s": round(prefill_s, 3),
+                   "prefill_tok_per_s": round(prefill_tokens / prefill_s, 1), "kv_cache_GB": round(g.st.nbytes() / 1e9, 3)},
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+def roofline_c5(make_rollout, eng, cfg, W, K, every=8):
+    """Average launch duration and algorithmic bytes of the global-layer decode-attention kernel over the timed steps:
+    the same rollout is replayed eagerly and every `every`-th step's attention calls are bracketed by HIP events on the
+    launch stream.  A 512 MB fill ahead of the first event keeps the GPU busy while the host enqueues event, kernel,
+    event (so the interval is not the host's launch path) and evicts the KV cache from the last-level cache, as the
+    other layers' traffic does in a real step; the cost of an empty event pair, measured the same way, is subtracted."""
+    g = make_rollout(False)
+    g._admit()
+    ev = {"global": [], "ring": []}
+    byts = {"global": 0, "ring": 0}
+    orig = g._attention
+    state = {"on": False}
+    scratch = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0")
+
+    def pair(fn=None):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        scratch.zero_()
+        e0.record()
+        out = fn() if fn else None
+        e1.record()
+        return (e0, e1), out
+
+    def timed(l, q, st, pos, starts, n, act):
+        if not state["on"]:
+            return orig(l, q, st, pos, starts, n, act)
+        p, out = pair(lambda: orig(l, q, st, pos, starts, n, act))
+        ev["global" if cfg.is_global(l) else "ring"].append(p)
+        return out
+
+    g._attention = timed
+    empty = [pair()[0] for _ in range(40)]
+    for s in range(W + K):
+        on = s >= W and (s - W) % every == 0
+        state["on"] = on
+        g.step()
+        if on:
+            torch.cuda.synchronize()
+            n = g.bucket_for(g.n_active_host)
+            live = g.act[:n].cpu().numpy() >= 0
+            p, st = g.pos_c[:n].cpu().numpy()[live], g.starts_c[:n].cpu().numpy()[live]  # what the kernels saw this step
+            byts["global"] += 2 * _attn_bytes(p, st, 0, n)
+            byts["ring"] += 8 * _attn_bytes(p, st, cfg.window, n)
+        if (s + 1) % g.ce == 0:
+            g.poll()
+    torch.cuda.synchronize()
+    overhead_us = float(np.median([a.elapsed_time(b) * 1e3 for a, b in empty]))
+    res = {}
+    for kind in ("global", "ring"):
+        us = [max(a.elapsed_time(b) * 1e3 - overhead_us, 0.1) for a, b in ev[kind]]
+        tot_us = float(np.sum(us))
+        res[kind] = {"launches": len(us), "avg_us": tot_us / max(len(us), 1), "bytes_per_launch": byts[kind] / max(len(us), 1),
+                     "GBps": byts[kind] / tot_us / 1e3 if tot_us else 0.0}
+    a = res["global"]
+    return {"bound": "hbm", "achieved": round(a["GBps"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(a["GBps"] / HBM_PEAK_GBS, 4),
+            "traffic": None, "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 4> (global layers: bf16 q, bf16 out, 4 waves per row)",
+            "avg_launch_us": round(a["avg_us"], 2), "bytes_per_launch": int(a["bytes_per_launch"]), "launches_timed": a["launches"],
+            "event_pair_overhead_us": round(overhead_us, 2),
+            "ring_layers": {"kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 2>", "achieved": round(res["ring"]["GBps"], 1),
+                            "frac": round(res["ring"]["GBps"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(res["ring"]["avg_us"], 2),
+                            "bytes_per_launch": int(res["ring"]["bytes_per_launch"]), "launches_timed": res["ring"]["launches"]}}
+
+
+def cpu_baseline_c5(cfg, prompts, limits, budget_s=15.0, rows=32):
+    """The CPU restatement of the reference path (oracle.model, torch fp32 eager) on a bounded sample: the first `rows`
+    sequences of the same workload, prefilled and then decoded greedily until the time budget is spent."""
+    from oracle.model import OracleModel, OracleState
+    from ultraviolet_amd.engine.weights import random_params
+    params = random_params(cfg, 0, perturb=0.02)
+    m = OracleModel(cfg, params, torch.float32)
+    sub = prompts[:rows]
+    st = OracleState(cfg, rows, 256 + 2048 + 1)
+    t0 = time.perf_counter()
+    tok = m.logits(m.prefill(sub, list(range(rows)), st)).argmax(-1).numpy()
+    t_pre = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    steps = 0
+    while time.perf_counter() - t0 < budget_s:
+        tok = m.logits(m.decode_step(tok, st)).argmax(-1).numpy()
+        steps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(rows * steps / dt, 2), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{rows} of the 2048 sequences (prompts U{{64..256}}), fp32 eager torch CPU oracle of the reference path, "
+                      f"{steps} greedy decode steps after a {t_pre:.1f} s prefill; host cpu_count={os.cpu_count()}, torch {torch.__version__}"}
+
+
+def bench_c2(args):
+    """BASELINE configs[1]: 256 sequences, 8 heads x 64, KH = 1, contexts U{64..1024}, bf16 q, int8 KV (cold: rotating sets)."""
+    from ultraviolet_amd.kernels import decode_attention
+    dev = "cuda:0"
+    B, S = 256, 1024
+    g = torch.Generator(device=dev).manual_seed(0)
+    nsets = 32
+    sets = []
+    for _ in range(nsets):
+        sets.append((torch.randint(-127, 128, (B, 1, S, 64), device=dev, dtype=torch.int8, generator=g),
+                     torch.randint(-127, 128, (B, 1, S, 64), device=dev, dtype=torch.int8, generator=g),
+                     (torch.rand(B, 1, S, device=dev, generator=g) * 0.03 + 0.01).half(),
+                     (torch.rand(B, 1, S, device=dev, generator=g) * 0.03 + 0.01).half()))
+    q = torch.randn(B, 8, 64, device=dev, generator=g).bfloat16()
+    n = np.random.default_rng(0).integers(64, 1025, size=B)
+    pos, starts = torch.from_numpy(n - 1).to(dev), torch.zeros(B, dtype=torch.long, device=dev)
+    byts = _attn_bytes(n - 1, np.zeros(B, np.int64), 0, B)
+    f = lambda s: decode_attention(q, s[0], s[1], pos, starts, 0.14125, k_scale=s[2], v_scale=s[3])
+    for i in range(args.warmup):
+        f(sets[i % nsets])
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        for s in sets:
+            f(s)
+    torch.cuda.synchronize()
+    reps = max(1, args.steps // nsets)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        gr.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (reps * nsets)
+    gbs = byts / us / 1e3
+    print(json.dumps({"metric": "decode attention GB/s, 256 x [64,1024] int8 KV", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+                      "steps": reps * nsets, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 5), "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "C2 single-layer ragged int8-KV decode attention, cold (32 rotating cache sets)"},
+                      "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=0, help="timed decode steps (0: the whole rollout after warm-up)")
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--workload", default="c5", choices=["c5", "c2"])
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (rollouts shard by sequence with no communication; see DESIGN.md); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    if args.workload == "c2":
+        if args.steps <= 0:
+            args.steps = 3200
+        bench_c2(args)
+    else:
+        bench_c5(args)
+
+
+if __name__ == "__main__":
+    main()

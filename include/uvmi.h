@@ -106,6 +106,13 @@ typedef struct uvmi_attn_args {
                                               decode_attn.py:42-44); > 0: chunks of at least this many keys, so short
                                               rows use fewer work items and a row that fits one chunk skips the combine */
   void* workspace; size_t workspace_bytes; /* >= uvmi_decode_attn_workspace_bytes(...) when num_splits > 1 */
+  /* Optional fused epilogue, used when post_vhat != NULL (needs head_dim 64, int8 cache, num_splits == 1): Attention.post
+   * before the output projection (ultraviolet/model.py:321-333): XSA z -= xsa[h] (z . v_hat) v_hat with the unquantized
+   * current v, then z *= 2 sigmoid(gate_w[h] . xn[:gate_ch]); out then holds that result in out_dtype. */
+  const float* post_vhat;                  /* (B, KH, hd) fp32 normalized current v (uvmi_qkv_post vhat_out); enables the epilogue */
+  const float* post_gate;                  /* (B, H) fp32 gate values (uvmi_qkv_post gate_out), or NULL */
+  const float* post_xsa;                   /* (H,) tanh(alpha) fp32, or NULL */
+  int post_round_dtype;                    /* activation dtype whose rounding the epilogue follows (F16 / BF16 / F32) */
 } uvmi_attn_args;
 
 /* Keys attended by row b: absolute positions max(starts[b], pos[b]-window+1, 0) .. pos[b]; a row with no valid
@@ -182,6 +189,10 @@ typedef struct uvmi_qkv_post_args {
   int64_t n, vocab;
   int H, KH, hd, d, ve_ch, n_pairs, S, ring, has_ve, rope;
   float eps;                           /* QK-norm epsilon */
+  /* optional inputs of the attention kernel's fused epilogue (Attention.post, model.py:324-333) */
+  const float* gate_w; int gate_ch;    /* (H, gate_ch) fp32 output-gate weights */
+  float* gate_out;                     /* (n, H) fp32: 2 sigmoid(gate_w[h] . xn[:gate_ch]), rounded as in dtype; or NULL */
+  float* vhat_out; float xsa_eps;      /* (n, KH, hd) fp32: v / max(|v|, xsa_eps); or NULL */
 } uvmi_qkv_post_args;
 int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream);
 

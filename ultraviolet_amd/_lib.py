@@ -37,7 +37,8 @@ class AttnArgs(C.Structure):
                 ("out", C.c_void_p), ("out_dtype", C.c_int), ("sob", C.c_int64), ("soh", C.c_int64),
                 ("B", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("S", C.c_int), ("hd", C.c_int),
                 ("scale", C.c_float), ("window", C.c_int), ("ring", C.c_int), ("num_splits", C.c_int),
-                ("chunk_keys", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+                ("chunk_keys", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+                ("post_vhat", C.c_void_p), ("post_gate", C.c_void_p), ("post_xsa", C.c_void_p), ("post_round_dtype", C.c_int)]
 
 
 class KvAppendArgs(C.Structure):
@@ -67,7 +68,8 @@ class QkvPostArgs(C.Structure):
                 ("n", C.c_int64), ("vocab", C.c_int64),
                 ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int), ("d", C.c_int), ("ve_ch", C.c_int),
                 ("n_pairs", C.c_int), ("S", C.c_int), ("ring", C.c_int), ("has_ve", C.c_int), ("rope", C.c_int),
-                ("eps", C.c_float)]
+                ("eps", C.c_float), ("gate_w", C.c_void_p), ("gate_ch", C.c_int), ("gate_out", C.c_void_p),
+                ("vhat_out", C.c_void_p), ("xsa_eps", C.c_float)]
 
 
 class SchedState(C.Structure):

@@ -49,6 +49,8 @@ struct AttnParams {
   int B, H, KH, G, S, hd, window, ring, splits, idx64, chunk_keys, gran;  // gran: chunk granularity (keys)
   int64_t n_items;
   float scale_log2;
+  // optional fused epilogue (Attention.post of the reference, model.py:321-333)
+  const float* post_vhat; const float* post_gate; const float* post_xsa; int post_dt;
 };
 
 // Key range of a row and how it is cut.  The span starts at lo rounded down to 32 so tiles stay aligned to the
@@ -389,7 +391,47 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
     if (rp.nsplit == 1) {
       const float inv = lfin > 0.f ? 1.0f / lfin : 0.f;
       const int64_t off = (int64_t)b * P.sob + (int64_t)(h * G + head) * P.soh + 16 * g;
-      if (ODT == UVMI_F32) {
+      if (P.post_vhat) {
+        // z (rounded to the q dtype, as the attention output tensor would be) -> XSA -> gate, written in the output type.
+        // All lanes of a head column (n, g = 0..3) are active here, so the cross-group swaps are well defined.
+        auto rnd = [&](float x, int dt) -> float {
+          return dt == UVMI_F32 ? x : (dt == UVMI_BF16 ? bf16_to_float(float_to_bf16(x)) : (float)(half_t)x);
+        };
+        const float4* vp = (const float4*)(P.post_vhat + ((int64_t)b * P.KH + h) * 64 + 16 * g);
+        const float4 v0 = vp[0], v1 = vp[1], v2 = vp[2], v3 = vp[3];
+        const float vv[16] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
+        const float gate = P.post_gate ? P.post_gate[(int64_t)b * P.H + h * G + head] : 1.0f;
+        float proj = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          o[i] = rnd(o[i] * inv, QDT);
+          proj += o[i] * vv[i];
+        }
+        if (P.post_xsa) {
+          proj = xsum32(xsum16(proj));
+          const float ah = P.post_xsa[h * G + head] * proj;
+#pragma unroll
+          for (int i = 0; i < 16; i++) o[i] = rnd(o[i] - ah * vv[i], QDT);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[i] *= gate;
+        if (ODT == UVMI_F32) {
+          float* op = (float*)P.out + off;
+#pragma unroll
+          for (int i = 0; i < 4; i++) *(float4*)(op + 4 * i) = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+        } else {
+          uint32_t w[8];
+#pragma unroll
+          for (int i = 0; i < 8; i++) {
+            const uint32_t l16 = ODT == UVMI_BF16 ? float_to_bf16(o[2 * i]) : float_to_half_bits(o[2 * i]);
+            const uint32_t h16 = ODT == UVMI_BF16 ? float_to_bf16(o[2 * i + 1]) : float_to_half_bits(o[2 * i + 1]);
+            w[i] = l16 | (h16 << 16);
+          }
+          uint16_t* op = (uint16_t*)P.out + off;
+          *(uint4*)op = uint4{w[0], w[1], w[2], w[3]};
+          *(uint4*)(op + 8) = uint4{w[4], w[5], w[6], w[7]};
+        }
+      } else if (ODT == UVMI_F32) {
         float* op = (float*)P.out + off;
 #pragma unroll
         for (int i = 0; i < 4; i++) *(float4*)(op + 4 * i) = float4{o[4 * i] * inv, o[4 * i + 1] * inv, o[4 * i + 2] * inv, o[4 * i + 3] * inv};
@@ -668,6 +710,12 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   P.n_items = (int64_t)a->B * a->KH * a->num_splits;
   P.scale_log2 = a->scale * LOG2E;
   P.ws_o = P.ws_m = P.ws_l = nullptr;
+  P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa; P.post_dt = a->post_round_dtype;
+  if (a->post_vhat) {
+    UVMI_REQUIRE(mfma_ok(a) && a->num_splits == 1, UVMI_EUNSUPPORTED,
+                 "uvmi_decode_attn: the fused post epilogue needs the MFMA kernel (head_dim 64, int8 cache) and num_splits == 1");
+    UVMI_REQUIRE(is_float_dtype(a->post_round_dtype) && ((uintptr_t)a->post_vhat % 16) == 0, UVMI_EINVAL, "uvmi_decode_attn: bad post arguments");
+  }
   if (a->num_splits > 1) {
     const size_t need = uvmi_decode_attn_workspace_bytes(a->B, a->H, a->KH, a->hd, a->num_splits);
     UVMI_REQUIRE(a->workspace && a->workspace_bytes >= need, UVMI_EWORKSPACE,

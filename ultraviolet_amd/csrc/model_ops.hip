@@ -25,6 +25,57 @@ template <> __device__ __forceinline__ float round_t<UVMI_F32>(float v) { return
 template <> __device__ __forceinline__ float round_t<UVMI_F16>(float v) { return (float)(half_t)v; }
 template <> __device__ __forceinline__ float round_t<UVMI_BF16>(float v) { return bf16_to_float(float_to_bf16(v)); }
 
+template <int DT>
+__device__ __forceinline__ void ld2(const void* p, int64_t i, float& a, float& b) {  // elements i, i+1 (i even)
+  if (DT == UVMI_F32) { const float2 v = *(const float2*)((const float*)p + i); a = v.x; b = v.y; }
+  else {
+    const uint32_t w = *(const uint32_t*)((const uint16_t*)p + i);
+    if (DT == UVMI_BF16) { a = __uint_as_float(w << 16); b = __uint_as_float(w & 0xffff0000u); }
+    else { a = half_bits_to_float(w & 0xffff); b = half_bits_to_float(w >> 16); }
+  }
+}
+template <int DT>
+__device__ __forceinline__ void st2(void* p, int64_t i, float a, float b) {
+  if (DT == UVMI_F32) *(float2*)((float*)p + i) = float2{a, b};
+  else {
+    const uint32_t lo = DT == UVMI_BF16 ? float_to_bf16(a) : float_to_half_bits(a);
+    const uint32_t hi = DT == UVMI_BF16 ? float_to_bf16(b) : float_to_half_bits(b);
+    *(uint32_t*)((uint16_t*)p + i) = lo | (hi << 16);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void ld8(const void* p, int64_t i, float (&o)[8]) {  // 8 consecutive elements starting at i
+  if (DT == UVMI_F32) {
+    const float4 a = *(const float4*)((const float*)p + i), b = *(const float4*)((const float*)p + i + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  } else {
+    const uint4 w = *(const uint4*)((const uint16_t*)p + i);
+    const uint32_t r[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      if (DT == UVMI_BF16) { o[2 * j] = __uint_as_float(r[j] << 16); o[2 * j + 1] = __uint_as_float(r[j] & 0xffff0000u); }
+      else { o[2 * j] = half_bits_to_float(r[j] & 0xffff); o[2 * j + 1] = half_bits_to_float(r[j] >> 16); }
+    }
+  }
+}
+template <int DT>
+__device__ __forceinline__ void st8(void* p, int64_t i, const float (&v)[8]) {
+  if (DT == UVMI_F32) {
+    *(float4*)((float*)p + i) = float4{v[0], v[1], v[2], v[3]};
+    *(float4*)((float*)p + i + 4) = float4{v[4], v[5], v[6], v[7]};
+  } else {
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint32_t lo = DT == UVMI_BF16 ? float_to_bf16(v[2 * j]) : float_to_half_bits(v[2 * j]);
+      const uint32_t hi = DT == UVMI_BF16 ? float_to_bf16(v[2 * j + 1]) : float_to_half_bits(v[2 * j + 1]);
+      r[j] = lo | (hi << 16);
+    }
+    *(uint4*)((uint16_t*)p + i) = uint4{r[0], r[1], r[2], r[3]};
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ embed / residual
 // MODE 0: src = E[tok[r]] ; x = rmsnorm(src)        MODE 1: x = a*xin + b*yin
 // then n = rmsnorm(x) (of the rounded x).  d <= 64 * 2 * NP.
@@ -50,10 +101,13 @@ __global__ __launch_bounds__(256) void norm_kernel(const void* __restrict__ xin,
     const int pidx = lane + 64 * i;
     v0[i] = v1[i] = 0.f;
     if (pidx < np) {
-      float x0 = elem<DT>::ld(xin, src * d + 2 * pidx), x1 = elem<DT>::ld(xin, src * d + 2 * pidx + 1);
+      float x0, x1;
+      ld2<DT>(xin, src * d + 2 * pidx, x0, x1);
       if (MODE == 1) {
-        x0 = round_t<DT>(a * x0 + b * elem<DT>::ld(yin, r * d + 2 * pidx));
-        x1 = round_t<DT>(a * x1 + b * elem<DT>::ld(yin, r * d + 2 * pidx + 1));
+        float y0, y1;
+        ld2<DT>(yin, r * d + 2 * pidx, y0, y1);
+        x0 = round_t<DT>(a * x0 + b * y0);
+        x1 = round_t<DT>(a * x1 + b * y1);
       }
       v0[i] = x0; v1[i] = x1;
       ss += x0 * x0 + x1 * x1;
@@ -73,9 +127,8 @@ __global__ __launch_bounds__(256) void norm_kernel(const void* __restrict__ xin,
   for (int i = 0; i < NP; i++) {
     const int pidx = lane + 64 * i;
     if (pidx < np) {
-      if (xout) { elem<DT>::st(xout, r * d + 2 * pidx, v0[i]); elem<DT>::st(xout, r * d + 2 * pidx + 1, v1[i]); }
-      elem<DT>::st(nout, r * d + 2 * pidx, v0[i] * rn);
-      elem<DT>::st(nout, r * d + 2 * pidx + 1, v1[i] * rn);
+      if (xout) st2<DT>(xout, r * d + 2 * pidx, v0[i], v1[i]);
+      st2<DT>(nout, r * d + 2 * pidx, v0[i] * rn, v1[i] * rn);
     }
   }
 }
@@ -86,15 +139,12 @@ struct QkvArgs {
   const int64_t* pos; const int64_t* rows; const int64_t* last_pos; const float* inv_freq;
   void* q_out; void* k_out; void* v_out;
   int8_t* k_cache; int8_t* v_cache; uint16_t* k_scale; uint16_t* v_scale;
+  const float* gate_w; float* gate_out; float* vhat_out;
   int64_t scb, sch, scs, ssb, ssh;
   int64_t n, vocab;
-  int H, KH, d, ve_ch, n_pairs, S, ring, has_ve, rope, q_dt;
-  float eps;
+  int H, KH, d, ve_ch, n_pairs, S, ring, has_ve, rope, q_dt, gate_ch;
+  float eps, xsa_eps;
 };
-
-__device__ __forceinline__ void store_q(void* p, int dt, int64_t i, float v) {
-  if (dt == UVMI_BF16) elem<UVMI_BF16>::st(p, i, v); else elem<UVMI_F16>::st(p, i, v);
-}
 
 template <int DT>
 __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
@@ -104,34 +154,107 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
   const int W = (A.H + 2 * A.KH) * 64;
   const int64_t base = r * W;
   const int64_t p = A.pos[r];
-  // RoPE angle of this lane's pair (lanes 0..n_pairs-1 and n_pairs..2n_pairs-1 share a frequency)
-  float cs = 1.f, sn = 0.f;
-  const bool rot = A.rope && lane < 2 * A.n_pairs;
-  if (rot) {
-    const float th = (float)p * A.inv_freq[lane % A.n_pairs];
-    cs = round_t<DT>(cosf(th));
-    sn = round_t<DT>(sinf(th));
+  const int np_ = A.n_pairs;
+  // ---- queries: lane (hh = lane / 8, c = lane % 8) owns dims 8c..8c+7 of head 8*pass + hh
+  {
+    const int hh = lane >> 3, c = lane & 7;
+    // RoPE angles of this lane's 8 dims (dims < 2 n_pairs rotate; dim j pairs with j +- n_pairs): one cos / sin per
+    // frequency is computed by lanes 0..n_pairs-1 and fetched by shuffle
+    float cs[8], sn[8];
+    {
+      float cl = 1.f, sl = 0.f;
+      if (A.rope && lane < np_) {
+        const float th = (float)p * A.inv_freq[lane];
+        cl = round_t<DT>(cosf(th));
+        sl = round_t<DT>(sinf(th));
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int dim = 8 * c + j;
+        const int src = A.rope ? dim % np_ : 0;
+        const float cj = __shfl(cl, src, 64), sj = __shfl(sl, src, 64);
+        const bool rot = A.rope && dim < 2 * np_;
+        cs[j] = rot ? cj : 1.f;
+        sn[j] = rot ? sj : 0.f;
+      }
+    }
+    const int pl = np_ / 8;  // lane distance of the RoPE partner chunk (n_pairs is a multiple of 8, host-checked)
+    for (int h0 = 0; h0 < A.H; h0 += 8) {
+      const int h = h0 + hh;
+      float x[8];
+      if (h < A.H) ld8<DT>(A.qkv, base + h * 64 + 8 * c, x);
+      else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = 0.f;
+      }
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+      ss += __shfl_xor(ss, 1, 64); ss += __shfl_xor(ss, 2, 64); ss += __shfl_xor(ss, 4, 64);
+      const float rs = rsqrtf(ss * (1.0f / 64.0f) + A.eps);
+#pragma unroll
+      for (int j = 0; j < 8; j++) x[j] = round_t<DT>(x[j] * rs);
+      if (A.rope) {
+        const bool first = 8 * c < np_, rot = 8 * c < 2 * np_;
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) y[j] = __shfl_xor(x[j], pl, 64);  // partner chunk: c <-> c ^ pl inside the head
+        if (rot) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) x[j] = first ? round_t<DT>(x[j] * cs[j] - y[j] * sn[j]) : round_t<DT>(y[j] * sn[j] + x[j] * cs[j]);
+        }
+      }
+      if (h < A.H) {
+        const int64_t o = (r * A.H + h) * 64 + 8 * c;
+        if (A.q_dt == UVMI_BF16) st8<UVMI_BF16>(A.q_out, o, x); else st8<UVMI_F16>(A.q_out, o, x);
+      }
+    }
+    // ---- per-head output gate 2 sigmoid(W_h . xn[:gate_ch]) for the attention epilogue (model.py:330-333)
+    if (A.gate_out) {
+      const int cpl = A.gate_ch / 8;  // channels per lane (a multiple of 8 when gate_ch % 64 == 0, else the scalar loop)
+      for (int h0 = 0; h0 < A.H; h0 += 8) {
+        const int h = h0 + hh;
+        float dot = 0.f;
+        if (h < A.H) {
+          if (cpl % 8 == 0 && (A.d % 8) == 0) {
+            for (int j = 0; j < cpl; j += 8) {
+              float xv[8];
+              ld8<DT>(A.xn, r * A.d + c * cpl + j, xv);
+              const float4 w0 = *(const float4*)(A.gate_w + h * A.gate_ch + c * cpl + j), w1 = *(const float4*)(A.gate_w + h * A.gate_ch + c * cpl + j + 4);
+              dot += xv[0] * w0.x + xv[1] * w0.y + xv[2] * w0.z + xv[3] * w0.w + xv[4] * w1.x + xv[5] * w1.y + xv[6] * w1.z + xv[7] * w1.w;
+            }
+          } else {
+            for (int j = 0; j < cpl; j++) dot += elem<DT>::ld(A.xn, r * A.d + c * cpl + j) * A.gate_w[h * A.gate_ch + c * cpl + j];
+          }
+        }
+        dot += __shfl_xor(dot, 1, 64); dot += __shfl_xor(dot, 2, 64); dot += __shfl_xor(dot, 4, 64);
+        dot = round_t<DT>(dot);
+        if (h < A.H && c == 0) A.gate_out[r * A.H + h] = round_t<DT>(2.0f * round_t<DT>(1.0f / (1.0f + __expf(-dot))));
+      }
+    }
   }
-  auto norm_rope = [&](float x) -> float {  // QK-norm over the 64 lanes, then partial RoPE (half-split pairing)
-    const float rs = rsqrtf(wave_sum(x * x) * (1.0f / 64.0f) + A.eps);
-    const float xn = round_t<DT>(x * rs);
-    if (!A.rope) return xn;
-    const float other = __shfl_xor(xn, A.n_pairs, 64);  // lane d <-> d + n_pairs (n_pairs is a power of two)
-    if (!rot) return xn;
-    return lane < A.n_pairs ? round_t<DT>(xn * cs - other * sn) : round_t<DT>(other * sn + xn * cs);
-  };
-  // ---- queries
-  for (int h = 0; h < A.H; h++) {
-    const float q = norm_rope(elem<DT>::ld(A.qkv, base + h * 64 + lane));
-    store_q(A.q_out, A.q_dt, (r * A.H + h) * 64 + lane, q);
+  // ---- keys / values per kv head: lane = dim
+  float cs1 = 1.f, sn1 = 0.f;
+  const bool rot1 = A.rope && lane < 2 * np_;
+  if (rot1) {
+    const float th = (float)p * A.inv_freq[lane % np_];
+    cs1 = round_t<DT>(cosf(th));
+    sn1 = round_t<DT>(sinf(th));
   }
-  // ---- keys / values per kv head
   const int64_t row = A.rows ? A.rows[r] : r;
   const int64_t slot = A.ring ? (p % A.S) : p;
   bool wr = A.k_cache && row >= 0 && p >= 0 && slot < A.S;
   if (wr && A.ring && A.last_pos) wr = p > A.last_pos[r] - A.S;  // only the last S positions of a prompt survive in a ring
   for (int kh = 0; kh < A.KH; kh++) {
-    const float k = norm_rope(elem<DT>::ld(A.qkv, base + (A.H + kh) * 64 + lane));
+    float k = elem<DT>::ld(A.qkv, base + (A.H + kh) * 64 + lane);
+    {
+      const float rs = rsqrtf(wave_sum(k * k) * (1.0f / 64.0f) + A.eps);
+      k = round_t<DT>(k * rs);
+      if (A.rope) {
+        const float other = __shfl_xor(k, np_, 64);
+        if (rot1) k = lane < np_ ? round_t<DT>(k * cs1 - other * sn1) : round_t<DT>(other * sn1 + k * cs1);
+      }
+    }
     float v = elem<DT>::ld(A.qkv, base + (A.H + A.KH + kh) * 64 + lane);
     if (A.has_ve) {  // v += 2 sigmoid(W xn[:ve_ch]) * value_embed[tok]
       float dot = 0.f;
@@ -146,6 +269,10 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
     }
     if (A.k_out) elem<DT>::st(A.k_out, (r * A.KH + kh) * 64 + lane, k);
     if (A.v_out) elem<DT>::st(A.v_out, (r * A.KH + kh) * 64 + lane, v);
+    if (A.vhat_out) {  // v / max(|v|, eps) in fp32 for the XSA epilogue (model.py:327)
+      const float nv = sqrtf(wave_sum(v * v));
+      A.vhat_out[(r * A.KH + kh) * 64 + lane] = v / fmaxf(nv, A.xsa_eps);
+    }
     if (wr) {  // int8 append, same arithmetic as the standalone quantizer
       const float vals[2] = {k, v};
       int8_t* caches[2] = {A.k_cache, A.v_cache};
@@ -198,15 +325,20 @@ __global__ __launch_bounds__(256) void attn_post_kernel(PostArgs A) {
 }
 
 // ------------------------------------------------------------------------------------------------ swiglu
+// f % 8 == 0 (host-checked): thread t handles 8 consecutive columns of one row
 template <int DT>
 __global__ __launch_bounds__(256) void swiglu_kernel(const void* __restrict__ gu, void* __restrict__ out, int64_t rows, int f) {
-  const int64_t total = rows * f;
+  const int f8 = f / 8;
+  const int64_t total = rows * f8;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    const int64_t r = i / f;
-    const int j = (int)(i % f);
-    const float g = elem<DT>::ld(gu, r * 2 * f + j), u = elem<DT>::ld(gu, r * 2 * f + f + j);
-    const float s = round_t<DT>(g / (1.0f + __expf(-g)));
-    elem<DT>::st(out, i, s * u);
+    const int64_t r = i / f8;
+    const int j = (int)(i % f8) * 8;
+    float g[8], u[8], o[8];
+    ld8<DT>(gu, r * 2 * f + j, g);
+    ld8<DT>(gu, r * 2 * f + f + j, u);
+#pragma unroll
+    for (int k = 0; k < 8; k++) o[k] = round_t<DT>(g[k] / (1.0f + __expf(-g[k]))) * u[k];
+    st8<DT>(out, r * (int64_t)f + j, o);
   }
 }
 
@@ -249,8 +381,11 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   UVMI_REQUIRE(a->hd == 64, UVMI_EUNSUPPORTED, "uvmi_qkv_post: head_dim %d (only 64)", a->hd);
   UVMI_REQUIRE(is_float_dtype(a->dtype) && (a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16), UVMI_EINVAL, "uvmi_qkv_post: bad dtype");
   UVMI_REQUIRE(a->n >= 0 && a->H > 0 && a->KH > 0 && a->H % a->KH == 0, UVMI_EINVAL, "uvmi_qkv_post: bad sizes");
-  UVMI_REQUIRE(!a->rope || (a->inv_freq && a->n_pairs > 0 && a->n_pairs <= 32 && (a->n_pairs & (a->n_pairs - 1)) == 0), UVMI_EUNSUPPORTED,
-               "uvmi_qkv_post: rope needs inv_freq and a power-of-two pair count <= 32");
+  UVMI_REQUIRE(!a->rope || (a->inv_freq && a->n_pairs >= 8 && a->n_pairs <= 32 && (a->n_pairs & (a->n_pairs - 1)) == 0), UVMI_EUNSUPPORTED,
+               "uvmi_qkv_post: rope needs inv_freq and 8, 16 or 32 rotated pairs");
+  UVMI_REQUIRE(!a->gate_out || (a->gate_w && a->xn && a->gate_ch > 0 && a->gate_ch % 8 == 0 && a->gate_ch <= a->d), UVMI_EINVAL,
+               "uvmi_qkv_post: gate_out needs gate_w, xn and a gate_ch that is a multiple of 8");
+  UVMI_REQUIRE(((uintptr_t)a->qkv % 16) == 0 && ((uintptr_t)a->q_out % 16) == 0, UVMI_EUNSUPPORTED, "uvmi_qkv_post: qkv and q_out must be 16-byte aligned");
   UVMI_REQUIRE(!a->has_ve || (a->xn && a->ve_table && a->ve_gate && a->tok && a->ve_ch > 0 && a->ve_ch <= 64 && a->vocab > 0), UVMI_EINVAL,
                "uvmi_qkv_post: value-embedding inputs missing");
   UVMI_REQUIRE(!a->k_cache || (a->v_cache && a->k_scale && a->v_scale && a->S > 0), UVMI_EINVAL, "uvmi_qkv_post: incomplete cache arguments");
@@ -262,6 +397,7 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   A.scb = a->scb; A.sch = a->sch; A.scs = a->scs; A.ssb = a->ssb; A.ssh = a->ssh; A.n = a->n; A.vocab = a->vocab;
   A.H = a->H; A.KH = a->KH; A.d = a->d; A.ve_ch = a->ve_ch; A.n_pairs = a->n_pairs; A.S = a->S; A.ring = a->ring; A.has_ve = a->has_ve;
   A.rope = a->rope; A.q_dt = a->q_dtype; A.eps = a->eps;
+  A.gate_w = a->gate_w; A.gate_out = a->gate_out; A.vhat_out = a->vhat_out; A.gate_ch = a->gate_ch; A.xsa_eps = a->xsa_eps;
   const dim3 grid((unsigned)((a->n + 3) / 4)), blk(256);
   dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
   UVMI_CHECK_LAUNCH("uvmi_qkv_post");
@@ -287,9 +423,10 @@ extern "C" int uvmi_attn_post(const void* z, int z_dtype, const void* v, const v
 extern "C" int uvmi_swiglu(const void* gu, int dtype, int64_t rows, int f, void* out, void* stream) {
   UVMI_REQUIRE(gu && out, UVMI_EINVAL, "uvmi_swiglu: null pointer");
   UVMI_REQUIRE(is_float_dtype(dtype) && rows >= 0 && f > 0, UVMI_EINVAL, "uvmi_swiglu: bad arguments");
+  UVMI_REQUIRE(f % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0, UVMI_EUNSUPPORTED, "uvmi_swiglu: f %% 8 and 16-byte alignment needed");
   if (rows == 0) return UVMI_OK;
-  int64_t blocks = (rows * f + 256 * 4 - 1) / (256 * 4);
-  if (blocks > 8192) blocks = 8192;
+  int64_t blocks = (rows * (f / 8) + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
   const dim3 grid((unsigned)blocks), blk(256);
   dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((swiglu_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, gu, out, rows, f); });
   UVMI_CHECK_LAUNCH("uvmi_swiglu");

@@ -16,7 +16,7 @@ import torch
 from torch import Tensor
 
 from .. import _lib as L
-from ..kernels.decode_attn import decode_attention
+from ..kernels.decode_attn import decode_attention, decode_attention_post
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
 from .weights import UVWeights
@@ -28,8 +28,11 @@ class KVState:
     layers; pos / starts (B,) int64 on the device.  pos is the next position to write."""
 
     def __init__(self, cfg: UVConfig, B: int, max_len: int, device="cuda"):
-        self.cfg, self.B, self.max_len = cfg, B, max_len
+        # Global caches are allocated with S rounded up to 32 slots: the MFMA attention kernel streams 32-key tiles and
+        # needs S % 4 == 0 for its 8-byte scale loads (other S fall back to the generic kernel).  Ring length is unchanged.
         self.local_len = min(cfg.window, max_len)
+        max_len = (max_len + 31) // 32 * 32
+        self.cfg, self.B, self.max_len = cfg, B, max_len
         dev = torch.device(device)
         self.k, self.v, self.k_scale, self.v_scale = [], [], [], []
         for l in range(cfg.n_layers):
@@ -76,7 +79,8 @@ class UVEngine:
         n, d, H, K, hd, f = max_tokens, cfg.d_model, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_ff
         e = lambda *s, dtype=dt: torch.empty(*s, dtype=dtype, device=dev)
         self.buf = dict(x=e(n, d), xn=e(n, d), h=e(n, d), qkv=e(n, (H + 2 * K) * hd), q=e(n, H, hd, dtype=self.q_dtype),
-                        k=e(n, K, hd), v=e(n, K, hd), zg=e(n, H * hd), a=e(n, d), gu=e(n, 2 * f), act=e(n, f), m=e(n, d))
+                        k=e(n, K, hd), v=e(n, K, hd), zg=e(n, H * hd), a=e(n, d), gu=e(n, 2 * f), act=e(n, f), m=e(n, d),
+                        vhat=e(n, K, hd, dtype=torch.float32), gate=e(n, H, dtype=torch.float32))
         L.lib()  # fail now if the library is missing
 
     # ------------------------------------------------------------------------------------------------ kernels
@@ -116,6 +120,10 @@ class UVEngine:
         a.ring, a.has_ve = int(not glob), int(has_ve)
         a.rope = int(((not glob) or cfg.global_rope) and cfg.n_pairs > 0)
         a.eps = self.eps
+        if cfg.xsa:
+            a.vhat_out, a.xsa_eps = b["vhat"].data_ptr(), float(cfg.xsa_eps)
+        if W["attn_gate"] is not None:
+            a.gate_w, a.gate_ch, a.gate_out = W["attn_gate"].data_ptr(), cfg.gate_ch, b["gate"].data_ptr()
         L.check(L.lib().uvmi_qkv_post(C.byref(a), L.stream_ptr(pos)), "uvmi_qkv_post")
 
     def _attn_post(self, l: int, z: Tensor, n: int):
@@ -132,9 +140,24 @@ class UVEngine:
         L.check(rc, "uvmi_swiglu")
 
     # ------------------------------------------------------------------------------------------------ trunk
+    def cache_attention(self, l: int, q: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
+        """Decode attention of layer l over the int8 cache with the fused XSA + gate epilogue; writes buf zg."""
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        glob = cfg.is_global(l)
+        S = st.k[l].size(2)
+        kw = dict(window=0 if glob else cfg.window, ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=rows)
+        # the MFMA kernel (which carries the epilogue) streams 32-key tiles: rings need S % 32 == 0, linear caches S % 4 == 0
+        if cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0:
+            out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
+            decode_attention_post(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, vhat=b["vhat"][:n],
+                                  gate=None if W["attn_gate"] is None else b["gate"][:n], xsa=W["xsa"], out=out, **kw)
+            return None
+        return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, num_splits=1, **kw)
+
     def _trunk(self, tok: Tensor, pos: Tensor, n: int, attn, rows=None, last_pos=None, st: KVState | None = None) -> Tensor:
-        """n token rows through all layers; attn(l, q (n, H, hd)) -> z (n, H, hd) runs after K/V of the layer have been
-        appended to the cache and written unquantized to buf k / v.  Returns the final normed hidden (n, d) (a buffer)."""
+        """n token rows through all layers; attn(l, q (n, H, hd)) -> z (n, H, hd) (or None when it wrote the post-processed
+        result to buf zg itself) runs after K/V of the layer have been appended to the cache and written unquantized to
+        buf k / v.  Returns the final normed hidden (n, d) (a buffer)."""
         cfg, b = self.cfg, self.buf
         assert n <= self.max_tokens
         self._embed_norm(tok, n)
@@ -143,7 +166,8 @@ class UVEngine:
             torch.mm(xn, W["wqkv"].t(), out=b["qkv"][:n])
             self._qkv_post(l, tok, pos, rows, last_pos, st, n)
             z = attn(l, b["q"][:n])
-            self._attn_post(l, z, n)
+            if z is not None:   # None: the attention kernel already applied XSA + gate and wrote buf zg
+                self._attn_post(l, z, n)
             torch.mm(b["zg"][:n], W["wo"].t(), out=b["a"][:n])
             # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
             self._add_norm(x, b["a"][:n], W["resid_attn"], W["post_attn"], n, b["h"], b["xn"])
@@ -174,11 +198,12 @@ class UVEngine:
         ns = num_splits or {}
 
         def attn(l, q):
-            if cfg.is_global(l):
-                return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0, ring=False,
-                                        k_scale=st.k_scale[l], v_scale=st.v_scale[l], num_splits=ns.get("global"))
-            return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=cfg.window, ring=True,
-                                    k_scale=st.k_scale[l], v_scale=st.v_scale[l], num_splits=ns.get("local"))
+            key = "global" if cfg.is_global(l) else "local"
+            if ns.get(key) in (None, 1):
+                return self.cache_attention(l, q, st, pos, starts, B)
+            glob = cfg.is_global(l)
+            return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0 if glob else cfg.window, ring=not glob,
+                                    k_scale=st.k_scale[l], v_scale=st.v_scale[l], num_splits=ns[key])
 
         h = self._trunk(tok, pos, B, attn, st=st)
         st.pos.add_(1)

@@ -21,7 +21,6 @@ import numpy as np
 import torch
 
 from .. import _lib as L
-from ..kernels.decode_attn import decode_attention
 from ..kernels.fused_sample import fused_sample_seeded, greedy_sample
 from .model import KVState, UVEngine
 
@@ -127,11 +126,7 @@ class Rollout:
         act, pos, starts = self.act[:n], self.pos_c[:n], self.starts_c[:n]
 
         def attn(l, q):
-            if cfg.is_global(l):
-                return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0, ring=False,
-                                        k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=act, num_splits=1)
-            return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=cfg.window, ring=True,
-                                    k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=act, num_splits=1)
+            return self._attention(l, q, st, pos, starts, n, act)
 
         h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st)
         x = e.head(h)
@@ -144,8 +139,38 @@ class Rollout:
         L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
                                       self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
 
+    def _attention(self, l, q, st, pos, starts, n, act):
+        return self.e.cache_attention(l, q, st, pos, starts, n, rows=act)
+
     def bucket_for(self, n_active: int) -> int:
         return min(self.B, max(self.bucket, -(-n_active // self.bucket) * self.bucket))
+
+    def _capture(self, n: int):
+        """Capture the step for a bucket of n rows.  A captured step mutates the slot table, so the kernels and GEMM
+        shapes are first warmed up on the live state, which is then restored; capture itself executes nothing."""
+        keep = [t.clone() for t in self._mutable()]
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self._step_body(n)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        for t, k in zip(self._mutable(), keep):
+            t.copy_(k)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._step_body(n)
+        self.graphs[n] = g
+        return g
+
+    @torch.no_grad()
+    def precapture(self):
+        """Capture every bucket from the current active count downwards (the count only shrinks between admissions), so
+        that no capture happens inside a timed or latency-sensitive region."""
+        if self.use_graph:
+            for n in range(self.bucket, self.bucket_for(self.n_active_host) + 1, self.bucket):
+                if n not in self.graphs:
+                    self._capture(min(n, self.B))
 
     @torch.no_grad()
     def step(self):
@@ -154,24 +179,7 @@ class Rollout:
         if not self.use_graph:
             self._step_body(n)
         else:
-            g = self.graphs.get(n)
-            if g is None:
-                # Capture without running: a captured step mutates the slot table, so nothing is executed until replay.
-                # The kernels and GEMM shapes for this bucket are warmed up on a scratch copy of the mutable state.
-                keep = [t.clone() for t in self._mutable()]
-                s = torch.cuda.Stream()
-                s.wait_stream(torch.cuda.current_stream())
-                with torch.cuda.stream(s):
-                    self._step_body(n)
-                torch.cuda.current_stream().wait_stream(s)
-                torch.cuda.synchronize()
-                for t, k in zip(self._mutable(), keep):
-                    t.copy_(k)
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    self._step_body(n)
-                self.graphs[n] = g
-            g.replay()
+            (self.graphs.get(n) or self._capture(n)).replay()
         self.n_decode_steps += 1
 
     def _mutable(self):

@@ -37,7 +37,8 @@ def supported(q: Tensor, k_cache: Tensor) -> bool:
                 and q.dtype in (torch.float16, torch.bfloat16))
 
 
-def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0, rows=None):
+def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0, rows=None,
+            post=None):
     B, H, hd = q.shape
     KH, S = k_cache.shape[1], k_cache.shape[2]
     int8 = k_cache.dtype == torch.int8
@@ -66,6 +67,16 @@ def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_sc
     a.scale, a.window, a.ring, a.num_splits = float(scale), int(window), int(bool(ring)), int(num_splits)
     a.chunk_keys = int(chunk_keys)
     a.workspace, a.workspace_bytes = (ws.data_ptr() if ws is not None else None), ws_bytes
+    if post is not None:
+        vhat, gate, xsa, round_dtype = post
+        assert vhat.dtype == torch.float32 and vhat.is_contiguous()
+        a.post_vhat, a.post_round_dtype = vhat.data_ptr(), L.dtype_code(round_dtype)
+        if gate is not None:
+            assert gate.dtype == torch.float32 and gate.is_contiguous()
+            a.post_gate = gate.data_ptr()
+        if xsa is not None:
+            assert xsa.dtype == torch.float32 and xsa.is_contiguous()
+            a.post_xsa = xsa.data_ptr()
     L.check(L.lib().uvmi_decode_attn(C.byref(a), L.stream_ptr(q)), "uvmi_decode_attn")
     return out
 
@@ -124,3 +135,17 @@ def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, s
         starts = starts.to(pos.dtype)
     return _decode_attn_op(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window),
                            bool(ring), k_scale, v_scale, int(num_splits), bool(out_fp32), int(chunk_keys), rows)
+
+
+def decode_attention_post(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float, *,
+                          window: int, ring: bool, k_scale: Tensor, v_scale: Tensor, vhat: Tensor, gate: Tensor | None,
+                          xsa: Tensor | None, out: Tensor, rows: Tensor | None = None) -> Tensor:
+    """decode_attention followed by the reference's Attention.post up to the output projection (XSA with the
+    unquantized current v, per-head sigmoid gate; ultraviolet/model.py:321-333) in the same kernel.  vhat (B, K, hd) fp32
+    is v / max(|v|, eps) and gate (B, H) fp32 the gate values, both produced by the qkv_post kernel; out (B, H, hd) in
+    the activation dtype is written in place.  int8 cache, head_dim 64, one chunk per row."""
+    L.require_cuda(q, k_cache, pos)
+    if rows is not None:
+        rows = rows.to(pos.dtype).contiguous()
+    return _launch(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window), bool(ring), k_scale,
+                   v_scale, 1, out, 0, rows, (vhat, gate, xsa, out.dtype))
