@@ -34,6 +34,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch / algorithmic bytes per launch of the global-layer attention kernel, from the FETCH_SIZE and
+# WRITE_SIZE counter runs summarised in profiles/c5_attention_hbm_counters.md (FETCH_SIZE scaled x2.000 and WRITE_SIZE
+# x1.000 by what they read for a 1 GiB device copy).
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.05
 
 
 def _c5_requests(cfg, n_prompts=256, group=8, seed=0):
@@ -123,66 +127,70 @@ def bench_c5(args):
     print(json.dumps(out))
 
 
-def roofline_c5(make_rollout, eng, cfg, W, K, every=8):
-    """Average launch duration and algorithmic bytes of the global-layer decode-attention kernel over the timed steps:
-    the same rollout is replayed eagerly and every `every`-th step's attention calls are bracketed by HIP events on the
-    launch stream.  A 512 MB fill ahead of the first event keeps the GPU busy while the host enqueues event, kernel,
-    event (so the interval is not the host's launch path) and evicts the KV cache from the last-level cache, as the
-    other layers' traffic does in a real step; the cost of an empty event pair, measured the same way, is subtracted."""
+def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
+    """Average launch duration and algorithmic bytes of the decode-attention kernel over the timed steps, by HIP events
+    on the launch stream.  The same rollout is replayed eagerly; after every `every`-th timed step the step's ten
+    attention launches are re-issued through the C ABI on that step's state, `reps` times back to back, between two
+    events (sequence A), and likewise the eight ring-layer launches alone (sequence B).  One step's attention working set
+    (~0.5 GB) exceeds the 256 MB last-level cache, so every launch streams from HBM as in the real step; re-issuing a
+    single launch in a loop would be served from that cache.  Global-layer time = (A - B) / 2 per step.  The launches go
+    through ctypes directly (a few microseconds each), so the host stays ahead of the GPU, and a fill kernel ahead of the
+    first event keeps the queue non-empty while the sequence is enqueued."""
+    import ctypes as C
+    from ultraviolet_amd import _lib as L
+    lib = L.lib()
     g = make_rollout(False)
     g._admit()
-    ev = {"global": [], "ring": []}
-    byts = {"global": 0, "ring": 0}
-    orig = g._attention
-    state = {"on": False}
-    scratch = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0")
+    layers = list(range(cfg.n_layers))
+    ring_layers = [l for l in layers if not cfg.is_global(l)]
+    n_glob = len(layers) - len(ring_layers)
+    scratch = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    samples = []   # (events A, events B, bytes global, bytes ring)
 
-    def pair(fn=None):
+    def timed_seq(args_list):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         scratch.zero_()
         e0.record()
-        out = fn() if fn else None
+        for _ in range(reps):
+            for a in args_list:
+                rc = lib.uvmi_decode_attn(C.byref(a), stream)
+                if rc:
+                    L.check(rc, "uvmi_decode_attn")
         e1.record()
-        return (e0, e1), out
+        return e0, e1
 
-    def timed(l, q, st, pos, starts, n, act):
-        if not state["on"]:
-            return orig(l, q, st, pos, starts, n, act)
-        p, out = pair(lambda: orig(l, q, st, pos, starts, n, act))
-        ev["global" if cfg.is_global(l) else "ring"].append(p)
-        return out
-
-    g._attention = timed
-    empty = [pair()[0] for _ in range(40)]
     for s in range(W + K):
-        on = s >= W and (s - W) % every == 0
-        state["on"] = on
         g.step()
-        if on:
+        if s >= W and (s - W) % every == 0:
             torch.cuda.synchronize()
             n = g.bucket_for(g.n_active_host)
-            live = g.act[:n].cpu().numpy() >= 0
-            p, st = g.pos_c[:n].cpu().numpy()[live], g.starts_c[:n].cpu().numpy()[live]  # what the kernels saw this step
-            byts["global"] += 2 * _attn_bytes(p, st, 0, n)
-            byts["ring"] += 8 * _attn_bytes(p, st, cfg.window, n)
+            act, pos, starts = g.act[:n], g.pos_c[:n], g.starts_c[:n]
+            built = {l: eng.cache_attention_args(l, g.st, pos, starts, n, rows=act) for l in layers}
+            evA = timed_seq([built[l][0] for l in layers])
+            evB = timed_seq([built[l][0] for l in ring_layers])
+            torch.cuda.synchronize()
+            live = act.cpu().numpy() >= 0
+            p, st = pos.cpu().numpy()[live], starts.cpu().numpy()[live]   # what the kernels saw (padding rows: no keys)
+            samples.append((evA, evB, _attn_bytes(p, st, 0, n), _attn_bytes(p, st, cfg.window, n)))
+            del built
         if (s + 1) % g.ce == 0:
             g.poll()
-    torch.cuda.synchronize()
-    overhead_us = float(np.median([a.elapsed_time(b) * 1e3 for a, b in empty]))
-    res = {}
-    for kind in ("global", "ring"):
-        us = [max(a.elapsed_time(b) * 1e3 - overhead_us, 0.1) for a, b in ev[kind]]
-        tot_us = float(np.sum(us))
-        res[kind] = {"launches": len(us), "avg_us": tot_us / max(len(us), 1), "bytes_per_launch": byts[kind] / max(len(us), 1),
-                     "GBps": byts[kind] / tot_us / 1e3 if tot_us else 0.0}
-    a = res["global"]
-    return {"bound": "hbm", "achieved": round(a["GBps"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(a["GBps"] / HBM_PEAK_GBS, 4),
-            "traffic": None, "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 4> (global layers: bf16 q, bf16 out, 4 waves per row)",
-            "avg_launch_us": round(a["avg_us"], 2), "bytes_per_launch": int(a["bytes_per_launch"]), "launches_timed": a["launches"],
-            "event_pair_overhead_us": round(overhead_us, 2),
-            "ring_layers": {"kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 2>", "achieved": round(res["ring"]["GBps"], 1),
-                            "frac": round(res["ring"]["GBps"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(res["ring"]["avg_us"], 2),
-                            "bytes_per_launch": int(res["ring"]["bytes_per_launch"]), "launches_timed": res["ring"]["launches"]}}
+    tA = sum(a.elapsed_time(b) for (a, b), _, _, _ in samples) * 1e3 / reps      # us, all layers, summed over samples
+    tB = sum(a.elapsed_time(b) for _, (a, b), _, _ in samples) * 1e3 / reps      # us, ring layers only
+    ns = len(samples)
+    glob_us = (tA - tB) / (n_glob * ns)
+    ring_us = tB / (len(ring_layers) * ns)
+    glob_bytes = sum(x[2] for x in samples) / ns
+    ring_bytes = sum(x[3] for x in samples) / ns
+    gb, rb = glob_bytes / glob_us / 1e3, ring_bytes / ring_us / 1e3
+    return {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBS, 4),
+            "traffic": int(glob_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
+            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 4> (global layers: bf16 q, bf16 out, 4 waves per row)",
+            "avg_launch_us": round(glob_us, 2), "bytes_per_launch": int(glob_bytes), "steps_sampled": ns, "launches_timed": n_glob * ns * reps,
+            "ring_layers": {"kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 2>", "achieved": round(rb, 1), "frac": round(rb / HBM_PEAK_GBS, 4),
+                            "avg_launch_us": round(ring_us, 2), "bytes_per_launch": int(ring_bytes),
+                            "launches_timed": len(ring_layers) * ns * reps}}
 
 
 def cpu_baseline_c5(cfg, prompts, limits, budget_s=15.0, rows=32):
@@ -250,12 +258,34 @@ def bench_c2(args):
                                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}))
 
 
+def bench_copy(args):
+    """Plain device-to-device copy of a known size: the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters."""
+    n = 1 << 30
+    a = torch.empty(n, dtype=torch.uint8, device="cuda:0").fill_(1)
+    b = torch.empty_like(a)
+    for _ in range(max(args.warmup, 1)):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    reps = args.steps if args.steps > 0 else 10
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        b.copy_(a)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    print(json.dumps({"metric": "device copy GB/s (read + write)", "value": round(2 * n / us / 1e3, 1), "unit": "GB/s", "n_gpus": 1,
+                      "steps": reps, "warmup": args.warmup, "ms_per_step": round(us / 1e3, 4), "higher_is_better": True, "scaling": "weak",
+                      "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+                      "config": {"workload": "copy of 1 GiB (counter calibration): reads 1073741824 B, writes 1073741824 B per launch"}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed decode steps (0: the whole rollout after warm-up)")
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c2"])
+    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "copy"])
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (rollouts shard by sequence with no communication; see DESIGN.md); "
@@ -265,7 +295,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    if args.workload == "c2":
+    if args.workload == "copy":
+        bench_copy(args)
+    elif args.workload == "c2":
         if args.steps <= 0:
             args.steps = 3200
         bench_c2(args)

@@ -16,7 +16,7 @@ import torch
 from torch import Tensor
 
 from .. import _lib as L
-from ..kernels.decode_attn import decode_attention, decode_attention_post
+from ..kernels.decode_attn import build_attn_args, decode_attention, decode_attention_post
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
 from .weights import UVWeights
@@ -153,6 +153,16 @@ class UVEngine:
                                   gate=None if W["attn_gate"] is None else b["gate"][:n], xsa=W["xsa"], out=out, **kw)
             return None
         return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, num_splits=1, **kw)
+
+    def cache_attention_args(self, l: int, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
+        """The uvmi_attn_args struct cache_attention would launch for layer l on the engine's buffers (fused path only):
+        lets a benchmark re-issue exactly the step's attention launches through the C ABI without the Python wrapper."""
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        glob = cfg.is_global(l)
+        out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
+        return build_attn_args(b["q"][:n], st.k[l], st.v[l], pos, starts, cfg.attn_scale, 0 if glob else cfg.window, not glob,
+                               st.k_scale[l], st.v_scale[l], 1, out, 0, rows,
+                               (b["vhat"][:n], None if W["attn_gate"] is None else b["gate"][:n], W["xsa"], out.dtype))
 
     def _trunk(self, tok: Tensor, pos: Tensor, n: int, attn, rows=None, last_pos=None, st: KVState | None = None) -> Tensor:
         """n token rows through all layers; attn(l, q (n, H, hd)) -> z (n, H, hd) (or None when it wrote the post-processed

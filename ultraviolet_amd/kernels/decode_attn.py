@@ -37,8 +37,10 @@ def supported(q: Tensor, k_cache: Tensor) -> bool:
                 and q.dtype in (torch.float16, torch.bfloat16))
 
 
-def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0, rows=None,
-            post=None):
+def build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0,
+                    rows=None, post=None):
+    """Fill a uvmi_attn_args struct for these tensors.  Returns (args, keepalive): the struct holds raw pointers, so the
+    caller keeps `keepalive` (and the tensors) alive until the launch has been enqueued."""
     B, H, hd = q.shape
     KH, S = k_cache.shape[1], k_cache.shape[2]
     int8 = k_cache.dtype == torch.int8
@@ -77,7 +79,15 @@ def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_sc
         if xsa is not None:
             assert xsa.dtype == torch.float32 and xsa.is_contiguous()
             a.post_xsa = xsa.data_ptr()
+    return a, (ws, rows)
+
+
+def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0, rows=None,
+            post=None):
+    a, keep = build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys,
+                              rows, post)
     L.check(L.lib().uvmi_decode_attn(C.byref(a), L.stream_ptr(q)), "uvmi_decode_attn")
+    del keep
     return out
 
 
