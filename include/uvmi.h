@@ -128,6 +128,34 @@ int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus);
 int uvmi_decode_attn_path(const uvmi_attn_args* a);
 
 /* ------------------------------------------------------------------------------------------------------------
+ * Packed (cu_seqlens) causal self-attention with an optional sliding window over unquantized K/V: the attention of
+ * a packed prefill.  Replaces varlen_attention (ultraviolet/kernels/varlen_attn.py:87-93, forward only) as called
+ * by the packed prefill (ultraviolet/kernels/fast_decode.py:117-163, 210-269).
+ * Query i of a segment sees keys j of the same segment with i - window < j <= i (window 0: every j <= i).
+ * ---------------------------------------------------------------------------------------------------------- */
+typedef struct uvmi_prefill_attn_args {
+  const void* q; int q_dtype;              /* (N, H, hd) F16 / BF16, inner stride 1 */
+  int64_t sqn, sqh;                        /* strides in elements */
+  const void* k; const void* v; int kv_dtype; /* (N, KH, hd) F16 / BF16 / F32, inner stride 1 */
+  int64_t skn, skh, svn, svh;
+  const void* cu_seqlens; int idx_dtype;   /* (n_seg + 1,) I32 / I64, non-decreasing, cu[0] = 0, cu[n_seg] = N */
+  int n_seg;
+  void* out; int out_dtype;                /* (N, H, hd) F16 / BF16 / F32, inner stride 1 */
+  int64_t son, soh;
+  int N, H, KH, hd;
+  float scale;
+  int window;
+  void* workspace; size_t workspace_bytes; /* >= uvmi_prefill_attn_workspace_bytes(N): per-token segment table */
+} uvmi_prefill_attn_args;
+/* The MFMA kernel runs when hd == 64, H / KH <= 8, q and k/v share a 16-bit dtype and rows are 16-byte aligned
+ * (probabilities are rounded to that dtype for P.V, accumulation is fp32); anything else that uvmi_decode_attn's
+ * generic kernel accepts runs there, token by token.  Two launches: the segment table, then the attention. */
+int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream);
+size_t uvmi_prefill_attn_workspace_bytes(int N);
+/* 1 = MFMA kernel, 0 = generic kernel, negative = unsupported */
+int uvmi_prefill_attn_path(const uvmi_prefill_attn_args* a);
+
+/* ------------------------------------------------------------------------------------------------------------
  * Fused softcap + categorical draw + behaviour log-prob.  Replaces fused_sample
  * (ultraviolet/kernels/fused_sample.py:68-77) and the torch.rand call feeding it (ultraviolet/perf.py:595).
  * ---------------------------------------------------------------------------------------------------------- */

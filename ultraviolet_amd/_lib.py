@@ -41,6 +41,16 @@ class AttnArgs(C.Structure):
                 ("post_vhat", C.c_void_p), ("post_gate", C.c_void_p), ("post_xsa", C.c_void_p), ("post_round_dtype", C.c_int)]
 
 
+class PrefillAttnArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("q_dtype", C.c_int), ("sqn", C.c_int64), ("sqh", C.c_int64),
+                ("k", C.c_void_p), ("v", C.c_void_p), ("kv_dtype", C.c_int),
+                ("skn", C.c_int64), ("skh", C.c_int64), ("svn", C.c_int64), ("svh", C.c_int64),
+                ("cu_seqlens", C.c_void_p), ("idx_dtype", C.c_int), ("n_seg", C.c_int),
+                ("out", C.c_void_p), ("out_dtype", C.c_int), ("son", C.c_int64), ("soh", C.c_int64),
+                ("N", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int),
+                ("scale", C.c_float), ("window", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 class KvAppendArgs(C.Structure):
     _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("x_dtype", C.c_int), ("sxb", C.c_int64), ("sxh", C.c_int64),
                 ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
@@ -96,6 +106,10 @@ def lib() -> C.CDLL:
         L.uvmi_default_splits.argtypes = [C.c_int64, C.c_int, C.c_int]
         L.uvmi_decode_attn.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
         L.uvmi_decode_attn_path.argtypes = [C.POINTER(AttnArgs)]
+        L.uvmi_prefill_attn.argtypes = [C.POINTER(PrefillAttnArgs), C.c_void_p]
+        L.uvmi_prefill_attn_path.argtypes = [C.POINTER(PrefillAttnArgs)]
+        L.uvmi_prefill_attn_workspace_bytes.restype = C.c_size_t
+        L.uvmi_prefill_attn_workspace_bytes.argtypes = [C.c_int]
         L.uvmi_quantize_rows.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int64, C.c_void_p, C.c_void_p,
                                          C.c_void_p]
         L.uvmi_dequantize_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
@@ -141,6 +155,7 @@ def require_cuda(*ts: torch.Tensor) -> None:
 
 EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_rows", "uvmi_dequantize_rows",
            "uvmi_kv_write", "uvmi_kv_append", "uvmi_decode_attn", "uvmi_decode_attn_workspace_bytes",
-           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
+           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
+           "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu",
            "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit"]

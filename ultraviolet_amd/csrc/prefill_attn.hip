@@ -1,0 +1,385 @@
+// Packed causal self-attention with an optional sliding window over unquantized K/V: the attention of a packed prefill.
+//
+// Contract (ultraviolet/kernels/varlen_attn.py:87-115 of the reference): q (N, H, hd), k / v (N, KH, hd) hold the
+// tokens of several sequences back to back, cu_seqlens their boundaries; query i sees keys j of its own sequence with
+// i - window < j <= i.
+//
+// prefill_attn_mfma_hd64 (head_dim 64, 16-bit q/k/v of one dtype, up to 8 query heads per kv head):
+//   * a wave owns 16 consecutive packed tokens x 4 query heads of one kv head, and walks the keys in 32-key
+//     super-tiles.  Query blocks are aligned to the packed index, not to the sequences: a block that straddles a
+//     boundary walks the union of its rows' key ranges and masks per (row, key), so the grid is ceil(N / 16) blocks
+//     with no search for "which sequence is block i in";
+//   * S^T = K . Q^T with v_mfma_f32_16x16x32 (A = 16 keys x 32 dims, B = 32 dims x 16 rows): a lane of the accumulator
+//     holds 4 consecutive keys of one query row, for two 16-key tiles A and B.  Exactly these 8 values, rounded to
+//     the 16-bit input type, are the lane's slice of the B operand of O^T = V^T . P^T when contraction slot 8g+j is
+//     key 4g+j of tile A (j < 4) or of tile B (j >= 4): probabilities never move between lanes;
+//   * V^T operands come from 8-byte loads (lane = dims 4m..4m+3 of 8 keys) regrouped with v_perm_b32 into four
+//     operands whose row m is head dim 4m + t; they are built once per super-tile and shared by the wave's 4 heads,
+//     as are the K operands (16-byte loads, lane = key m, dims 8g..8g+7 of each half);
+//   * loads are raw buffer loads (wave-uniform descriptor + lane-invariant offset + scalar tile offset); rows past N
+//     read as zero through the descriptor's bound.  The next super-tile is requested before the current one is used;
+//   * online softmax per (row, head) in the exp2 domain, rescaling only when some row's maximum grew; tiles that
+//     every row of the block sees completely skip the mask arithmetic;
+//   * the 4 waves of a workgroup are independent (2 query blocks x 2 head groups), so K/V of a block are fetched
+//     from L2 once per pair of waves; workgroup ids are remapped so that each XCD (one L2 each) owns a contiguous
+//     range of query blocks and therefore whole sequences.
+//
+// Everything else (fp32 K/V, other head dims) goes token by token through the decode kernel's generic path with the
+// packed K/V as a batch-stride-0 "cache".
+#include "common.h"
+
+#include <climits>
+
+namespace uvmi {
+
+typedef _Float16 ph8 __attribute__((ext_vector_type(8)));
+typedef _Float16 ph2 __attribute__((ext_vector_type(2)));
+typedef __bf16 pb8 __attribute__((ext_vector_type(8)));
+typedef __bf16 pb2 __attribute__((ext_vector_type(2)));
+typedef float pf4 __attribute__((ext_vector_type(4)));
+typedef unsigned int pu4 __attribute__((ext_vector_type(4)));
+typedef unsigned int pu2 __attribute__((ext_vector_type(2)));
+
+struct PrefillParams {
+  const void* q; const void* k; const void* v; void* out;
+  const int32_t* seg_start;  // (N,) packed index of the first token of each token's sequence
+  int64_t sqn, sqh, skn, skh, svn, svh, son, soh;
+  int N, H, KH, G, window, n_hg;
+  int64_t n_items;
+  float scale_log2;
+};
+
+// seg_start[i] = cu[s] for the last s with cu[s] <= i (empty sequences are skipped); pidx[i] = i.
+__global__ __launch_bounds__(256) void prefill_segments(const void* cu, int idx64, int n_seg, int N, int32_t* seg_start, int32_t* pidx) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  int lo = 0, hi = n_seg;  // invariant: cu[lo] <= i, and hi == n_seg or cu[hi] > i
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (load_index(cu, idx64, mid) <= i) lo = mid; else hi = mid;
+  }
+  seg_start[i] = (int32_t)load_index(cu, idx64, lo);
+  pidx[i] = i;
+}
+
+template <int DT>
+__device__ __forceinline__ pf4 mfma16(pu4 a, pu4 b, pf4 c) {
+  if constexpr (DT == UVMI_F16) {
+    ph8 x, y;
+    __builtin_memcpy(&x, &a, 16);
+    __builtin_memcpy(&y, &b, 16);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, c, 0, 0, 0);
+  } else {
+    pb8 x, y;
+    __builtin_memcpy(&x, &a, 16);
+    __builtin_memcpy(&y, &b, 16);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, c, 0, 0, 0);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {  // two fp32 -> one dword of 16-bit values, round to nearest even
+  uint32_t r;
+  if constexpr (DT == UVMI_F16) {
+    const ph2 v = ph2{(_Float16)a, (_Float16)b};
+    __builtin_memcpy(&r, &v, 4);
+  } else {
+    const pb2 v = pb2{(__bf16)a, (__bf16)b};
+    __builtin_memcpy(&r, &v, 4);
+  }
+  return r;
+}
+
+__device__ __forceinline__ float pmax16(float v) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pmax32(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float psum16(float v) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float psum32(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+struct PTile {   // one 32-key super-tile as loaded (32 dwords per lane)
+  pu4 k[4];      // [tile A dims 0..31, tile A dims 32..63, tile B dims 0..31, tile B dims 32..63]: key m, dims 8g..8g+7
+  pu2 v[8];      // keys 4g+j of tile A (j < 4) / tile B (j >= 4), dims 4m..4m+3
+};
+
+constexpr int HPW = 4;  // query heads per wave
+
+template <int DT, int ODT>
+__global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // gridDim.x is a multiple of 8; ids congruent mod 8 run on one XCD and get a contiguous range of work
+  const int per = gridDim.x >> 3;
+  const int bid = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  const int64_t item = (int64_t)bid * 4 + wave;
+  if (item >= P.n_items) return;
+  const int hg = (int)(item % P.n_hg);
+  const int64_t rest = item / P.n_hg;
+  const int kvh = (int)(rest % P.KH);
+  const int qb = (int)(rest / P.KH);
+  const int m = lane & 15, g = lane >> 4;
+  const int G = P.G;
+  const float c = P.scale_log2;
+
+  // ---- this lane's query row (accumulator column m) and its key range
+  const int r0 = qb * 16;
+  const int row = r0 + m;
+  const bool row_ok = row < P.N;
+  const int rowc = row_ok ? row : P.N - 1;
+  int lo_n = P.seg_start[rowc];
+  if (P.window > 0 && row - P.window + 1 > lo_n) lo_n = row - P.window + 1;
+  if (!row_ok) lo_n = INT_MAX;
+  const int rl = min(r0 + 15, P.N - 1);                                       // last real row of the block
+  const int lo_first = __builtin_amdgcn_readfirstlane(lo_n);                  // lo is non-decreasing in the row
+  const int lo_last = __builtin_amdgcn_readfirstlane(__shfl(lo_n, rl - r0, 64));
+  const int kbeg = lo_first & ~31, kend = rl + 1;
+
+  // ---- Q^T operands: lane (row m, group g) holds q[row][head][32 s + 8 g .. + 8] for s = 0, 1
+  pu4 Q[HPW][2];
+#pragma unroll
+  for (int hh = 0; hh < HPW; hh++) {
+    const int hq = hg * HPW + hh;
+    Q[hh][0] = Q[hh][1] = pu4{0u, 0u, 0u, 0u};
+    if (hq < G) {
+      const uint16_t* qp = (const uint16_t*)P.q + (int64_t)rowc * P.sqn + (int64_t)(kvh * G + hq) * P.sqh + 8 * g;
+      Q[hh][0] = *(const pu4*)qp;
+      Q[hh][1] = *(const pu4*)(qp + 32);
+    }
+  }
+
+  pf4 O[HPW][4];
+  float mrun[HPW], lrun[HPW];
+#pragma unroll
+  for (int hh = 0; hh < HPW; hh++) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) O[hh][t] = pf4{0.f, 0.f, 0.f, 0.f};
+    mrun[hh] = -INFINITY;
+    lrun[hh] = 0.f;
+  }
+
+  // ---- addressing: one descriptor per stream, lane-invariant byte offsets, scalar tile offsets
+  const uint16_t* kbase = (const uint16_t*)P.k + (int64_t)kvh * P.skh;
+  const uint16_t* vbase = (const uint16_t*)P.v + (int64_t)kvh * P.svh;
+  const uint32_t skn2 = (uint32_t)P.skn * 2, svn2 = (uint32_t)P.svn * 2;  // row strides in bytes
+  const uint32_t uskn2 = __builtin_amdgcn_readfirstlane(skn2), usvn2 = __builtin_amdgcn_readfirstlane(svn2);
+  const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)((uint32_t)(P.N - 1) * skn2 + 128), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (int)((uint32_t)(P.N - 1) * svn2 + 128), 0x00020000);
+  const uint32_t koA = m * skn2 + 16 * g, koB = koA + 16 * skn2;
+  const uint32_t voA = 4 * g * svn2 + 8 * m;
+
+  auto load_tile = [&](int tb_in, PTile& T) {
+    const int tb = __builtin_amdgcn_readfirstlane(tb_in);
+    const uint32_t ok = (uint32_t)tb * uskn2, ov = (uint32_t)tb * usvn2;
+    T.k[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koA, ok, 0);
+    T.k[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koA + 64, ok, 0);
+    T.k[2] = __builtin_amdgcn_raw_buffer_load_b128(rK, koB, ok, 0);
+    T.k[3] = __builtin_amdgcn_raw_buffer_load_b128(rK, koB + 64, ok, 0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      T.v[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + j * usvn2, 0);
+      T.v[4 + j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + (16 + j) * usvn2, 0);
+    }
+  };
+
+  auto step = [&](const PTile& T, int tb, bool edge) {
+    // V^T operands: operand t, row m is head dim 4m + t; dword p of an operand holds contraction slots 2p, 2p+1
+    pu4 VA[4];
+    {
+      constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;
+#pragma unroll
+      for (int p = 0; p < 4; p++) {
+        VA[0][p] = __builtin_amdgcn_perm(T.v[2 * p + 1].x, T.v[2 * p].x, LO);
+        VA[1][p] = __builtin_amdgcn_perm(T.v[2 * p + 1].x, T.v[2 * p].x, HI);
+        VA[2][p] = __builtin_amdgcn_perm(T.v[2 * p + 1].y, T.v[2 * p].y, LO);
+        VA[3][p] = __builtin_amdgcn_perm(T.v[2 * p + 1].y, T.v[2 * p].y, HI);
+      }
+    }
+    const int kA = tb + 4 * g, kB = kA + 16;  // first of this lane's 4 keys in tile A / B
+#pragma unroll
+    for (int hh = 0; hh < HPW; hh++) {
+      pf4 sA = pf4{0.f, 0.f, 0.f, 0.f}, sB = pf4{0.f, 0.f, 0.f, 0.f};
+      sA = mfma16<DT>(T.k[0], Q[hh][0], sA);
+      sB = mfma16<DT>(T.k[2], Q[hh][0], sB);
+      sA = mfma16<DT>(T.k[1], Q[hh][1], sA);
+      sB = mfma16<DT>(T.k[3], Q[hh][1], sB);
+      float t[8] = {sA[0], sA[1], sA[2], sA[3], sB[0], sB[1], sB[2], sB[3]};
+      if (edge) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          if (kA + i < lo_n || kA + i > row) t[i] = -INFINITY;
+          if (kB + i < lo_n || kB + i > row) t[4 + i] = -INFINITY;
+        }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3])), fmaxf(fmaxf(t[4], t[5]), fmaxf(t[6], t[7])));
+      mx = pmax32(pmax16(mx));
+      if (__builtin_amdgcn_ballot_w64(mx > mrun[hh]) != 0) {  // some row's maximum grew: rescale (alpha = 1 elsewhere)
+        const float mnew = fmaxf(mrun[hh], mx);
+        const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((mrun[hh] - mnew) * c);
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) O[hh][tt] *= alpha;
+        lrun[hh] *= alpha;
+        mrun[hh] = mnew;
+      }
+      const float mc = mrun[hh] == -INFINITY ? 0.f : mrun[hh] * c;
+      float p[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) p[i] = __builtin_amdgcn_exp2f(fmaf(t[i], c, -mc));
+      lrun[hh] += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      const pu4 PB = pu4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) O[hh][tt] = mfma16<DT>(VA[tt], PB, O[hh][tt]);
+    }
+  };
+
+  {
+    // a tile needs no mask when every row of the block sees all of it: it starts at or after the last row's lower
+    // bound and ends at or before the first row
+    auto edge_of = [&](int tb) { return !(tb >= lo_last && tb + 31 <= r0); };
+    auto next_of = [&](int tb) { return tb + 32 < kend ? tb + 32 : tb; };  // past the end: re-read (a cache hit)
+    int tb = kbeg;
+    PTile TA, TB;
+    load_tile(tb, TA);
+    while (true) {
+      load_tile(next_of(tb), TB);
+      step(TA, tb, edge_of(tb));
+      tb += 32;
+      if (tb >= kend) break;
+      load_tile(next_of(tb), TA);
+      step(TB, tb, edge_of(tb));
+      tb += 32;
+      if (tb >= kend) break;
+    }
+  }
+
+  // ---- normalise and store: lane (row m, group g) holds head dims 16g .. 16g+15 (O[t][i] is dim 16g + 4i + t)
+#pragma unroll
+  for (int hh = 0; hh < HPW; hh++) {
+    const int hq = hg * HPW + hh;
+    const float l = psum32(psum16(lrun[hh]));
+    if (hq >= G || !row_ok) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float o[16];
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[4 * i + t] = O[hh][t][i] * inv;
+    const int64_t off = (int64_t)row * P.son + (int64_t)(kvh * G + hq) * P.soh + 16 * g;
+    if (ODT == UVMI_F32) {
+      float* op = (float*)P.out + off;
+#pragma unroll
+      for (int i = 0; i < 4; i++) *(float4*)(op + 4 * i) = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+    } else {
+      uint32_t w[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) w[i] = ODT == UVMI_BF16 ? pack2<UVMI_BF16>(o[2 * i], o[2 * i + 1]) : pack2<UVMI_F16>(o[2 * i], o[2 * i + 1]);
+      uint16_t* op = (uint16_t*)P.out + off;
+      *(uint4*)op = uint4{w[0], w[1], w[2], w[3]};
+      *(uint4*)(op + 8) = uint4{w[4], w[5], w[6], w[7]};
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------- host side
+static int check_prefill(const uvmi_prefill_attn_args* a) {
+  UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_prefill_attn: null args");
+  UVMI_REQUIRE(a->N >= 0 && a->H > 0 && a->KH > 0 && a->hd > 0 && a->n_seg >= 0, UVMI_EINVAL, "uvmi_prefill_attn: bad sizes");
+  if (a->N == 0) return UVMI_OK;
+  UVMI_REQUIRE(a->q && a->k && a->v && a->cu_seqlens && a->out, UVMI_EINVAL, "uvmi_prefill_attn: null pointer");
+  UVMI_REQUIRE(a->n_seg >= 1, UVMI_EINVAL, "uvmi_prefill_attn: N > 0 needs at least one sequence");
+  UVMI_REQUIRE(a->H % a->KH == 0, UVMI_EINVAL, "uvmi_prefill_attn: H=%d is not a multiple of KH=%d", a->H, a->KH);
+  UVMI_REQUIRE(a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16, UVMI_EUNSUPPORTED, "uvmi_prefill_attn: q must be F16 or BF16");
+  UVMI_REQUIRE(is_float_dtype(a->kv_dtype), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: k/v must be F16, BF16 or F32");
+  UVMI_REQUIRE(is_float_dtype(a->out_dtype), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: out must be F16, BF16 or F32");
+  UVMI_REQUIRE(a->idx_dtype == UVMI_I64 || a->idx_dtype == UVMI_I32, UVMI_EINVAL, "uvmi_prefill_attn: cu_seqlens must be I32 or I64");
+  UVMI_REQUIRE(a->window >= 0, UVMI_EINVAL, "uvmi_prefill_attn: negative window");
+  UVMI_REQUIRE(a->hd <= 256 && a->H / a->KH <= 16, UVMI_EUNSUPPORTED, "uvmi_prefill_attn: head_dim %d / group %d beyond 256 / 16", a->hd,
+               a->H / a->KH);
+  const size_t need = uvmi_prefill_attn_workspace_bytes(a->N);
+  UVMI_REQUIRE(a->workspace && a->workspace_bytes >= need, UVMI_EWORKSPACE, "uvmi_prefill_attn: workspace of %zu bytes needed, %zu given",
+               need, a->workspace_bytes);
+  UVMI_REQUIRE(((uintptr_t)a->workspace % 16) == 0, UVMI_EWORKSPACE, "uvmi_prefill_attn: workspace must be 16-byte aligned");
+  return UVMI_OK;
+}
+
+static bool prefill_mfma_ok(const uvmi_prefill_attn_args* a) {
+  if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype) return false;
+  if (!(a->scale > 0.f)) return false;  // the running maximum is tracked before the (positive) softmax scale
+  auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
+  if (!al(a->q, 16) || a->sqn % 8 || a->sqh % 8) return false;
+  if (!al(a->k, 16) || a->skn % 8 || a->skh % 8 || !al(a->v, 16) || a->svn % 8 || a->svh % 8) return false;
+  if (a->skn <= 0 || a->svn <= 0) return false;
+  if ((int64_t)a->N * a->skn * 2 >= (1LL << 31) || (int64_t)a->N * a->svn * 2 >= (1LL << 31)) return false;  // 32-bit buffer offsets
+  const int ob = a->out_dtype == UVMI_F32 ? 4 : 2;
+  if (!al(a->out, 16) || (a->son * ob) % 16 || (a->soh * ob) % 16) return false;
+  return true;
+}
+
+}  // namespace uvmi
+
+using namespace uvmi;
+
+extern "C" size_t uvmi_prefill_attn_workspace_bytes(int N) {
+  if (N <= 0) return 0;
+  return (((size_t)N * 4 + 255) / 256 * 256) * 2;
+}
+
+extern "C" int uvmi_prefill_attn_path(const uvmi_prefill_attn_args* a) {
+  int rc = check_prefill(a);
+  if (rc) return rc;
+  return prefill_mfma_ok(a) ? 1 : 0;
+}
+
+extern "C" int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream) {
+  int rc = check_prefill(a);
+  if (rc) return rc;
+  if (a->N == 0) return UVMI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  int32_t* seg_start = (int32_t*)a->workspace;
+  int32_t* pidx = (int32_t*)((char*)a->workspace + ((size_t)a->N * 4 + 255) / 256 * 256);
+  hipLaunchKernelGGL(prefill_segments, dim3((unsigned)((a->N + 255) / 256)), dim3(256), 0, st, a->cu_seqlens, a->idx_dtype == UVMI_I64 ? 1 : 0,
+                     a->n_seg, a->N, seg_start, pidx);
+  UVMI_CHECK_LAUNCH("uvmi_prefill_attn(segments)");
+  if (!prefill_mfma_ok(a)) {
+    // every packed token is a decode row whose "cache" is the packed K / V of the call (batch stride 0)
+    uvmi_attn_args d = {};
+    d.q = a->q; d.q_dtype = a->q_dtype; d.sqb = a->sqn; d.sqh = a->sqh;
+    d.k_cache = a->k; d.v_cache = a->v; d.kv_dtype = a->kv_dtype;
+    d.skb = 0; d.skh = a->skh; d.sks = a->skn; d.svb = 0; d.svh = a->svh; d.svs = a->svn;
+    d.pos = pidx; d.starts = seg_start; d.idx_dtype = UVMI_I32;
+    d.out = a->out; d.out_dtype = a->out_dtype; d.sob = a->son; d.soh = a->soh;
+    d.B = a->N; d.H = a->H; d.KH = a->KH; d.S = a->N; d.hd = a->hd;
+    d.scale = a->scale; d.window = a->window; d.ring = 0; d.num_splits = 1;
+    return uvmi_decode_attn(&d, stream);
+  }
+  PrefillParams P;
+  P.q = a->q; P.k = a->k; P.v = a->v; P.out = a->out; P.seg_start = seg_start;
+  P.sqn = a->sqn; P.sqh = a->sqh; P.skn = a->skn; P.skh = a->skh; P.svn = a->svn; P.svh = a->svh; P.son = a->son; P.soh = a->soh;
+  P.N = a->N; P.H = a->H; P.KH = a->KH; P.G = a->H / a->KH; P.window = a->window;
+  P.n_hg = (P.G + HPW - 1) / HPW;
+  P.n_items = (int64_t)((a->N + 15) / 16) * a->KH * P.n_hg;
+  P.scale_log2 = a->scale * 1.4426950408889634f;
+  UVMI_REQUIRE(P.n_items < (1LL << 31), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: too many work items");
+  const unsigned nblk = (unsigned)(((P.n_items + 3) / 4 + 7) / 8 * 8);
+  const dim3 grid(nblk), blk(256);
+  const int od = a->out_dtype;
+#define UVMI_L(QD)                                                                                                \
+  do {                                                                                                            \
+    if (od == UVMI_F16) hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_F16>), grid, blk, 0, st, P);          \
+    else if (od == UVMI_BF16) hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_BF16>), grid, blk, 0, st, P);   \
+    else hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_F32>), grid, blk, 0, st, P);                         \
+  } while (0)
+  if (a->q_dtype == UVMI_F16) UVMI_L(UVMI_F16); else UVMI_L(UVMI_BF16);
+#undef UVMI_L
+  UVMI_CHECK_LAUNCH("uvmi_prefill_attn");
+  return UVMI_OK;
+}

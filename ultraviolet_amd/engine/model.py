@@ -17,6 +17,7 @@ from torch import Tensor
 
 from .. import _lib as L
 from ..kernels.decode_attn import build_attn_args, decode_attention, decode_attention_post
+from ..kernels.varlen_attn import packed_attention
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
 from .weights import UVWeights
@@ -81,7 +82,7 @@ class UVEngine:
         self.buf = dict(x=e(n, d), xn=e(n, d), h=e(n, d), qkv=e(n, (H + 2 * K) * hd), q=e(n, H, hd, dtype=self.q_dtype),
                         k=e(n, K, hd), v=e(n, K, hd), zg=e(n, H * hd), a=e(n, d), gu=e(n, 2 * f), act=e(n, f), m=e(n, d),
                         vhat=e(n, K, hd, dtype=torch.float32), gate=e(n, H, dtype=torch.float32))
-        L.lib()  # fail now if the library is missing
+        self.pf_ws = torch.empty(L.lib().uvmi_prefill_attn_workspace_bytes(n), dtype=torch.uint8, device=dev)  # fails now if the library is missing
 
     # ------------------------------------------------------------------------------------------------ kernels
     def _embed_norm(self, tok: Tensor, n: int):
@@ -246,15 +247,14 @@ class UVEngine:
         tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
         tok_t, pos_t, row_t = tt(x), tt(pos), tt(rows_np[seg])
         last_t = tt((starts + lens - 1)[seg])
-        pidx_t, pstart_t = tt(idx), tt(cu[:-1][seg])   # packed index of each token and of its segment's first token
-        K, hd, b = cfg.n_kv_heads, cfg.head_dim, self.buf
+        b = self.buf
+
+        cu_t = tt(cu)
 
         def attn(l, q):
-            # every packed token is a "row" whose cache is the packed unquantized K / V of this call (batch stride 0)
-            kp = b["k"][:N].transpose(0, 1).unsqueeze(0).expand(N, K, N, hd)
-            vp = b["v"][:N].transpose(0, 1).unsqueeze(0).expand(N, K, N, hd)
+            # causal (windowed on local layers) attention of every prompt over its own unquantized K / V of this call
             w = 0 if cfg.is_global(l) else cfg.window
-            return decode_attention(q, kp, vp, pidx_t, pstart_t, cfg.attn_scale, window=w, ring=False, num_splits=1)
+            return packed_attention(q, b["k"][:N], b["v"][:N], cu_t, cfg.attn_scale, w, workspace=self.pf_ws)
 
         h = self._trunk(tok_t, pos_t, N, attn, rows=row_t, last_pos=last_t, st=st)
         rt = tt(rows_np)

@@ -1,0 +1,72 @@
+"""Packed (cu_seqlens) causal attention with an optional sliding window: host side of uvmi_prefill_attn.
+
+Mirrors ultraviolet/kernels/varlen_attn.py:87-93 of the reference (forward only; the reference's backward belongs to
+the trainer).  q / k / v must be device tensors; there is no CPU path."""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+from torch import Tensor
+
+from .. import _lib as L
+
+
+def _args(q, k, v, cu, scale, window, out, ws):
+    N, H, hd = q.shape
+    a = L.PrefillAttnArgs()
+    a.q, a.q_dtype, a.sqn, a.sqh = q.data_ptr(), L.dtype_code(q.dtype), q.stride(0), q.stride(1)
+    a.k, a.v, a.kv_dtype = k.data_ptr(), v.data_ptr(), L.dtype_code(k.dtype)
+    a.skn, a.skh, a.svn, a.svh = k.stride(0), k.stride(1), v.stride(0), v.stride(1)
+    a.cu_seqlens, a.idx_dtype, a.n_seg = cu.data_ptr(), L.dtype_code(cu.dtype), cu.numel() - 1
+    a.out, a.out_dtype, a.son, a.soh = out.data_ptr(), L.dtype_code(out.dtype), out.stride(0), out.stride(1)
+    a.N, a.H, a.KH, a.hd = N, H, k.size(1), hd
+    a.scale, a.window = float(scale), int(window or 0)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    return a
+
+
+def packed_attention(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, scale: float, window: int | None = None,
+                     out: Tensor | None = None, out_fp32: bool = False, workspace: Tensor | None = None) -> Tensor:
+    """q (N, H, hd) fp16 / bf16, k / v (N, K, hd) (same dtype for the MFMA kernel; fp32 runs the generic kernel),
+    cu_seqlens (S+1,) int32 / int64 on the device.  Returns (N, H, hd) in q's dtype (fp32 with out_fp32), or fills `out`.
+    `workspace` (uint8, >= uvmi_prefill_attn_workspace_bytes(N)) avoids the allocation."""
+    L.require_cuda(q, k, v, cu_seqlens)
+    assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape and k.size(0) == q.size(0) and k.size(2) == q.size(2)
+    assert q.size(1) % k.size(1) == 0, "H must be a multiple of K"
+    assert cu_seqlens.dim() == 1 and cu_seqlens.numel() >= 1 and cu_seqlens.is_contiguous()
+    assert v.dtype == k.dtype
+    if q.stride(2) != 1:
+        q = q.contiguous()
+    if k.stride(2) != 1:
+        k = k.contiguous()
+    if v.stride(2) != 1:
+        v = v.contiguous()
+    N = q.size(0)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32 if out_fp32 else q.dtype, device=q.device)
+    assert out.shape == q.shape and out.stride(2) == 1
+    if N == 0:
+        return out
+    need = L.lib().uvmi_prefill_attn_workspace_bytes(N)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    assert workspace.dtype == torch.uint8 and workspace.numel() >= need
+    a = _args(q, k, v, cu_seqlens, scale, window, out, workspace)
+    L.check(L.lib().uvmi_prefill_attn(C.byref(a), L.stream_ptr(q)), "uvmi_prefill_attn")
+    return out
+
+
+def packed_attention_path(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, scale: float, window: int | None = None) -> int:
+    """1 when the MFMA kernel would run for these tensors, 0 for the generic kernel."""
+    ws = torch.empty(L.lib().uvmi_prefill_attn_workspace_bytes(q.size(0)), dtype=torch.uint8, device=q.device)
+    a = _args(q, k, v, cu_seqlens, scale, window, torch.empty_like(q), ws)
+    return int(L.lib().uvmi_prefill_attn_path(C.byref(a)))
+
+
+def varlen_attention(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, max_seqlen: int, scale: float,
+                     window: int | None = None) -> Tensor:
+    """The reference's signature: q (1, N, H, hd), k / v (1, N, K, hd) packed along N, cu_seqlens (S+1,) with cu[0] = 0
+    and cu[-1] = N; returns (1, N, H, hd).  max_seqlen is accepted for compatibility (the kernel does not need it)."""
+    assert q.dim() == 4 and q.size(0) == 1 and k.size(0) == 1 and v.size(0) == 1
+    return packed_attention(q[0], k[0], v[0], cu_seqlens, scale, window)[None]
