@@ -157,3 +157,51 @@ def test_prefill_left_pad_vs_zero_start_positions():
     d1 = eng.logits(eng.decode_step(tok, st1))
     d2 = eng.logits(eng.decode_step(tok[[1, 2, 0]], st2))
     assert (d1 - d2[[2, 0, 1]]).abs().max() < 5e-2   # keys are rotated, hence quantized, at different absolute positions
+
+
+@pytest.mark.parametrize("window", [16, 32])
+def test_mixed_step_matches_separate_prefill_and_decode(window):
+    """A mixed batch (two new prompts prefilled into free cache rows while three running rows decode, one pass over all
+    token rows) against the oracle's separate prefill and decode step: logits close, positions exact, the new rows'
+    layer-0 cache bytes equal, the running rows' appended keys equal.  window 16 takes the unfused attention epilogue,
+    window 32 the fused one."""
+    from oracle.model import OracleState
+    from ultraviolet_amd.engine import KVState
+    cfg, params, eng, OracleModel = _setup(window=window)
+    om = OracleModel(cfg, params, torch.float32)
+    old, new = _prompts(cfg, (9, 21, 14), seed=5), _prompts(cfg, (18, 7), seed=6)
+    cont = np.random.default_rng(7).integers(1, cfg.vocab_size, size=(3, 6))
+    st = KVState(cfg, 6, 64, DEV)
+    ost, ost_new = OracleState(cfg, 3, 64), OracleState(cfg, 2, 64)
+    eng.prefill(old, [0, 1, 2], st)       # left-padded positions, as the oracle (and the reference) lay prompts out
+    om.prefill(old, [0, 1, 2], ost)
+    dec_rows = torch.tensor([0, 1, 2], device=DEV)
+    for t in range(5):   # rows 0..2 run ahead with plain decode steps over their three rows
+        tok = torch.as_tensor(cont[:, t]).to(DEV)
+        h = eng._trunk(tok, st.pos[dec_rows].clone(), 3, lambda l, q: eng.cache_attention(l, q, st, st.pos[dec_rows], st.starts[dec_rows], 3, rows=dec_rows),
+                       rows=dec_rows, st=st)
+        st.pos[dec_rows] += 1
+        om.decode_step(cont[:, t], ost)
+    pk = eng.pack_prompts(new, [4, 5], st.max_len)
+    rows_d = torch.tensor([0, 1, 2, -1], device=DEV)                      # one padding row, as a bucketed step has
+    tok_d = torch.as_tensor(np.append(cont[:, 5], 0)).to(DEV)
+    pos_d = torch.cat([st.pos[dec_rows], torch.zeros(1, dtype=torch.long, device=DEV)])
+    starts_d = torch.cat([st.starts[dec_rows], torch.zeros(1, dtype=torch.long, device=DEV)])
+    hp, hd = eng.mixed_step(pk, tok_d, pos_d, starts_d, rows_d, st)
+    lg_p, lg_d = eng.logits(hp).cpu().numpy(), eng.logits(hd[:3]).cpu().numpy()
+    ref_p = om.logits(om.prefill(new, [0, 1], ost_new)).numpy()
+    ref_d = om.logits(om.decode_step(cont[:, 5], ost)).numpy()
+    assert np.abs(lg_p - ref_p).max() < 2e-2 and np.abs(lg_d - ref_d).max() < 2e-2
+    assert (lg_p.argmax(-1) == ref_p.argmax(-1)).all() and (lg_d.argmax(-1) == ref_d.argmax(-1)).all()
+    assert st.pos[4:6].tolist() == ost_new.pos.tolist() and st.starts[4:6].tolist() == ost_new.starts.tolist()
+    k0 = st.k[0].cpu().numpy()
+    S = k0.shape[2]
+    for j in range(2):                      # slots the new prompts' real tokens were written to
+        lo, hi = int(ost_new.starts[j]), int(ost_new.pos[j])
+        sl = [t if cfg.is_global(0) else t % S for t in range(lo if cfg.is_global(0) else max(lo, hi - S), hi)]
+        assert (k0[4 + j][:, sl] != ost_new.k[0][j][:, sl]).mean() < 5e-3
+    p_old = ost.pos - 1                     # the position the mixed step appended for rows 0..2
+    for r in range(3):
+        t = int(p_old[r])
+        s_ = t if cfg.is_global(0) else t % k0.shape[2]
+        assert (k0[r, :, s_] != ost.k[0][r, :, s_]).mean() < 5e-2

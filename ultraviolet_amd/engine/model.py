@@ -127,12 +127,13 @@ class UVEngine:
             a.gate_w, a.gate_ch, a.gate_out = W["attn_gate"].data_ptr(), cfg.gate_ch, b["gate"].data_ptr()
         L.check(L.lib().uvmi_qkv_post(C.byref(a), L.stream_ptr(pos)), "uvmi_qkv_post")
 
-    def _attn_post(self, l: int, z: Tensor, n: int):
+    def _attn_post(self, l: int, z: Tensor, n: int, off: int = 0):
+        """XSA + gate of rows off..off+n of the call (z holds just those rows); writes buf zg[off:off+n]."""
         cfg, b, W = self.cfg, self.buf, self.w.layers[l]
-        rc = L.lib().uvmi_attn_post(z.data_ptr(), L.dtype_code(z.dtype), b["v"].data_ptr(), b["xn"].data_ptr(), self.dt_code,
+        rc = L.lib().uvmi_attn_post(z.data_ptr(), L.dtype_code(z.dtype), b["v"][off:].data_ptr(), b["xn"][off:].data_ptr(), self.dt_code,
                                     None if W["attn_gate"] is None else W["attn_gate"].data_ptr(),
                                     None if W["xsa"] is None else W["xsa"].data_ptr(), float(cfg.xsa_eps), n, cfg.n_heads,
-                                    cfg.n_kv_heads, cfg.head_dim, cfg.d_model, cfg.gate_ch, b["zg"].data_ptr(), L.stream_ptr(z))
+                                    cfg.n_kv_heads, cfg.head_dim, cfg.d_model, cfg.gate_ch, b["zg"][off:].data_ptr(), L.stream_ptr(z))
         L.check(rc, "uvmi_attn_post")
 
     def _swiglu(self, n: int):
@@ -141,17 +142,20 @@ class UVEngine:
         L.check(rc, "uvmi_swiglu")
 
     # ------------------------------------------------------------------------------------------------ trunk
-    def cache_attention(self, l: int, q: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
-        """Decode attention of layer l over the int8 cache with the fused XSA + gate epilogue; writes buf zg."""
+    def cache_attention(self, l: int, q: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None,
+                        off: int = 0):
+        """Decode attention of layer l over the int8 cache with the fused XSA + gate epilogue for the n rows that sit at
+        off..off+n of the call's buffers (q is already that slice); writes buf zg[off:off+n] and returns None, or, where
+        the fused epilogue does not apply, returns the plain attention output for _attn_post."""
         cfg, b, W = self.cfg, self.buf, self.w.layers[l]
         glob = cfg.is_global(l)
         S = st.k[l].size(2)
         kw = dict(window=0 if glob else cfg.window, ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=rows)
         # the MFMA kernel (which carries the epilogue) streams 32-key tiles: rings need S % 32 == 0, linear caches S % 4 == 0
         if cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0:
-            out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
-            decode_attention_post(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, vhat=b["vhat"][:n],
-                                  gate=None if W["attn_gate"] is None else b["gate"][:n], xsa=W["xsa"], out=out, **kw)
+            out = b["zg"][off:off + n].view(n, cfg.n_heads, cfg.head_dim)
+            decode_attention_post(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, vhat=b["vhat"][off:off + n],
+                                  gate=None if W["attn_gate"] is None else b["gate"][off:off + n], xsa=W["xsa"], out=out, **kw)
             return None
         return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, num_splits=1, **kw)
 
@@ -221,6 +225,63 @@ class UVEngine:
         return h
 
     # ------------------------------------------------------------------------------------------------ prefill
+    def pack_prompts(self, prompts: list[list[int]], rows: list[int], max_len: int, left_pad: bool = True) -> dict:
+        """Host-built packed indices of a prefill call (reference: prefill_packed_host, fast_decode.py:210-269): per packed
+        token its id, position, cache row and the last position of its prompt; cu_seqlens; the packed index of every
+        prompt's last token; per prompt the cache row, start and end position.  All as device tensors."""
+        dev = self.device
+        lens = np.fromiter((len(p) for p in prompts), dtype=np.int64, count=len(prompts))
+        assert lens.min() > 0
+        T = int(lens.max())
+        assert T <= max_len
+        starts = (T - lens) if left_pad else np.zeros_like(lens)
+        cu = np.zeros(len(prompts) + 1, dtype=np.int64)
+        cu[1:] = np.cumsum(lens)
+        N = int(cu[-1])
+        assert N <= self.max_tokens, f"{N} prefill tokens exceed the engine's max_tokens {self.max_tokens}"
+        x = np.fromiter((t for p in prompts for t in p), dtype=np.int64, count=N)
+        seg = np.repeat(np.arange(len(prompts), dtype=np.int64), lens)
+        pos = np.arange(N, dtype=np.int64) - cu[:-1][seg] + starts[seg]
+        rows_np = np.asarray(rows, dtype=np.int64)
+        tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+        return dict(N=N, tok=tt(x), pos=tt(pos), row=tt(rows_np[seg]), last=tt((starts + lens - 1)[seg]), cu=tt(cu),
+                    last_idx=tt(cu[1:] - 1), rows=tt(rows_np), starts=tt(starts), ends=tt(starts + lens))
+
+    @staticmethod
+    def bind_prompts(pk: dict, st: KVState):
+        """Point the cache rows of a packed prefill at their prompts: starts = first position, pos = next position."""
+        st.starts[pk["rows"]] = pk["starts"]
+        st.pos[pk["rows"]] = pk["ends"]
+
+    @torch.no_grad()
+    def mixed_step(self, pk: dict, tok_d: Tensor, pos_d: Tensor, starts_d: Tensor, rows_d: Tensor, st: KVState) -> tuple[Tensor, Tensor]:
+        """One forward pass over a mixed batch: the packed prompts of `pk` (prefilled into their cache rows) followed by
+        n_d decode rows (token tok_d at position pos_d of cache row rows_d; rows_d < 0 marks padding).  Every GEMM, norm
+        and the fused QKV post-processing / cache append run once over all N_p + n_d token rows; attention runs as one
+        packed causal launch over the prompt tokens and one cache launch over the decode rows per layer.  The reference
+        runs these as two passes (its refill prefill, then the decode step: model.py:1296-1313, 1321-1330).
+        Returns the final normed hidden of each prompt's last token and of each decode row.  Does not advance st.pos of
+        the decode rows (the caller's slot table does), but binds the prompts' rows."""
+        cfg, b = self.cfg, self.buf
+        Np, nd = pk["N"], tok_d.numel()
+        N = Np + nd
+        assert N <= self.max_tokens, f"{N} token rows exceed the engine's max_tokens {self.max_tokens}"
+        tok, pos = torch.cat([pk["tok"], tok_d]), torch.cat([pk["pos"], pos_d])
+        rows, last = torch.cat([pk["row"], rows_d]), torch.cat([pk["last"], pos_d])
+
+        def attn(l, q):
+            w = 0 if cfg.is_global(l) else cfg.window
+            zp = packed_attention(q[:Np], b["k"][:Np], b["v"][:Np], pk["cu"], cfg.attn_scale, w, workspace=self.pf_ws)
+            self._attn_post(l, zp, Np)
+            zd = self.cache_attention(l, q[Np:N], st, pos_d, starts_d, nd, rows=rows_d, off=Np)
+            if zd is not None:
+                self._attn_post(l, zd, nd, off=Np)
+            return None
+
+        h = self._trunk(tok, pos, N, attn, rows=rows, last_pos=last, st=st)
+        self.bind_prompts(pk, st)
+        return h.index_select(0, pk["last_idx"]), h[Np:N]
+
     @torch.no_grad()
     def prefill(self, prompts: list[list[int]], rows: list[int], st: KVState, left_pad: bool = True) -> Tensor:
         """Packed prefill of whole prompts into cache rows `rows` (reference: prefill_packed_host, fast_decode.py:210-269):
@@ -229,38 +290,17 @@ class UVEngine:
         positions (token j of a prompt of length n sits at T - n + j, T = longest prompt of the call) so the cache
         layout equals the reference's; left_pad=False starts every prompt at position 0.  Sets st.pos / st.starts of the
         rows and returns the final normed hidden of each prompt's last token (len(prompts), d)."""
-        cfg, dev = self.cfg, self.device
-        lens = np.fromiter((len(p) for p in prompts), dtype=np.int64, count=len(prompts))
-        assert lens.min() > 0
-        T = int(lens.max())
-        assert T <= st.max_len
-        starts = (T - lens) if left_pad else np.zeros_like(lens)
-        cu = np.zeros(len(prompts) + 1, dtype=np.int64)
-        cu[1:] = np.cumsum(lens)
-        N = int(cu[-1])
-        assert N <= self.max_tokens, f"{N} prefill tokens exceed the engine's max_tokens {self.max_tokens}"
-        x = np.fromiter((t for p in prompts for t in p), dtype=np.int64, count=N)
-        seg = np.repeat(np.arange(len(prompts), dtype=np.int64), lens)
-        idx = np.arange(N, dtype=np.int64)
-        pos = idx - cu[:-1][seg] + starts[seg]
-        rows_np = np.asarray(rows, dtype=np.int64)
-        tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-        tok_t, pos_t, row_t = tt(x), tt(pos), tt(rows_np[seg])
-        last_t = tt((starts + lens - 1)[seg])
-        b = self.buf
-
-        cu_t = tt(cu)
+        pk = self.pack_prompts(prompts, rows, st.max_len, left_pad)
+        N, b, cfg = pk["N"], self.buf, self.cfg
 
         def attn(l, q):
             # causal (windowed on local layers) attention of every prompt over its own unquantized K / V of this call
             w = 0 if cfg.is_global(l) else cfg.window
-            return packed_attention(q, b["k"][:N], b["v"][:N], cu_t, cfg.attn_scale, w, workspace=self.pf_ws)
+            return packed_attention(q, b["k"][:N], b["v"][:N], pk["cu"], cfg.attn_scale, w, workspace=self.pf_ws)
 
-        h = self._trunk(tok_t, pos_t, N, attn, rows=row_t, last_pos=last_t, st=st)
-        rt = tt(rows_np)
-        st.starts[rt] = tt(starts)
-        st.pos[rt] = tt(starts + lens)
-        return h.index_select(0, tt(cu[1:] - 1))
+        h = self._trunk(pk["tok"], pk["pos"], N, attn, rows=pk["row"], last_pos=pk["last"], st=st)
+        self.bind_prompts(pk, st)
+        return h.index_select(0, pk["last_idx"])
 
     # ------------------------------------------------------------------------------------------------ generation
     @torch.no_grad()

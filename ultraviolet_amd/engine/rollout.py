@@ -28,12 +28,14 @@ from .model import KVState, UVEngine
 class Rollout:
     def __init__(self, engine: UVEngine, slots: int, max_prompt: int, max_new: int, temperature: float = 1.0,
                  seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
-                 use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False):
+                 use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False):
         self.e, self.cfg = engine, engine.cfg
         self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
         self.T, self.seed, self.eos = float(temperature), int(seed), eos_id
         self.ce, self.bucket, self.use_graph = check_every, bucket, use_graph
         self.retire_p, self.left_pad = float(retire_p), left_pad
+        self.mixed = mixed                        # admit while decoding: prompts ride in the same pass as the decode rows
+        self.n_mixed_steps = 0
         dev = engine.device
         self.dev = dev
         assert slots <= engine.max_tokens
@@ -115,6 +117,52 @@ class Rollout:
             for r, b in zip(reqs, batch):
                 self.meta[r] = (b[1], self.version)
             self.n_active_host += len(batch)
+
+    def _sample(self, x, req, cnt):
+        if self.T > 0:
+            return fused_sample_seeded(x, self.seed, req, cnt, self.cfg.softcap, self.T)
+        return greedy_sample(x, self.cfg.softcap)
+
+    @torch.no_grad()
+    def _admit_mixed(self) -> bool:
+        """Admission fused with a decode step: queued prompts (FIFO, as many as fit the engine's token rows next to the
+        decode bucket) are prefilled in the same forward pass that decodes the active slots; one head GEMM and one
+        sampler launch cover the prompts' first tokens and the decode rows.  Returns False when nothing fits."""
+        e, lib = self.e, L.lib()
+        n = self.bucket_for(self.n_active_host)
+        batch, ntok = [], 0
+        while self.queue and len(batch) < len(self.free) and ntok + len(self.queue[0][0]) <= e.max_tokens - n:
+            it = self.queue.popleft()
+            batch.append(it)
+            ntok += len(it[0])
+        if not batch:
+            return False
+        A = len(batch)
+        slots = [self.free.pop() for _ in batch]
+        reqs = list(range(self.next_req, self.next_req + A))
+        self.next_req += A
+        tt = lambda a: torch.as_tensor(a, dtype=torch.long, device=self.dev)
+        slot_t, req_t, lim_t = tt(slots), tt(reqs), tt([b[2] for b in batch])
+        pk = e.pack_prompts([b[0] for b in batch], slots, self.st.max_len, self.left_pad)
+        sp = L.stream_ptr(self.act)
+        L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                       self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
+        hp, hd = e.mixed_step(pk, self.tok_c[:n], self.pos_c[:n], self.starts_c[:n], self.act[:n], self.st)
+        x = e.head(torch.cat([hp, hd]))
+        tok, lp = self._sample(x, torch.cat([req_t, self.req_c[:n]]), torch.cat([torch.zeros_like(req_t), self.cnt_c[:n]]))
+        self.new_tok[:n].copy_(tok[A:])
+        self.new_lp[:n].copy_(lp[A:])
+        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
+                                      self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
+        tok_a, lp_a = tok[:A].contiguous(), lp[:A].contiguous()   # named: they must outlive the launch call
+        L.check(lib.uvmi_sched_admit(C.byref(self.sched), A, slot_t.data_ptr(), req_t.data_ptr(), lim_t.data_ptr(), tok_a.data_ptr(),
+                                     lp_a.data_ptr(), sp), "uvmi_sched_admit")
+        for r, b in zip(reqs, batch):
+            self.meta[r] = (b[1], self.version)
+        self.n_active_host += A
+        self.n_decode_steps += 1
+        self.n_mixed_steps += 1
+        return True
 
     # ------------------------------------------------------------------------------------------------ decode
     def _step_body(self, n: int):
@@ -218,11 +266,16 @@ class Rollout:
 
     def chunk(self):
         """Fill idle slots from the queue, decode check_every steps, harvest (reference: StreamGen.chunk)."""
+        steps = self.ce
         if self.queue and self.free:
-            self._admit()
+            if self.mixed and self.n_active() > 0:
+                while self.queue and self.free and steps > 0 and self._admit_mixed():
+                    steps -= 1
+            else:
+                self._admit()
         if self.n_active() == 0:
             return []
-        for _ in range(self.ce):
+        for _ in range(steps):
             self.step()
         return self.poll()
 
