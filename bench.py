@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the UV-50M decode hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c2|c3|c4|copy]
 
 Workload c5 (default; BASELINE.json configs[4], the configuration the metric is quoted on): GRPO-shaped rollout,
 256 prompts x group 8 = 2048 concurrent sequences, prompt lengths U{64..256} shared inside a group, T = 1.0 with seeded
@@ -11,13 +11,18 @@ steps of the rollout are timed; a step is compact -> 10-layer trunk over the act
 commit, replayed from a captured graph, with the inputs resident in HBM.  value = tokens generated in the timed steps /
 seconds.
 
-After the timed region the same steps are replayed eagerly with HIP events around every decode-attention call of a
-subsample of steps (torch's current stream is the stream the kernels are launched on) to get the attention kernel's
-average launch duration and algorithmic bytes (132 B per attended key + q/out + positions) for the roofline object.
+After the timed region the same rollout is replayed eagerly and, on a subsample of steps, the step's decode-attention
+launches are re-issued through the C ABI between HIP events on the launch stream to get the attention kernel's average
+launch duration and algorithmic bytes (132 B per attended key + q/out + positions) for the roofline object.
 The cpu_baseline object times this repo's CPU restatement of the reference path (oracle/, kind "port") on a bounded
 sample of the same workload on the host cores.
 
-Workload c2 (BASELINE.json configs[1]) times the single-layer ragged int8-KV attention op alone.
+Other workloads (parity-test configurations, timed for reference, not the headline):
+  c2    BASELINE.json configs[1]: the single-layer ragged int8-KV attention op alone, cold caches;
+  c3    configs[2]: 512 slots with contexts U{128..2048}, every step each slot retires with p = 0.01 (seeded, on the
+        device) and queued 64-token prompts are admitted into freed slots inside decode passes (mixed batches);
+  c4    configs[3]: one forward pass over 64 prompt chunks x 512 tokens packed with 448 decode rows, contexts U{256..2048};
+  copy  a 1 GiB device copy, the calibration kernel for the HBM traffic counters.
 """
 from __future__ import annotations
 
@@ -258,6 +263,131 @@ def bench_c2(args):
                                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}))
 
 
+def _fill_cache(st, rows, ctx, gen):
+    """Materialise contexts without running a prefill: random int8 K/V and fp16 scales in every cache row, pos = ctx."""
+    for l in range(len(st.k)):
+        for c, sc in ((st.k[l], st.k_scale[l]), (st.v[l], st.v_scale[l])):
+            c.copy_(torch.randint(-127, 128, c.shape, device=c.device, dtype=torch.int8, generator=gen))
+            sc.copy_((torch.rand(sc.shape, device=c.device, generator=gen) * 0.02 + 0.005).half())
+    st.pos[rows] = ctx
+    st.starts[rows] = 0
+
+
+def bench_c4(args):
+    """BASELINE configs[3]: mixed batch, 64 prompt chunks x 512 tokens + 448 decode rows, one forward pass per iteration."""
+    from ultraviolet_amd.engine import KVState, UVEngine, UVWeights, make_config
+    from ultraviolet_amd.kernels.varlen_attn import packed_attention
+    dev = "cuda:0"
+    cfg = make_config("uv-50m-alpha")
+    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02), max_tokens=64 * 512 + 512)
+    rng = np.random.default_rng(0)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    st = KVState(cfg, 512, 2048 + 64, dev)
+    nd, npf = 448, 64
+    rows_d = torch.arange(nd, device=dev)
+    ctx = torch.from_numpy(rng.integers(256, 2049, size=nd)).to(dev)
+    _fill_cache(st, rows_d, ctx, gen)
+    prompts = [rng.integers(1, cfg.vocab_size, size=512).tolist() for _ in range(npf)]
+    pk = eng.pack_prompts(prompts, list(range(nd, nd + npf)), st.max_len, left_pad=False)
+    tok_d = torch.from_numpy(rng.integers(1, cfg.vocab_size, size=nd)).to(dev)
+    pos_d, starts_d = ctx.clone(), torch.zeros(nd, dtype=torch.long, device=dev)
+    it = args.steps if args.steps > 0 else 100
+    for _ in range(max(args.warmup, 2)):
+        eng.mixed_step(pk, tok_d, pos_d, starts_d, rows_d, st)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(it):
+        eng.mixed_step(pk, tok_d, pos_d, starts_d, rows_d, st)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = e0.elapsed_time(e1) / it
+    # the two attention kernels alone, on the last pass's buffers
+    N = pk["N"]
+    b = eng.buf
+    phases = {}
+    for name, w in (("prefill_attn_global_us", 0), ("prefill_attn_local_us", cfg.window)):
+        out = torch.empty_like(b["q"][:N])
+        for _ in range(3):
+            packed_attention(b["q"][:N], b["k"][:N], b["v"][:N], pk["cu"], cfg.attn_scale, w, out=out, workspace=eng.pf_ws)
+        e0.record()
+        for _ in range(20):
+            packed_attention(b["q"][:N], b["k"][:N], b["v"][:N], pk["cu"], cfg.attn_scale, w, out=out, workspace=eng.pf_ws)
+        e1.record()
+        torch.cuda.synchronize()
+        phases[name] = round(e0.elapsed_time(e1) * 1e3 / 20, 1)
+    fl_g = 4 * 8 * 64 * npf * (512 * 513 // 2)
+    fl_l = 4 * 8 * 64 * npf * (512 * 256 - 256 * 255 // 2)
+    ntok = N + nd
+    print(json.dumps({"metric": "mixed-batch forward tok/s (64 x 512 prefill + 448 decode rows)", "value": round(ntok / (ms / 1e3), 1),
+                      "unit": "tok/s", "n_gpus": 1, "steps": it, "warmup": max(args.warmup, 2), "ms_per_step": round(ms, 4),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "C4 mixed batch: 64 prompt chunks x 512 tokens (causal, window 256 on local layers, int8 append "
+                                             "fused) packed with 448 decode rows, contexts U{256..2048}; one forward pass per step, eager launches",
+                                 "token_rows": ntok, "wall_ms_per_step": round(wall * 1e3 / it, 4), **phases,
+                                 "prefill_attn_global_TFLOPs": round(fl_g / phases["prefill_attn_global_us"] / 1e6, 1),
+                                 "prefill_attn_local_TFLOPs": round(fl_l / phases["prefill_attn_local_us"] / 1e6, 1)}}))
+
+
+def bench_c3(args):
+    """BASELINE configs[2]: 512 slots, contexts U{128..2048}, retire p = 0.01 per step, 64-token prompts admitted into freed
+    slots inside decode passes; 256 steps."""
+    from ultraviolet_amd.engine import UVEngine, UVWeights, make_config
+    from ultraviolet_amd.engine.rollout import Rollout
+    dev = "cuda:0"
+    cfg = make_config("uv-50m-alpha")
+    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02), max_tokens=4096)
+    rng = np.random.default_rng(0)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    B = 512
+    K = args.steps if args.steps > 0 else 256
+    W = args.warmup
+    g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + K + W + 64, temperature=1.0, seed=0, eos_id=None, check_every=4, bucket=128,
+                retire_p=0.01, mixed=True)
+    # running slots with materialised contexts: request ids 0..B-1, one token generated so far
+    rows = torch.arange(B, device=dev)
+    _fill_cache(g.st, rows, torch.from_numpy(rng.integers(128, 2049, size=B)).to(dev), gen)
+    g.slot_req.copy_(rows)
+    g.slot_cnt.fill_(1)
+    g.slot_limit.fill_(g.max_new)
+    g.slot_tok.copy_(torch.from_numpy(rng.integers(1, cfg.vocab_size, size=B)).to(dev))
+    g.free, g.next_req, g.n_active_host = [], B, B
+    for r in range(B):
+        g.meta[r] = (r, 0)
+    for i in range(int((W + K) * B * 0.01 * 2) + 64):
+        g.add(rng.integers(1, cfg.vocab_size, size=64).tolist(), B + i)
+    g.precapture()
+
+    def run(n):
+        s0 = g.n_decode_steps
+        while g.n_decode_steps - s0 < n:
+            g.chunk()
+
+    def generated():
+        return int(g.slot_cnt[g.slot_req >= 0].sum()) + g.n_tokens
+
+    run(W)
+    torch.cuda.synchronize()
+    tok0, s0, m0 = generated(), g.n_decode_steps, g.n_mixed_steps
+    t0 = time.perf_counter()
+    run(K)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    steps = g.n_decode_steps - s0
+    gen_tok = generated() - tok0
+    print(json.dumps({"metric": "decode tok/s, 512 slots with churn (retire p=0.01, 64-token prompts admitted in mixed batches)",
+                      "value": round(gen_tok / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": W,
+                      "ms_per_step": round(dt * 1e3 / steps, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "C3 continuous batching: UV-50M bf16, int8 KV, 512 slots, contexts U{128..2048} materialised in the "
+                                             "cache, Bernoulli(0.01) retirement per slot and step on the device, 64-token prompts admitted into "
+                                             "freed slots inside decode passes, host poll every 4 steps",
+                                 "tokens_timed": gen_tok, "mixed_steps": g.n_mixed_steps - m0, "requests_finished": g.next_req - len(g.meta),
+                                 "active_at_end": g.n_active(), "full_slot_tok_per_s": round(B * steps / dt, 1)}}))
+
+
 def bench_copy(args):
     """Plain device-to-device copy of a known size: the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters."""
     n = 1 << 30
@@ -285,7 +415,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed decode steps (0: the whole rollout after warm-up)")
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "copy"])
+    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy"])
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (rollouts shard by sequence with no communication; see DESIGN.md); "
@@ -301,6 +431,10 @@ def main():
         if args.steps <= 0:
             args.steps = 3200
         bench_c2(args)
+    elif args.workload == "c3":
+        bench_c3(args)
+    elif args.workload == "c4":
+        bench_c4(args)
     else:
         bench_c5(args)
 
