@@ -181,6 +181,11 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
             del built
         if (s + 1) % g.ce == 0:
             g.poll()
+    if os.environ.get("UVMI_BENCH_VERBOSE"):
+        for i, ((a0, a1), (b0, b1), gbts, rbts) in enumerate(samples):
+            ta, tb = a0.elapsed_time(a1) * 1e3 / reps, b0.elapsed_time(b1) * 1e3 / reps
+            print(f"# sample {i}: global {gbts / 1e6:.1f} MB {(ta - tb) / n_glob:.2f} us, ring {rbts / 1e6:.1f} MB {tb / len(ring_layers):.2f} us",
+                  file=sys.stderr)
     tA = sum(a.elapsed_time(b) for (a, b), _, _, _ in samples) * 1e3 / reps      # us, all layers, summed over samples
     tB = sum(a.elapsed_time(b) for _, (a, b), _, _ in samples) * 1e3 / reps      # us, ring layers only
     ns = len(samples)
@@ -191,7 +196,7 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
     gb, rb = glob_bytes / glob_us / 1e3, ring_bytes / ring_us / 1e3
     return {"bound": "hbm", "achieved": round(gb, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gb / HBM_PEAK_GBS, 4),
             "traffic": int(glob_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
-            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 4> (global layers: bf16 q, bf16 out, 4 waves per row)",
+            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR> (global layers: bf16 q, bf16 out; WPR = 2 waves per row while 4 would not fit the device in one round, else 4)",
             "avg_launch_us": round(glob_us, 2), "bytes_per_launch": int(glob_bytes), "steps_sampled": ns, "launches_timed": n_glob * ns * reps,
             "ring_layers": {"kernel": "uvmi::attn_mfma_i8_hd64<1, 1, 2>", "achieved": round(rb, 1), "frac": round(rb / HBM_PEAK_GBS, 4),
                             "avg_launch_us": round(ring_us, 2), "bytes_per_launch": int(ring_bytes),

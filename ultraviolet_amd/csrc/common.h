@@ -32,12 +32,12 @@ typedef _Float16 half_t;
 struct bf16_t { uint16_t bits; };
 
 __device__ __forceinline__ float bf16_to_float(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
-// round-to-nearest-even fp32 -> bf16 (NaN kept quiet)
+// round-to-nearest-even fp32 -> bf16: the hardware conversion of gfx950 (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  uint16_t r;
+  __builtin_memcpy(&r, &b, 2);
+  return r;
 }
 __device__ __forceinline__ float half_bits_to_float(uint16_t b) {
   half_t h;

@@ -56,12 +56,22 @@ struct AttnParams {
 // Key range of a row and how it is cut.  The span starts at lo rounded down to 32 so tiles stay aligned to the
 // slot grid; each work item gets `chunk` keys (a multiple of 32, at least chunk_keys, and large enough that at most
 // `splits` items cover the span).  A row with a single chunk is written directly, without partials.
-struct RowPlan { int lo, p, a0, chunk, nsplit; };
+struct RowPlan { int lo, p, a0, chunk, nsplit, cb; };
+// Low 32 bits of element i of an I32 / I64 index array (positions, starts and row ids fit 31 bits; -1 keeps its sign),
+// for a wave-uniform i: one 4-byte scalar load whatever the width (constant address space: the arrays are inputs of the
+// launch), so the three loads of a plan have no branches between them and go out together.
+__device__ __forceinline__ int load_idx32(const void* p, int is64, int64_t i) {
+  typedef const int32_t __attribute__((address_space(4))) * cptr32;
+  return *(cptr32)((uintptr_t)p + (uintptr_t)(i * (is64 ? 8 : 4)));
+}
 __device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b) {
   RowPlan r;
-  int p = (int)load_index(P.pos, P.idx64, b);
-  const int st = (int)load_index(P.starts, P.idx64, b);
-  if (P.rows && load_index(P.rows, P.idx64, b) < 0) p = -1;  // padding row of a compacted batch: no keys, output zeros
+  const int pv = load_idx32(P.pos, P.idx64, b);
+  const int st = load_idx32(P.starts, P.idx64, b);
+  const int rv = load_idx32(P.rows ? P.rows : P.pos, P.idx64, b);
+  r.cb = P.rows ? rv : b;               // cache row of this query row
+  const int p = r.cb < 0 ? -1 : pv;     // padding row of a compacted batch: no keys, output zeros
+  if (r.cb < 0) r.cb = 0;               // (dead rows have no keys; keep addresses valid)
   int lo = st > 0 ? st : 0;
   if (P.window > 0 && p - P.window + 1 > lo) lo = p - P.window + 1;
   r.lo = lo;
@@ -119,8 +129,23 @@ struct AttnState {
 // WPR waves of a workgroup share one work item (row, kv head, split): wave w takes super-tiles w, w + WPR, ... of the
 // chunk, so the workgroup streams 32 * WPR consecutive keys (2 KB * WPR of K and of V) per step, which keeps many more
 // DRAM pages open-and-hit than one wave per row does; the WPR online-softmax states are merged through LDS at the end.
+#ifdef UVMI_ATTN_TIMING
+__device__ unsigned long long g_attn_tim[1 << 15][8];
+#define UVMI_TS(k, force)                                          \
+  do {                                                             \
+    if (force) __builtin_amdgcn_s_waitcnt(0);                      \
+    tim_[k] = wall_clock64();                                      \
+  } while (0)
+#else
+#define UVMI_TS(k, force) do { } while (0)
+#endif
+
 template <int QDT, int ODT, int WPR>
 __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
+#ifdef UVMI_ATTN_TIMING
+  unsigned long long tim_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  UVMI_TS(0, 0);
+#endif
   constexpr int IPB = 4 / WPR;  // items per block
   __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
   __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
@@ -135,28 +160,36 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   }
   const int sid = (int)(item % P.splits);
   const int64_t bk = item / P.splits;
-  const int b = (int)(bk / P.KH), h = (int)(bk % P.KH);
+  const int b = __builtin_amdgcn_readfirstlane((int)(bk / P.KH)), h = __builtin_amdgcn_readfirstlane((int)(bk % P.KH));
+  const int m = lane & 15, g = lane >> 4;  // A/B operand (row, group) == accumulator (column, group)
+  const int strm = m >> 3, head = m & 7;
+  const int G = P.G;
+  const float c = P.scale_log2;
+  // The q loads depend only on the row index: they go out first, then the row's plan (three scalar loads issued
+  // together), then the first K/V tile; q is converted while that tile is in flight.
+  // (no branch around the loads: lanes of absent heads read head G-1 and are masked to zero when the operands are
+  // formed, which keeps the control flow, and with it every row-derived scalar, wave-uniform)
+  const uint32_t qmask = head < G ? 0xffffffffu : 0u;
+  const uint16_t* qp = (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + (head < G ? head : G - 1)) * P.sqh + 16 * g;
+  const uint4 qw0 = *(const uint4*)qp, qw1 = *(const uint4*)(qp + 8);
   const RowPlan rp = plan_row(P, b);
   const bool live = live_item && sid < rp.nsplit;
   if (WPR == 1 && !live) return;
   const int s0 = rp.a0 + sid * rp.chunk;
   const int s1 = live ? min(s0 + rp.chunk, rp.p + 1) : s0;
   const int lo_eff = max(rp.lo, s0);
-  const int m = lane & 15, g = lane >> 4;  // A/B operand (row, group) == accumulator (column, group)
-  const int strm = m >> 3, head = m & 7;
-  const int G = P.G;
-  const float c = P.scale_log2;
+  UVMI_TS(1, 0);
 
   // ---- Q^T operands: lane (n, g) holds q[head][16g + 8s + j] as fp16 (bf16 inputs are converted; exact for
   // 2^-14 <= |q| <= 65504).  The K operand carries a +1152 bias, cancelled by starting the accumulator at
   // -1152 * sum_d q[head][d].
-  uint32_t qr[8];
-  float qsum = 0.f;
-  {
-    const uint16_t* qp = (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + head) * P.sqh + 16 * g;
-    uint4 w0 = uint4{0, 0, 0, 0}, w1 = uint4{0, 0, 0, 0};
-    if (head < G) { w0 = *(const uint4*)qp; w1 = *(const uint4*)(qp + 8); }
-    const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+  const uint32_t mA = strm == 0 ? qmask : 0u, mB = strm == 0 ? 0u : qmask;
+  h8 QA0, QA1, QB0, QB1;
+  float cinit;
+  auto prep_q = [&]() {
+    uint32_t qr[8];
+    float qsum = 0.f;
+    const uint32_t w[8] = {qw0.x, qw0.y, qw0.z, qw0.w, qw1.x, qw1.y, qw1.z, qw1.w};
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       float f0, f1;
@@ -167,11 +200,10 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
       qsum += half_bits_to_float(l16) + half_bits_to_float(h16);
     }
     qsum = xsum32(xsum16(qsum));  // all 64 dims of this head
-  }
-  const uint32_t mA = strm == 0 ? 0xffffffffu : 0u, mB = ~mA;
-  const h8 QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA), QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
-  const h8 QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB), QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
-  const float cinit = -1152.0f * qsum;
+    QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA); QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
+    QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB); QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
+    cinit = qmask ? -1152.0f * qsum : 0.f;
+  };
 
   AttnState st;
 #pragma unroll
@@ -181,8 +213,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   st.psum = 0.f;
 
   // ---- addressing: wave-uniform row base + wave-uniform tile offset (scalar) + lane-invariant 32-bit offsets
-  int64_t cb = P.rows ? load_index(P.rows, P.idx64, b) : (int64_t)b;  // cache row of this query row
-  if (cb < 0) cb = 0;                                                 // (dead rows have no keys; keep addresses valid)
+  const int64_t cb = rp.cb;
   const int8_t* kbase = (const int8_t*)P.kc + cb * P.skb + (int64_t)h * P.skh;
   const int8_t* vbase = (const int8_t*)P.vc + cb * P.svb + (int64_t)h * P.svh;
   const uint16_t* ksb = (const uint16_t*)P.ks + cb * P.ssb + (int64_t)h * P.ssh;
@@ -307,16 +338,21 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
     constexpr int STEP = 32 * WPR;
     const int s1f = P.ring ? s1 : min(s1, S & ~31);
     int tb = s0 + 32 * wsub;
-    if (tb < s1f) {
-      int slot = P.ring ? tb % S : tb;
-      auto next_slot = [&](int sl, int t) {
-        if (t + STEP >= s1f) return sl;
-        sl += STEP;
-        if (P.ring) while (sl >= S) sl -= S;
-        return sl;
-      };
-      Tile TA, TB;
-      load_tile(slot, TA);
+    const bool has = tb < s1f;
+    int slot = has ? (P.ring ? tb % S : tb) : 0;
+    auto next_slot = [&](int sl, int t) {
+      if (t + STEP >= s1f) return sl;
+      sl += STEP;
+      if (P.ring) while (sl >= S) sl -= S;
+      return sl;
+    };
+    // The first tile is requested unconditionally (a wave without a pipelined tile reads slot 0 and drops it; the
+    // descriptor bounds the access), so that the q conversion, which waits for q only, follows it on every path.
+    Tile TA, TB;
+    load_tile(slot, TA);
+    __builtin_amdgcn_sched_barrier(0);
+    prep_q();
+    if (has) {
       while (true) {
         slot = next_slot(slot, tb);
         load_tile(slot, TB);
@@ -337,6 +373,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
     }
   }
 
+  UVMI_TS(2, 0);
   // ---- reduce l and sum P' over the 4 lane groups, merge stream B into stream A (lanes n and n^8), undo the bias
   float lsum = xsum32(xsum16(st.lrun)), ps = xsum32(xsum16(st.psum));
   const float m2 = st.mrun == -INFINITY ? -INFINITY : st.mrun * c;  // exp2 domain
@@ -364,6 +401,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
       if (g == 0) { sh_ml[wave][head][0] = mm; sh_ml[wave][head][1] = lm; }
     }
     __syncthreads();
+    UVMI_TS(3, 0);
     if (wsub != 0 || !live) return;
     if (strm == 0) {
       float mw[WPR];
@@ -401,6 +439,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
         const float4 v0 = vp[0], v1 = vp[1], v2 = vp[2], v3 = vp[3];
         const float vv[16] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
         const float gate = P.post_gate ? P.post_gate[(int64_t)b * P.H + h * G + head] : 1.0f;
+        UVMI_TS(4, 1);
         float proj = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -459,6 +498,13 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
       }
     }
   }
+#ifdef UVMI_ATTN_TIMING
+  UVMI_TS(5, 0);
+  if (lane == 0 && item < (1 << 15)) {
+    for (int k = 0; k < 6; k++) g_attn_tim[item][k] = tim_[k];
+    g_attn_tim[item][6] = (unsigned long long)(s1 - s0);
+  }
+#endif
 }
 
 // ------------------------------------------------------------------------------------------------- generic kernel
@@ -687,6 +733,12 @@ extern "C" int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus) {
   return (int)s;
 }
 
+#ifdef UVMI_ATTN_TIMING
+extern "C" int uvmi_debug_attn_timing(void* host_dst, size_t bytes) {
+  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(g_attn_tim), bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
+
 extern "C" int uvmi_decode_attn_path(const uvmi_attn_args* a) {
   int rc = check_common(a);
   if (rc) return rc;
@@ -728,9 +780,17 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   }
   UVMI_REQUIRE(P.n_items < (1LL << 31), UVMI_EUNSUPPORTED, "uvmi_decode_attn: too many work items");
   if (mfma_ok(a)) {
-    // waves per work item: long rows are streamed by all 4 waves of a workgroup, short ones by 2 or 1
+    // Waves per work item.  Long rows are streamed by all 4 waves of a workgroup, short ones by 2 or 1; and when 4 waves
+    // per item would need more wave slots than the device has at this kernel's occupancy (4 per SIMD), 2 per item keep
+    // the whole launch resident in one round instead of two (measured: 2000 rows x ~230 keys, 15.6 us against 18.9 us).
     const int ctx = a->window > 0 && a->window < a->S ? a->window : a->S;
     int wpr = ctx >= 512 ? 4 : (ctx >= 128 ? 2 : 1);
+    {
+      int cus = uvmi_device_cus();
+      if (cus <= 0) cus = 256;
+      const int64_t slots = (int64_t)cus * 16;
+      while (wpr > 1 && P.n_items * wpr > slots && P.n_items * (wpr / 2) <= slots) wpr /= 2;
+    }
     if (const char* e = getenv("UVMI_ATTN_WPR")) { const int v = atoi(e); if (v == 1 || v == 2 || v == 4) wpr = v; }
     P.gran = 32 * wpr;
     if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
