@@ -205,3 +205,57 @@ def test_mixed_step_matches_separate_prefill_and_decode(window):
         t = int(p_old[r])
         s_ = t if cfg.is_global(0) else t % k0.shape[2]
         assert (k0[r, :, s_] != ost.k[0][r, :, s_]).mean() < 5e-2
+
+
+class _StubModel:
+    """Stands in for the reference's MathLM: patch_model only reads .cfg (the reference's field names) and .state_dict()
+    (the reference's parameter names) and binds methods on the instance."""
+
+    def __init__(self, cfg, params):
+        import types
+        self.cfg = types.SimpleNamespace(**cfg.to_dict(), mudd=False, local_mixer="attn", conv_layers=None, bigram_rows=0)
+        self._sd = {k: torch.as_tensor(np.asarray(v), dtype=torch.float32, device=DEV) for k, v in params.items()}
+
+    def state_dict(self):
+        return self._sd
+
+
+def test_patch_model_binds_the_reference_entry_points():
+    """patch_model / new_state / prefill(idx, starts, st) / decode_step(tok, st, g_len) / unpatch_model with the reference's
+    signatures (fast_decode.py:70-115, 272-334, 341-364) give the engine's results; weights refresh in place."""
+    from ultraviolet_amd.engine import KVState
+    from ultraviolet_amd.kernels import fast_decode as fd
+    cfg, params, eng, _ = _setup(window=32)
+    m = fd.patch_model(_StubModel(cfg, params), kv_dtype="int8", dtype=torch.float32, max_tokens=512)
+    prompts = _prompts(cfg, (7, 19, 12), seed=8)
+    T = 19
+    idx = torch.zeros(3, T, dtype=torch.long)
+    starts = torch.tensor([T - len(p) for p in prompts])
+    for b, p in enumerate(prompts):
+        idx[b, T - len(p):] = torch.as_tensor(p)
+    st = m.new_state(3, 48)
+    assert isinstance(st, fd.KernelDecodeState) and st.kv_dtype == "int8" and st.k[0].dtype == torch.int8
+    lg = m.prefill(idx.to(DEV), starts.to(DEV), st)
+    st2 = KVState(cfg, 3, 48, DEV)
+    ref = eng.logits(eng.prefill(prompts, [0, 1, 2], st2))
+    torch.testing.assert_close(lg, ref, atol=1e-5, rtol=1e-5)
+    assert st.pos.tolist() == [T] * 3 and st.starts.tolist() == starts.tolist() and st.host_pos.tolist() == [T] * 3
+    tok = lg.argmax(-1)
+    lg1 = m.decode_step(tok, st, 64)
+    ref1 = eng.logits(eng.decode_step(tok, st2))
+    torch.testing.assert_close(lg1, ref1, atol=1e-5, rtol=1e-5)
+    assert st.pos.tolist() == [T + 1] * 3
+    h = fd.decode_step_fast(m, lg1.argmax(-1), st, 64, return_hidden=True)
+    assert h.shape == (3, cfg.d_model)
+    # in-place refresh: new parameters, same device addresses
+    ptr = m._uvmi_engine.w.layers[0]["wqkv"].data_ptr()
+    m._sd = {k: v * 1.01 if k.endswith("wq") else v for k, v in m._sd.items()}
+    fd.sync_patched_weights(m)
+    assert m._uvmi_engine.w.layers[0]["wqkv"].data_ptr() == ptr
+    lg2 = m.decode_step(tok, st, 64)
+    assert not torch.allclose(lg2, lg1)
+    fd.unpatch_model(m)
+    assert not hasattr(m, "decode_step")
+    from ultraviolet_amd import _lib as L
+    with pytest.raises(L.UvmiError):
+        fd.patch_model(_StubModel(cfg, params), kv_dtype="fp16")

@@ -167,3 +167,41 @@ def test_rollout_mixed_sampled_with_random_retirement():
         assert sorted(outs[-1]) == list(range(40))
     same = sum(outs[0][i][0] == outs[1][i][0] for i in range(40))
     assert same >= 36, same
+
+
+def test_sync_weights_inplace_keeps_graphs_and_bumps_version():
+    """New weights between chunks (scripts/rl_stream.py:22-36): tensors are overwritten in place so captured step graphs
+    keep working and pick the new weights up; requests admitted afterwards carry the new start version."""
+    from ultraviolet_amd.engine import random_params
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg, eng = _engine(torch.float32, window=32)
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(2, cfg.vocab_size, size=10).tolist() for _ in range(8)]
+    g = Rollout(eng, slots=4, max_prompt=16, max_new=12, temperature=0.0, check_every=2, bucket=4)
+    for i, p in enumerate(prompts[:4]):
+        g.add(p, i)
+    first = g.chunk()
+    n_graphs = len(g.graphs)
+    assert n_graphs > 0
+    p2 = random_params(cfg, 0, perturb=0.06)
+    for k in list(p2):
+        if k.endswith(".wq") or k.endswith("w_up"):
+            p2[k] = p2[k] * 1.05
+    g.sync_weights_inplace(p2)
+    assert g.version == 1 and len(g.graphs) == n_graphs          # no residual scalar changed: graphs kept
+    for i, p in enumerate(prompts[4:]):
+        g.add(p, 4 + i)
+    res = first + g.run(max_chunks=200)
+    assert sorted(r[0] for r in res) == list(range(8))
+    v = {r[0]: r[3] for r in res}
+    assert all(v[i] == 0 for i in range(4)) and all(v[i] == 1 for i in range(4, 8))
+    # the late requests were generated entirely under the new weights: equal to a fresh engine built from them
+    from ultraviolet_amd.engine import UVEngine, UVWeights
+    eng2 = UVEngine(UVWeights(cfg, p2, torch.float32, DEV), max_tokens=256)
+    out = {r[0]: r[1] for r in res}
+    same = sum(out[4 + i] == eng2.generate([prompts[4 + i]], 12, temperature=0.0)[0] for i in range(4))
+    assert same >= 3, same
+    p3 = dict(p2)
+    p3["blocks.0.resid_attn"] = np.float32(0.9)
+    g.sync_weights_inplace(p3)
+    assert g.version == 2 and len(g.graphs) == 0                 # a launch-argument scalar changed: recapture

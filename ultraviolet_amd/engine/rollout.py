@@ -86,6 +86,17 @@ class Rollout:
         self.queue = collections.deque(keep)
         return n
 
+    @torch.no_grad()
+    def sync_weights_inplace(self, params: dict):
+        """New policy weights for the following steps (reference: sync_weights_inplace + the version counter of
+        StreamGen, scripts/rl_stream.py:22-36, 152-154): the fused tensors are overwritten in place, so captured step
+        graphs stay valid; they are only dropped when a residual scalar (a launch argument) changed.  Requests admitted
+        from now on carry the new version as their start_version."""
+        if self.e.w.load_(params):
+            self.graphs.clear()
+        torch.cuda.synchronize(self.dev)
+        self.version += 1
+
     # ------------------------------------------------------------------------------------------------ admission
     @torch.no_grad()
     def _admit(self):

@@ -64,11 +64,24 @@ class UVWeights:
 
     def __init__(self, cfg: UVConfig, params: dict, dtype=torch.bfloat16, device="cuda"):
         self.cfg, self.dtype, self.device = cfg, dtype, torch.device(device)
-        t = lambda a: torch.as_tensor(np.asarray(a), dtype=torch.float32)
-        dev = self.device
-        self.embed = t(params["embed.weight"]).to(dtype).to(dev).contiguous()
-        self.value_embed = t(params["value_embed.weight"]).to(dtype).to(dev).contiguous() if cfg.use_ve else None
-        self.layers = []
+        self.embed, self.value_embed, self.layers = self._fuse(params)
+        n_pairs = cfg.n_pairs
+        # Rotary.inv_freq (model.py:203-205), same torch expression so the buffer is bit-identical
+        self.inv_freq = ((1.0 / cfg.rope_base) ** torch.linspace(0, 1, n_pairs, dtype=torch.float32)).to(self.device) \
+            if n_pairs else torch.zeros(1, device=self.device)
+
+    def _fuse(self, params: dict):
+        """The reference's fuse_for_inference (model.py:289-300, 384-386) on a name -> array mapping."""
+        cfg, dtype, dev = self.cfg, self.dtype, self.device
+
+        def t(a):
+            if isinstance(a, torch.Tensor):
+                return a.detach().to("cpu", torch.float32)
+            return torch.as_tensor(np.asarray(a), dtype=torch.float32)
+
+        embed = t(params["embed.weight"]).to(dtype).to(dev).contiguous()
+        value_embed = t(params["value_embed.weight"]).to(dtype).to(dev).contiguous() if cfg.use_ve else None
+        layers = []
         for l in range(cfg.n_layers):
             a, m = f"blocks.{l}.attn.", f"blocks.{l}.mlp."
             # fuse(): cat(wq, wk, wv) * qkv_scale and wo * o_scale are formed in fp32, then cast (model.py:292-293)
@@ -88,11 +101,27 @@ class UVWeights:
             # the four residual scalars are cast to the activation dtype before use (model.py:568-571)
             for s in ("resid_attn", "post_attn", "resid_mlp", "post_mlp"):
                 L[s] = float(torch.tensor(float(params[f"blocks.{l}.{s}"])).to(dtype).float())
-            self.layers.append(L)
-        n_pairs = cfg.n_pairs
-        # Rotary.inv_freq (model.py:203-205), same torch expression so the buffer is bit-identical
-        self.inv_freq = ((1.0 / cfg.rope_base) ** torch.linspace(0, 1, n_pairs, dtype=torch.float32)).to(dev) \
-            if n_pairs else torch.zeros(1, device=dev)
+            layers.append(L)
+        return embed, value_embed, layers
+
+    @torch.no_grad()
+    def load_(self, params: dict) -> bool:
+        """Refresh every fused tensor in place from new parameters (same names and shapes), keeping device addresses, as
+        the reference's sync_weights_inplace does for its fused weights (scripts/rl_stream.py:22-36).  Returns True when
+        one of the residual scalars changed: those are launch arguments, so graphs captured earlier must be recaptured."""
+        embed, value_embed, layers = self._fuse(params)
+        self.embed.copy_(embed)
+        if self.value_embed is not None:
+            self.value_embed.copy_(value_embed)
+        scalars_changed = False
+        for old, new in zip(self.layers, layers):
+            for k, v in new.items():
+                if isinstance(v, torch.Tensor):
+                    old[k].copy_(v)
+                elif v is not None and old[k] != v:
+                    old[k] = v
+                    scalars_changed = True
+        return scalars_changed
 
     @classmethod
     def random(cls, cfg: UVConfig, seed: int = 0, dtype=torch.bfloat16, device="cuda", **kw) -> "UVWeights":
@@ -103,8 +132,7 @@ class UVWeights:
         """ckpt = {"model": state_dict, "cfg": dict} as the reference saves it (README.md:26-28)."""
         fields = UVConfig.__dataclass_fields__
         cfg = UVConfig(**{k: v for k, v in ckpt["cfg"].items() if k in fields})
-        sd = {k: (v.detach().float().cpu().numpy() if isinstance(v, torch.Tensor) else v) for k, v in ckpt["model"].items()}
-        return cls(cfg, sd, dtype, device)
+        return cls(cfg, ckpt["model"], dtype, device)
 
     def nbytes(self) -> int:
         n = self.embed.numel() * self.embed.element_size()

@@ -1,0 +1,141 @@
+"""Model-level mirror of ultraviolet/kernels/fast_decode.py: the names a caller of the reference's kernel decode path
+uses (KernelDecodeState, prefill_fast, decode_step_fast, patch_model, unpatch_model, kv_bytes_per_seq), backed by the
+UV engine of this package.  patch_model(model) reads model.cfg and model.state_dict() (the reference's MathLM: same field
+and parameter names), builds the fused device weights once, and binds new_state / prefill / decode_step onto the
+instance exactly as the reference's patch_model does (fast_decode.py:341-364); the model's own forward is untouched.
+
+Only the int8 KV layout is implemented (kv_dtype="int8"); attention-only presets (uv-50m-alpha) only."""
+from __future__ import annotations
+
+import dataclasses
+import types
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from .. import _lib as L
+from ..engine.config import UVConfig
+from ..engine.model import KVState, UVEngine
+from ..engine.model import kv_bytes_per_seq as _kv_bytes
+from ..engine.weights import UVWeights
+
+
+def as_uvconfig(cfg) -> UVConfig:
+    """UVConfig from a UVConfig, a dict, a dataclass or any object carrying the reference's MathConfig field names."""
+    if isinstance(cfg, UVConfig):
+        return cfg
+    if isinstance(cfg, dict):
+        d = cfg
+    elif dataclasses.is_dataclass(cfg):
+        d = dataclasses.asdict(cfg)
+    else:
+        d = {k: getattr(cfg, k) for k in UVConfig.__dataclass_fields__ if hasattr(cfg, k)}
+    for name in ("mudd", "bigram_rows", "conv_layers"):
+        if d.get(name):
+            raise L.UvmiError(f"this engine covers the attention-only presets; cfg.{name} is set")
+    if d.get("local_mixer", "attn") != "attn":
+        raise L.UvmiError(f"this engine covers the attention-only presets; cfg.local_mixer is {d['local_mixer']!r}")
+    return UVConfig(**{k: v for k, v in d.items() if k in UVConfig.__dataclass_fields__})
+
+
+class KernelDecodeState(KVState):
+    """KernelDecodeState(cfg, B, max_len, dtype, device, kv_dtype) of the reference (fast_decode.py:21-57): per-layer
+    k / v (B, K, S, hd) int8 and k_scale / v_scale (B, K, S) fp16, S = max_len on global layers (rounded up to a
+    multiple of 32 here) and min(window, max_len) on local ones, plus pos / starts / host_pos."""
+
+    def __init__(self, cfg, B: int, max_len: int, dtype=torch.float16, device="cuda", kv_dtype: str = "int8"):
+        if kv_dtype != "int8":
+            raise L.UvmiError(f"kv_dtype {kv_dtype!r}: only the int8 KV layout is implemented")
+        super().__init__(as_uvconfig(cfg), B, max_len, device)
+        self.dtype, self.kv_dtype = dtype, kv_dtype
+        self.local_len = min(self.cfg.window, self.max_len)
+        self.host_pos = np.zeros(B, dtype=np.int64)
+
+
+def kv_bytes_per_seq(cfg, ctx: int, kv_dtype: str = "int8") -> int:
+    assert kv_dtype == "int8"
+    return _kv_bytes(as_uvconfig(cfg), ctx)
+
+
+def _engine(model) -> UVEngine:
+    eng = model.__dict__.get("_uvmi_engine")
+    if eng is None:
+        raise L.UvmiError("model has not been patched: call patch_model(model) first")
+    return eng
+
+
+@torch.no_grad()
+def prefill_fast(self, idx: Tensor, starts: Tensor, st: KVState, rows: Tensor | None = None) -> Tensor:
+    """idx (n, T) left-padded prompts, starts (n,) first real column of each; writes the int8 caches of `rows` (all
+    rows when None), sets st.pos = T and st.starts = starts, returns the softcapped fp32 logits of the last position
+    (fast_decode.py:70-115).  Runs packed: pad columns are never computed."""
+    eng = _engine(self)
+    n, T = idx.shape
+    assert T <= st.max_len
+    if rows is None:
+        assert n == st.B
+        rows_l = list(range(n))
+    else:
+        rows_l = [int(r) for r in rows.tolist()]
+    idx_h, st_h = idx.cpu().numpy(), starts.cpu().numpy()
+    prompts = [idx_h[b, int(st_h[b]):].tolist() for b in range(n)]
+    assert max(len(p) for p in prompts) == T, "the longest prompt must fill all T columns (left padding)"
+    h = eng.prefill(prompts, rows_l, st, left_pad=True)
+    if hasattr(st, "host_pos"):
+        st.host_pos[np.asarray(rows_l)] = T
+    return eng.logits(h)
+
+
+@torch.no_grad()
+def decode_step_fast(self, tok: Tensor, st: KVState, g_len: int = 0, skip_attn: bool = False, num_splits: dict | None = None,
+                     backend: str = "auto", return_hidden: bool = False) -> Tensor:
+    """One token for all rows at st.pos, then st.pos += 1 (fast_decode.py:272-334).  g_len is accepted and ignored: the
+    kernels take every row's valid range from st.pos / st.starts.  Returns the logits, or the final normed hidden with
+    return_hidden (the caller then runs the head GEMM and the fused sampler)."""
+    assert not skip_attn, "skip_attn is a profiling switch of the reference and is not supported"
+    assert backend in ("auto", "hip"), f"backend {backend!r}: this library has one backend"
+    eng = _engine(self)
+    h = eng.decode_step(tok, st, num_splits)
+    if hasattr(st, "host_pos"):
+        st.host_pos += 1
+    return h if return_hidden else eng.logits(h)
+
+
+def patch_model(model, kv_dtype: str = "int8", num_splits: dict | None = None, backend: str = "auto",
+                dtype: torch.dtype = torch.bfloat16, max_tokens: int = 16384, device=None):
+    """Bind the kernel decode path onto `model` (instance attributes only).  model.cfg and model.state_dict() must use
+    the reference's names.  dtype: activation / weight dtype of the engine; max_tokens: largest number of token rows of
+    one call (decode rows or packed prefill tokens)."""
+    if kv_dtype != "int8":
+        raise L.UvmiError(f"kv_dtype {kv_dtype!r}: only the int8 KV layout is implemented")
+    cfg = as_uvconfig(model.cfg)
+    sd = model.state_dict()
+    dev = device or next(iter(sd.values())).device
+    if torch.device(dev).type != "cuda":
+        raise L.UvmiError("patch_model needs the model on a GPU (there is no CPU path)")
+    eng = UVEngine(UVWeights(cfg, sd, dtype, dev), max_tokens)
+
+    def new_state(self, batch, max_len, dtype=torch.float16, device=None):
+        return KernelDecodeState(cfg, batch, max_len, dtype, device or dev, kv_dtype)
+
+    def decode_step(self, tok, st, g_len=0, skip_attn=False):
+        return decode_step_fast(self, tok, st, g_len, skip_attn, num_splits, backend)
+
+    model.__dict__["_uvmi_engine"] = eng
+    model.__dict__["new_state"] = types.MethodType(new_state, model)
+    model.__dict__["prefill"] = types.MethodType(prefill_fast, model)
+    model.__dict__["decode_step"] = types.MethodType(decode_step, model)
+    return model
+
+
+def unpatch_model(model):
+    for n in ("new_state", "prefill", "decode_step", "_uvmi_engine"):
+        model.__dict__.pop(n, None)
+    return model
+
+
+@torch.no_grad()
+def sync_patched_weights(model) -> None:
+    """After model's parameters changed: refresh the engine's fused tensors in place from model.state_dict()."""
+    _engine(model).w.load_(model.state_dict())
