@@ -695,7 +695,7 @@ static bool mfma_ok(const uvmi_attn_args* a) {
   if (!(a->scale > 0.f)) return false;  // the running maximum is tracked before the (positive) softmax scale
   if (a->ring && (a->S % 32 != 0)) return false;
   if (a->sks > (1 << 20) || a->svs > (1 << 20) || a->sks < 0 || a->svs < 0) return false;  // 32-bit tile offsets
-  if (a->S % 4 != 0 || a->S < 4) return false;
+  if (a->S % 4 != 0 || a->S < 32) return false;  // 8-byte scale loads; a whole 32-key tile at slot 0 must exist
   auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
   if (!al(a->q, 16) || a->sqb % 8 || a->sqh % 8) return false;
   if (!al(a->k_cache, 16) || a->skb % 16 || a->skh % 16 || a->sks % 16) return false;

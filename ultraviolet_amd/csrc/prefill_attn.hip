@@ -16,10 +16,10 @@
 //   * V^T operands come from 8-byte loads (lane = dims 4m..4m+3 of 8 keys) regrouped with v_perm_b32 into four
 //     operands whose row m is head dim 4m + t; they are built once per super-tile and shared by the wave's 4 heads,
 //     as are the K operands (16-byte loads, lane = key m, dims 8g..8g+7 of each half);
-//   * loads are raw buffer loads (wave-uniform descriptor + lane-invariant offset + scalar tile offset); rows past N
-//     read as zero through the descriptor's bound.  The next super-tile is requested before the current one is used;
-//   * online softmax per (row, head) in the exp2 domain, rescaling only when some row's maximum grew; tiles that
-//     every row of the block sees completely skip the mask arithmetic;
+//   * loads are raw buffer loads with per-lane row offsets clamped to the last row; the next super-tile is requested
+//     before the current one is used;
+//   * online softmax per (row, head) in the exp2 domain; tiles that every row of the block sees completely skip the
+//     mask arithmetic (one branch per tile, so the four heads of a tile form one block the scheduler interleaves);
 //   * the 4 waves of a workgroup are independent (2 query blocks x 2 head groups), so K/V of a block are fetched
 //     from L2 once per pair of waves; workgroup ids are remapped so that each XCD (one L2 each) owns a contiguous
 //     range of query blocks and therefore whole sequences.
@@ -29,6 +29,7 @@
 #include "common.h"
 
 #include <climits>
+#include <type_traits>
 
 namespace uvmi {
 
@@ -167,31 +168,32 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
     lrun[hh] = 0.f;
   }
 
-  // ---- addressing: one descriptor per stream, lane-invariant byte offsets, scalar tile offsets
+  // ---- addressing: one descriptor per stream, per-lane byte offsets
   const uint16_t* kbase = (const uint16_t*)P.k + (int64_t)kvh * P.skh;
   const uint16_t* vbase = (const uint16_t*)P.v + (int64_t)kvh * P.svh;
   const uint32_t skn2 = (uint32_t)P.skn * 2, svn2 = (uint32_t)P.svn * 2;  // row strides in bytes
-  const uint32_t uskn2 = __builtin_amdgcn_readfirstlane(skn2), usvn2 = __builtin_amdgcn_readfirstlane(svn2);
   const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)((uint32_t)(P.N - 1) * skn2 + 128), 0x00020000);
   const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (int)((uint32_t)(P.N - 1) * svn2 + 128), 0x00020000);
-  const uint32_t koA = m * skn2 + 16 * g, koB = koA + 16 * skn2;
-  const uint32_t voA = 4 * g * svn2 + 8 * m;
 
+  // Rows are addressed per lane and clamped to N - 1 (the scalar offset of a buffer load is not part of its bounds
+  // check, so a tile reaching past row N must not rely on the descriptor); clamped rows are masked keys.
   auto load_tile = [&](int tb_in, PTile& T) {
     const int tb = __builtin_amdgcn_readfirstlane(tb_in);
-    const uint32_t ok = (uint32_t)tb * uskn2, ov = (uint32_t)tb * usvn2;
-    T.k[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koA, ok, 0);
-    T.k[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koA + 64, ok, 0);
-    T.k[2] = __builtin_amdgcn_raw_buffer_load_b128(rK, koB, ok, 0);
-    T.k[3] = __builtin_amdgcn_raw_buffer_load_b128(rK, koB + 64, ok, 0);
+    const int last = P.N - 1;
+    const uint32_t ka = (uint32_t)min(tb + m, last) * skn2 + 16 * g, kb = (uint32_t)min(tb + 16 + m, last) * skn2 + 16 * g;
+    T.k[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, ka, 0, 0);
+    T.k[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, ka + 64, 0, 0);
+    T.k[2] = __builtin_amdgcn_raw_buffer_load_b128(rK, kb, 0, 0);
+    T.k[3] = __builtin_amdgcn_raw_buffer_load_b128(rK, kb + 64, 0, 0);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      T.v[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + j * usvn2, 0);
-      T.v[4 + j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + (16 + j) * usvn2, 0);
+      T.v[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, (uint32_t)min(tb + 4 * g + j, last) * svn2 + 8 * m, 0, 0);
+      T.v[4 + j] = __builtin_amdgcn_raw_buffer_load_b64(rV, (uint32_t)min(tb + 16 + 4 * g + j, last) * svn2 + 8 * m, 0, 0);
     }
   };
 
-  auto step = [&](const PTile& T, int tb, bool edge) {
+  auto step_t = [&](const PTile& T, int tb, auto EDGE) {
+    constexpr bool edge = decltype(EDGE)::value;
     // V^T operands: operand t, row m is head dim 4m + t; dword p of an operand holds contraction slots 2p, 2p+1
     pu4 VA[4];
     {
@@ -222,7 +224,9 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
       }
       float mx = fmaxf(fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3])), fmaxf(fmaxf(t[4], t[5]), fmaxf(t[6], t[7])));
       mx = pmax32(pmax16(mx));
-      if (__builtin_amdgcn_ballot_w64(mx > mrun[hh]) != 0) {  // some row's maximum grew: rescale (alpha = 1 elsewhere)
+      {  // rescale by alpha = exp2((m_old - m_new) c), 1 where the row's maximum did not grow.  Unconditional: a branch
+         // here would split the four heads into separate blocks and stop the scheduler from overlapping one head's
+         // softmax arithmetic with the next head's MFMAs
         const float mnew = fmaxf(mrun[hh], mx);
         const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((mrun[hh] - mnew) * c);
 #pragma unroll
@@ -239,6 +243,12 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
 #pragma unroll
       for (int tt = 0; tt < 4; tt++) O[hh][tt] = mfma16<DT>(VA[tt], PB, O[hh][tt]);
     }
+  };
+
+  // the mask test is hoisted out of the head loop (one branch per tile, two straight-line bodies), so that the four
+  // heads of a tile form one block the scheduler can interleave
+  auto step = [&](const PTile& T, int tb, bool edge) {
+    if (edge) step_t(T, tb, std::true_type{}); else step_t(T, tb, std::false_type{});
   };
 
   {
