@@ -343,14 +343,14 @@ def bench_c3(args):
     from ultraviolet_amd.engine.rollout import Rollout
     dev = "cuda:0"
     cfg = make_config("uv-50m-alpha")
-    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02), max_tokens=4096)
+    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02), max_tokens=2048)
     rng = np.random.default_rng(0)
     gen = torch.Generator(device=dev).manual_seed(0)
     B = 512
     K = args.steps if args.steps > 0 else 256
     W = args.warmup
     g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + K + W + 64, temperature=1.0, seed=0, eos_id=None, check_every=4, bucket=128,
-                retire_p=0.01, mixed=True)
+                retire_p=0.01, mixed=True, admit_cap=24)
     # running slots with materialised contexts: request ids 0..B-1, one token generated so far
     rows = torch.arange(B, device=dev)
     _fill_cache(g.st, rows, torch.from_numpy(rng.integers(128, 2049, size=B)).to(dev), gen)

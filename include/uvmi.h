@@ -269,6 +269,15 @@ int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const int64_t* ac
 int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, const int64_t* req_ids,
                      const int64_t* limits, const int64_t* first_tok, const float* first_lp, void* stream);
 
+/* Per-token tables of the prompts admitted with a step, built on the device from their cu_seqlens (n_adm + 1 entries,
+ * non-decreasing; unused trailing entries repeat the total): for packed token i of prompt a, pos_t = adm_start[a] + i -
+ * cu[a], row_t = adm_slot[a], last_t = last position of the prompt; tokens at or after cu[n_adm], and prompts with
+ * adm_slot < 0, are padding (row -1).  last_idx[a] = packed index of prompt a's last token (0 if unused).  Also sets
+ * starts / pos of the admitted slots.  Replaces the host-built index tensors of prefill_packed_host
+ * (ultraviolet/kernels/fast_decode.py:210-269) so that a step that admits prompts can be captured in a graph. */
+int uvmi_sched_expand(const uvmi_sched_state* s, int n_adm, int n_tokens, const int64_t* cu_seqlens, const int64_t* adm_slot,
+                      const int64_t* adm_start, int64_t* pos_t, int64_t* row_t, int64_t* last_t, int64_t* last_idx, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

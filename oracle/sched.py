@@ -69,3 +69,29 @@ class SlotTable:
                 fin = float(philox.request_uniform(seed, int(self.req[s]), c, philox.DOMAIN_RETIRE)) < np.float32(retire_p)
             if fin:
                 self._finish(s, self.req[s], c + 1)
+
+
+def expand_prompts(cu, slots, starts, n_tokens: int):
+    """Per-token tables of a packed prefill, as the reference builds them on the host (prefill_packed_host,
+    ultraviolet/kernels/fast_decode.py:210-269): for packed token i of prompt a (cu[a] <= i < cu[a+1]) its position
+    starts[a] + i - cu[a], its cache row slots[a] and the last position of its prompt starts[a] + len[a] - 1; tokens at or
+    after cu[-1] are padding (row -1, position 0).  Also the packed index of every prompt's last token (0 for an empty or
+    unused entry, slot < 0) and the (start, end) positions of every admitted slot.  Plain loops."""
+    cu = [int(c) for c in cu]
+    A = len(cu) - 1
+    pos = np.zeros(n_tokens, np.int64)
+    row = np.full(n_tokens, -1, np.int64)
+    last = np.zeros(n_tokens, np.int64)
+    last_idx = np.zeros(A, np.int64)
+    bind = {}
+    for a in range(A):
+        n = cu[a + 1] - cu[a]
+        if n <= 0 or slots[a] < 0:
+            continue
+        for i in range(cu[a], min(cu[a + 1], n_tokens)):
+            pos[i] = starts[a] + i - cu[a]
+            row[i] = slots[a]
+            last[i] = starts[a] + n - 1
+        last_idx[a] = cu[a + 1] - 1
+        bind[int(slots[a])] = (int(starts[a]), int(starts[a] + n))
+    return pos, row, last, last_idx, bind

@@ -205,3 +205,54 @@ def test_sync_weights_inplace_keeps_graphs_and_bumps_version():
     p3["blocks.0.resid_attn"] = np.float32(0.9)
     g.sync_weights_inplace(p3)
     assert g.version == 2 and len(g.graphs) == 0                 # a launch-argument scalar changed: recapture
+
+
+def test_prompt_table_expansion_bit_exact():
+    """uvmi_sched_expand against the oracle's loops: positions, cache rows, last positions, last-token indices and the
+    slots' starts / pos, with empty prompts, unused entries (slot -1) and padding tokens."""
+    from oracle.sched import expand_prompts
+    from ultraviolet_amd import _lib as L
+    lib = L.lib()
+    rng = np.random.default_rng(3)
+    for A, Np, B in ((4, 64, 8), (16, 512, 40), (1, 16, 2), (7, 100, 9)):
+        t, s = _dev_table(B, 4, -1)
+        for _ in range(4):
+            na = int(rng.integers(0, A + 1))
+            lens = rng.integers(0, max(2, Np // max(A, 1)), size=A)
+            lens[na:] = 0
+            cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+            slots = np.full(A, -1, np.int64)
+            slots[:na] = rng.choice(B, size=na, replace=False)
+            if na > 1 and rng.random() < 0.5:
+                slots[rng.integers(0, na)] = -1                      # an entry the host withdrew
+            starts = rng.integers(0, 20, size=A).astype(np.int64)
+            tt = lambda a: torch.as_tensor(a, dtype=torch.long, device=DEV)
+            cu_d, sl_d, st_d = tt(cu), tt(slots), tt(starts)
+            pos_t, row_t, last_t, lidx = (torch.full((n,), 77, dtype=torch.long, device=DEV) for n in (Np, Np, Np, A))
+            p0, s0 = t["pos"].cpu().numpy().copy(), t["starts"].cpu().numpy().copy()
+            L.check(lib.uvmi_sched_expand(C.byref(s), A, Np, cu_d.data_ptr(), sl_d.data_ptr(), st_d.data_ptr(), pos_t.data_ptr(),
+                                          row_t.data_ptr(), last_t.data_ptr(), lidx.data_ptr(), None), "expand")
+            pos, row, last, last_idx, bind = expand_prompts(cu, slots, starts, Np)
+            assert np.array_equal(pos_t.cpu().numpy(), pos) and np.array_equal(row_t.cpu().numpy(), row)
+            assert np.array_equal(last_t.cpu().numpy(), last) and np.array_equal(lidx.cpu().numpy(), last_idx)
+            for sl, (a, b) in bind.items():
+                p0[sl], s0[sl] = b, a
+            assert np.array_equal(t["pos"].cpu().numpy(), p0) and np.array_equal(t["starts"].cpu().numpy(), s0)
+
+
+def test_rollout_mixed_graph_equals_eager_mixed():
+    """The captured mixed step (device-built prompt tables) gives exactly the streams of the same step launched eagerly."""
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg, eng = _engine(torch.float32, window=32)
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(2, cfg.vocab_size, size=int(rng.integers(3, 30))).tolist() for _ in range(30)]
+    outs = []
+    for graph in (False, True):
+        g = Rollout(eng, slots=6, max_prompt=32, max_new=16, temperature=1.0, seed=4, check_every=3, bucket=4, mixed=True,
+                    admit_cap=3, use_graph=graph, retire_p=0.05)
+        for i, p in enumerate(prompts):
+            g.add(p, i)
+        outs.append({m: (row, lp.tolist()) for m, row, lp, _ in g.run(max_chunks=1000)})
+        assert sorted(outs[-1]) == list(range(30)) and g.n_mixed_steps > 0
+        assert (len(g.mixed_graphs) > 0) == graph
+    assert outs[0] == outs[1]

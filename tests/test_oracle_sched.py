@@ -61,3 +61,26 @@ def test_bucket_smaller_than_active_and_retire_probability():
     tab2.commit(slot, [5] * 512, np.zeros(512, np.float32), retire_p=0.25, seed=7)
     frac = len(tab2.done) / 512
     assert 0.17 < frac < 0.33
+
+
+def test_expand_prompts_matches_vectorised_construction():
+    """The loop restatement against an independent vectorised construction (np.repeat of per-prompt values, the way the
+    reference's prefill_packed_host forms its index tensors, fast_decode.py:219-236) on random ragged prompt sets."""
+    import numpy as np
+    from oracle.sched import expand_prompts
+    rng = np.random.default_rng(0)
+    for _ in range(50):
+        A = int(rng.integers(1, 9))
+        lens = rng.integers(1, 30, size=A)
+        cu = np.concatenate([[0], np.cumsum(lens)])
+        slots = rng.permutation(20)[:A]
+        starts = rng.integers(0, 10, size=A)
+        n_tok = int(cu[-1]) + int(rng.integers(0, 8))
+        pos, row, last, last_idx, bind = expand_prompts(cu, slots, starts, n_tok)
+        seg = np.repeat(np.arange(A), lens)
+        N = int(cu[-1])
+        assert np.array_equal(pos[:N], np.arange(N) - cu[:-1][seg] + starts[seg])
+        assert np.array_equal(row[:N], slots[seg]) and np.array_equal(last[:N], (starts + lens - 1)[seg])
+        assert (row[N:] == -1).all() and (pos[N:] == 0).all()
+        assert np.array_equal(last_idx, cu[1:] - 1)
+        assert bind == {int(s): (int(a), int(a + n)) for s, a, n in zip(slots, starts, lens)}

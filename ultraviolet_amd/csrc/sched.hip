@@ -1,7 +1,8 @@
 // On-device continuous-batching bookkeeping: the slot table of the reference's host loop
 // (generate_continuous, ultraviolet/model.py:1283-1350; StreamGen, scripts/rl_stream.py:55-146) kept in HBM and
-// advanced by two tiny kernels per decode step, so a step needs no host synchronisation:
+// advanced by a few tiny kernels per decode step, so a step needs no host synchronisation:
 //
+//   sched_expand   per-token position / cache-row tables of the prompts admitted with a step, from their cu_seqlens;
 //   sched_compact  scan the slot table, list the active slots first (ascending), gather their token / position /
 //                  request id / token index into dense arrays of a fixed bucket length (padding rows get slot -1);
 //   sched_commit   scatter the sampled token and its log-prob into the slot's output row, advance count and position,
@@ -129,6 +130,37 @@ __global__ __launch_bounds__(256) void sched_admit_kernel(uvmi_sched_state S, in
   }
 }
 
+// Per-token tables of a packed prefill built on the device from its cu_seqlens (the reference builds them on the host
+// for every refill: prefill_packed_host, ultraviolet/kernels/fast_decode.py:210-269).  One thread per packed token:
+// binary search of its prompt, then position / cache row / last position; tokens past cu[n_adm] are padding (row -1).
+// The first n_adm threads also record the packed index of their prompt's last token and point the slot at its prompt
+// (starts = first position, pos = next position to write).
+__global__ __launch_bounds__(256) void sched_expand_kernel(uvmi_sched_state S, int n_adm, int n_tokens, const int64_t* cu,
+                                                           const int64_t* adm_slot, const int64_t* adm_start, int64_t* pos_t,
+                                                           int64_t* row_t, int64_t* last_t, int64_t* last_idx) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n_adm) {
+    const int64_t n = cu[i + 1] - cu[i], slot = adm_slot[i];
+    const bool ok = n > 0 && slot >= 0 && slot < S.B;
+    last_idx[i] = ok ? cu[i + 1] - 1 : 0;
+    if (ok) {
+      S.starts[slot] = adm_start[i];
+      S.pos[slot] = adm_start[i] + n;
+    }
+  }
+  if (i >= n_tokens) return;
+  int lo = 0, hi = n_adm;  // invariant: cu[lo] <= i, and hi == n_adm or cu[hi] > i
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= i) lo = mid; else hi = mid;
+  }
+  const int64_t slot = adm_slot[lo];
+  const bool real = i < cu[n_adm] && i < cu[lo + 1] && slot >= 0 && slot < S.B;
+  pos_t[i] = real ? adm_start[lo] + (i - cu[lo]) : 0;
+  row_t[i] = real ? slot : -1;
+  last_t[i] = real ? adm_start[lo] + (cu[lo + 1] - cu[lo]) - 1 : 0;
+}
+
 static int check_state(const uvmi_sched_state* s, const char* who) {
   UVMI_REQUIRE(s, UVMI_EINVAL, "%s: null state", who);
   UVMI_REQUIRE(s->slot_req && s->slot_cnt && s->slot_limit && s->slot_tok && s->pos && s->starts && s->out_tok && s->counters &&
@@ -170,5 +202,18 @@ extern "C" int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t*
   if (n == 0) return UVMI_OK;
   hipLaunchKernelGGL(sched_admit_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n, slots, req_ids, limits, first_tok, first_lp);
   UVMI_CHECK_LAUNCH("uvmi_sched_admit");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_expand(const uvmi_sched_state* s, int n_adm, int n_tokens, const int64_t* cu_seqlens, const int64_t* adm_slot,
+                                 const int64_t* adm_start, int64_t* pos_t, int64_t* row_t, int64_t* last_t, int64_t* last_idx, void* stream) {
+  int rc = check_state(s, "uvmi_sched_expand");
+  if (rc) return rc;
+  UVMI_REQUIRE(n_adm > 0 && n_tokens >= 0 && cu_seqlens && adm_slot && adm_start && pos_t && row_t && last_t && last_idx, UVMI_EINVAL,
+               "uvmi_sched_expand: bad arguments");
+  const int n = n_tokens > n_adm ? n_tokens : n_adm;
+  hipLaunchKernelGGL(sched_expand_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_adm, n_tokens, cu_seqlens, adm_slot,
+                     adm_start, pos_t, row_t, last_t, last_idx);
+  UVMI_CHECK_LAUNCH("uvmi_sched_expand");
   return UVMI_OK;
 }

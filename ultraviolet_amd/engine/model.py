@@ -262,25 +262,33 @@ class UVEngine:
         runs these as two passes (its refill prefill, then the decode step: model.py:1296-1313, 1321-1330).
         Returns the final normed hidden of each prompt's last token and of each decode row.  Does not advance st.pos of
         the decode rows (the caller's slot table does), but binds the prompts' rows."""
-        cfg, b = self.cfg, self.buf
         Np, nd = pk["N"], tok_d.numel()
-        N = Np + nd
-        assert N <= self.max_tokens, f"{N} token rows exceed the engine's max_tokens {self.max_tokens}"
         tok, pos = torch.cat([pk["tok"], tok_d]), torch.cat([pk["pos"], pos_d])
         rows, last = torch.cat([pk["row"], rows_d]), torch.cat([pk["last"], pos_d])
+        h = self.mixed_trunk(tok, pos, rows, last, Np, nd, pk["cu"], starts_d, st)
+        self.bind_prompts(pk, st)
+        return h.index_select(0, pk["last_idx"]), h[Np:Np + nd]
+
+    def mixed_trunk(self, tok: Tensor, pos: Tensor, rows: Tensor, last: Tensor, Np: int, nd: int, cu: Tensor, starts_d: Tensor,
+                    st: KVState) -> Tensor:
+        """The pass of mixed_step over already concatenated per-token arrays (Np packed prompt tokens, then nd decode rows;
+        cu: the prompts' cu_seqlens on the device).  Allocation-free apart from the packed attention output, so a caller
+        that builds the arrays on the device can capture it in a graph.  Returns the final normed hidden (Np + nd, d)."""
+        cfg, b = self.cfg, self.buf
+        N = Np + nd
+        assert N <= self.max_tokens, f"{N} token rows exceed the engine's max_tokens {self.max_tokens}"
+        pos_d, rows_d = pos[Np:N], rows[Np:N]
 
         def attn(l, q):
             w = 0 if cfg.is_global(l) else cfg.window
-            zp = packed_attention(q[:Np], b["k"][:Np], b["v"][:Np], pk["cu"], cfg.attn_scale, w, workspace=self.pf_ws)
+            zp = packed_attention(q[:Np], b["k"][:Np], b["v"][:Np], cu, cfg.attn_scale, w, workspace=self.pf_ws)
             self._attn_post(l, zp, Np)
             zd = self.cache_attention(l, q[Np:N], st, pos_d, starts_d, nd, rows=rows_d, off=Np)
             if zd is not None:
                 self._attn_post(l, zd, nd, off=Np)
             return None
 
-        h = self._trunk(tok, pos, N, attn, rows=rows, last_pos=last, st=st)
-        self.bind_prompts(pk, st)
-        return h.index_select(0, pk["last_idx"]), h[Np:N]
+        return self._trunk(tok[:N], pos[:N], N, attn, rows=rows[:N], last_pos=last[:N], st=st)
 
     @torch.no_grad()
     def prefill(self, prompts: list[list[int]], rows: list[int], st: KVState, left_pad: bool = True) -> Tensor:

@@ -28,7 +28,8 @@ from .model import KVState, UVEngine
 class Rollout:
     def __init__(self, engine: UVEngine, slots: int, max_prompt: int, max_new: int, temperature: float = 1.0,
                  seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
-                 use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False):
+                 use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False,
+                 admit_cap: int = 16):
         self.e, self.cfg = engine, engine.cfg
         self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
         self.T, self.seed, self.eos = float(temperature), int(seed), eos_id
@@ -55,10 +56,34 @@ class Rollout:
         s.done_req, s.done_slot, s.done_cnt, s.counters = (t.data_ptr() for t in (self.done_req, self.done_slot, self.done_cnt, self.counters))
         s.max_new, s.eos_id, s.B, s.done_cap = max_new, -1 if eos_id is None else int(eos_id), slots, self.done_cap
         self.sched = s
-        # dense per-step arrays (bucket length <= slots)
-        self.act, self.tok_c, self.pos_c, self.starts_c, self.req_c, self.cnt_c = (z(slots) for _ in range(6))
+        # Per-token arrays of a step: Np packed tokens of the prompts admitted with the step (mixed batches only), then
+        # the decode rows of the bucket (bucket length <= slots).  The decode views are what the compaction kernel fills.
+        self.A = int(admit_cap) if mixed else 0                     # prompts one mixed step can admit
+        self.Np = (self.A * max_prompt + 15) // 16 * 16             # packed prompt tokens of a mixed step
+        A, Np = self.A, self.Np
+        assert not mixed or Np + slots <= engine.max_tokens, "engine.max_tokens too small for admit_cap * max_prompt + slots"
+        self.tok_all, self.pos_all, self.row_all, self.last_all = (z(Np + slots) for _ in range(4))
+        self.req_all, self.cnt_all = z(A + slots), z(A + slots)
+        self.act, self.tok_c, self.pos_c = self.row_all[Np:], self.tok_all[Np:], self.pos_all[Np:]
+        self.req_c, self.cnt_c = self.req_all[A:], self.cnt_all[A:]
+        self.starts_c = z(slots)
         self.new_tok, self.new_lp = z(slots), z(slots, dt=torch.float32)
+        if mixed:
+            # admission staging, one host -> device copy per mixed step: [tokens Np | cu A+1 | slot A | start A | limit A | req A]
+            self.stage_n = Np + (A + 1) + 3 * A
+            self.stage_h = torch.zeros(self.stage_n + A, dtype=torch.long, pin_memory=True)
+            self.stage_d = z(self.stage_n)
+            o = Np
+            self.adm_cu, o = self.stage_d[o:o + A + 1], o + A + 1
+            self.adm_slot, o = self.stage_d[o:o + A], o + A
+            self.adm_start, o = self.stage_d[o:o + A], o + A
+            self.adm_limit, o = self.stage_d[o:o + A], o + A
+            self.gather_idx = torch.cat([z(A), Np + torch.arange(slots, device=dev)])   # rows of the hidden that get sampled
+            self.adm_tok, self.adm_lp = z(A), z(A, dt=torch.float32)
+            self.adm_slot.fill_(-1)
+            self._stage_ev = torch.cuda.Event()
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        self.mixed_graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.queue = collections.deque()
         self.meta: dict[int, tuple] = {}          # request id -> (meta, start_version)
         self.free = list(range(slots))[::-1]
@@ -94,6 +119,7 @@ class Rollout:
         from now on carry the new version as their start_version."""
         if self.e.w.load_(params):
             self.graphs.clear()
+            self.mixed_graphs.clear()
         torch.cuda.synchronize(self.dev)
         self.version += 1
 
@@ -136,44 +162,80 @@ class Rollout:
 
     @torch.no_grad()
     def _admit_mixed(self) -> bool:
-        """Admission fused with a decode step: queued prompts (FIFO, as many as fit the engine's token rows next to the
-        decode bucket) are prefilled in the same forward pass that decodes the active slots; one head GEMM and one
-        sampler launch cover the prompts' first tokens and the decode rows.  Returns False when nothing fits."""
-        e, lib = self.e, L.lib()
+        """Admission fused with a decode step: queued prompts (FIFO; at most admit_cap prompts and Np tokens) are prefilled
+        in the same forward pass that decodes the active slots; one head GEMM and one sampler launch cover the prompts'
+        first tokens and the decode rows.  The host only chooses the slots and uploads the packed prompt tokens with their
+        cu_seqlens (one copy); positions, cache rows and the slot table entries are built on the device, so the whole
+        step is one graph replay.  Returns False when nothing fits."""
         n = self.bucket_for(self.n_active_host)
+        A, Np = self.A, self.Np
         batch, ntok = [], 0
-        while self.queue and len(batch) < len(self.free) and ntok + len(self.queue[0][0]) <= e.max_tokens - n:
+        while self.queue and len(batch) < min(len(self.free), A) and ntok + len(self.queue[0][0]) <= Np:
             it = self.queue.popleft()
             batch.append(it)
             ntok += len(it[0])
         if not batch:
             return False
-        A = len(batch)
+        na = len(batch)
         slots = [self.free.pop() for _ in batch]
-        reqs = list(range(self.next_req, self.next_req + A))
-        self.next_req += A
-        tt = lambda a: torch.as_tensor(a, dtype=torch.long, device=self.dev)
-        slot_t, req_t, lim_t = tt(slots), tt(reqs), tt([b[2] for b in batch])
-        pk = e.pack_prompts([b[0] for b in batch], slots, self.st.max_len, self.left_pad)
-        sp = L.stream_ptr(self.act)
-        L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
-                                       self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
-        hp, hd = e.mixed_step(pk, self.tok_c[:n], self.pos_c[:n], self.starts_c[:n], self.act[:n], self.st)
-        x = e.head(torch.cat([hp, hd]))
-        tok, lp = self._sample(x, torch.cat([req_t, self.req_c[:n]]), torch.cat([torch.zeros_like(req_t), self.cnt_c[:n]]))
-        self.new_tok[:n].copy_(tok[A:])
-        self.new_lp[:n].copy_(lp[A:])
-        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
-                                      self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
-        tok_a, lp_a = tok[:A].contiguous(), lp[:A].contiguous()   # named: they must outlive the launch call
-        L.check(lib.uvmi_sched_admit(C.byref(self.sched), A, slot_t.data_ptr(), req_t.data_ptr(), lim_t.data_ptr(), tok_a.data_ptr(),
-                                     lp_a.data_ptr(), sp), "uvmi_sched_admit")
+        reqs = list(range(self.next_req, self.next_req + na))
+        self.next_req += na
+        lens = np.fromiter((len(b[0]) for b in batch), dtype=np.int64, count=na)
+        starts = (int(lens.max()) - lens) if self.left_pad else np.zeros(na, np.int64)
+        self._stage_ev.synchronize()                        # the previous upload has left the pinned buffer
+        h = self.stage_h.numpy()
+        h[:] = 0
+        h[:ntok] = np.fromiter((t for b in batch for t in b[0]), dtype=np.int64, count=ntok)
+        o = Np
+        h[o] = 0
+        h[o + 1:o + 1 + na] = np.cumsum(lens)
+        h[o + 1 + na:o + 1 + A] = ntok
+        o += A + 1
+        h[o:o + A] = -1
+        h[o:o + na] = slots
+        o += A
+        h[o:o + na] = starts
+        o += A
+        h[o:o + na] = [b[2] for b in batch]
+        o += A
+        h[o:o + na] = reqs                                  # request ids ride behind the staged block
+        self.stage_d.copy_(self.stage_h[:self.stage_n], non_blocking=True)
+        self.tok_all[:Np].copy_(self.stage_d[:Np])
+        self.req_all[:A].copy_(self.stage_h[self.stage_n:], non_blocking=True)
+        self._stage_ev.record()
+        if self.use_graph:
+            (self.mixed_graphs.get(n) or self._capture(n, mixed=True)).replay()
+        else:
+            self._mixed_body(n)
         for r, b in zip(reqs, batch):
             self.meta[r] = (b[1], self.version)
-        self.n_active_host += A
+        self.n_active_host += na
         self.n_decode_steps += 1
         self.n_mixed_steps += 1
         return True
+
+    def _mixed_body(self, n: int):
+        """compact -> prompt tables -> one trunk pass over Np prompt tokens + n decode rows -> head -> sampler -> commit
+        (decode rows) + admit (prompts).  Every launch has fixed shapes; what varies lives in device arrays."""
+        e, lib, A, Np = self.e, L.lib(), self.A, self.Np
+        sp = L.stream_ptr(self.act)
+        L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                       self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
+        L.check(lib.uvmi_sched_expand(C.byref(self.sched), A, Np, self.adm_cu.data_ptr(), self.adm_slot.data_ptr(), self.adm_start.data_ptr(),
+                                      self.pos_all.data_ptr(), self.row_all.data_ptr(), self.last_all.data_ptr(), self.gather_idx.data_ptr(),
+                                      sp), "uvmi_sched_expand")
+        self.last_all[Np:Np + n].copy_(self.pos_all[Np:Np + n])
+        h = e.mixed_trunk(self.tok_all, self.pos_all, self.row_all, self.last_all, Np, n, self.adm_cu, self.starts_c[:n], self.st)
+        x = e.head(h.index_select(0, self.gather_idx[:A + n]))
+        tok, lp = self._sample(x, self.req_all[:A + n], self.cnt_all[:A + n])
+        self.new_tok[:n].copy_(tok[A:])
+        self.new_lp[:n].copy_(lp[A:])
+        self.adm_tok.copy_(tok[:A])
+        self.adm_lp.copy_(lp[:A])
+        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
+                                      self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
+        L.check(lib.uvmi_sched_admit(C.byref(self.sched), A, self.adm_slot.data_ptr(), self.req_all.data_ptr(), self.adm_limit.data_ptr(),
+                                     self.adm_tok.data_ptr(), self.adm_lp.data_ptr(), sp), "uvmi_sched_admit")
 
     # ------------------------------------------------------------------------------------------------ decode
     def _step_body(self, n: int):
@@ -204,22 +266,24 @@ class Rollout:
     def bucket_for(self, n_active: int) -> int:
         return min(self.B, max(self.bucket, -(-n_active // self.bucket) * self.bucket))
 
-    def _capture(self, n: int):
-        """Capture the step for a bucket of n rows.  A captured step mutates the slot table, so the kernels and GEMM
-        shapes are first warmed up on the live state, which is then restored; capture itself executes nothing."""
+    def _capture(self, n: int, mixed: bool = False):
+        """Capture the step for a bucket of n rows (mixed: the step that also admits prompts).  A captured step mutates the
+        slot table, so the kernels and GEMM shapes are first warmed up on the live state, which is then restored; capture
+        itself executes nothing."""
+        body = self._mixed_body if mixed else self._step_body
         keep = [t.clone() for t in self._mutable()]
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
-            self._step_body(n)
+            body(n)
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         for t, k in zip(self._mutable(), keep):
             t.copy_(k)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            self._step_body(n)
-        self.graphs[n] = g
+            body(n)
+        (self.mixed_graphs if mixed else self.graphs)[n] = g
         return g
 
     @torch.no_grad()
@@ -230,6 +294,8 @@ class Rollout:
             for n in range(self.bucket, self.bucket_for(self.n_active_host) + 1, self.bucket):
                 if n not in self.graphs:
                     self._capture(min(n, self.B))
+                if self.mixed and self.queue and n not in self.mixed_graphs:
+                    self._capture(min(n, self.B), mixed=True)
 
     @torch.no_grad()
     def step(self):
