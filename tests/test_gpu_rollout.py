@@ -256,3 +256,47 @@ def test_rollout_mixed_graph_equals_eager_mixed():
         assert sorted(outs[-1]) == list(range(30)) and g.n_mixed_steps > 0
         assert (len(g.mixed_graphs) > 0) == graph
     assert outs[0] == outs[1]
+
+
+def test_full_size_rollout_properties():
+    """The 2048-sequence rollout configuration at its real shape (UV-50M bf16, 256 prompts x 8, prompts U{64..256}, seeded
+    T = 1 sampling), first 24 decode steps: size-independent properties instead of an oracle run - token accounting, valid
+    tokens and log-probs, positions = prompt length + tokens generated, and bit-identical streams when the whole rollout
+    is repeated (deterministic kernels, Philox keyed by request)."""
+    from ultraviolet_amd.engine import UVEngine, UVWeights, make_config
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg = make_config("uv-50m-alpha")
+    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=DEV, perturb=0.02), max_tokens=16384)
+    rng = np.random.default_rng(0)
+    prompts, limits = [], []
+    for _ in range(256):
+        p = rng.integers(1, cfg.vocab_size, size=int(rng.integers(64, 257))).tolist()
+        for _ in range(8):
+            prompts.append(p)
+            limits.append(int(min(rng.geometric(1.0 / 600.0), 2048)))
+    runs = []
+    for rep in range(2):
+        g = Rollout(eng, slots=2048, max_prompt=256, max_new=64, temperature=1.0, seed=0, check_every=8, bucket=128)
+        for i, (p, l) in enumerate(zip(prompts, limits)):
+            g.add(p, i, limit=min(l, 64))
+        done = []
+        for _ in range(3):
+            done += g.chunk()
+        torch.cuda.synchronize()
+        cnt, req, pos = g.slot_cnt.cpu().numpy(), g.slot_req.cpu().numpy(), g.st.pos.cpu().numpy()
+        out_tok, out_lp = g.out_tok.cpu().numpy(), g.out_lp.cpu().numpy()
+        live = req >= 0
+        assert g.n_decode_steps == 24
+        assert len(done) + int(live.sum()) == 2048                      # every request is either finished or in a slot
+        assert all(len(r[1]) == min(limits[r[0]], 64) for r in done)    # no EOS configured: finished rows are limit-long
+        assert (cnt[live] == 25).all()                                  # 1 token from the prefill + 24 steps
+        plen = np.array([len(prompts[r]) for r in req[live]])
+        assert np.array_equal(pos[live], plen + 24)                     # next write position (the last token is not yet appended)
+        rows = {int(r): out_tok[s, :25].tolist() for s, r in enumerate(req) if r >= 0}
+        rows.update({r[0]: r[1] for r in done})
+        lps = np.concatenate([out_lp[s, :25] for s in np.nonzero(live)[0]])
+        assert all(0 <= t < cfg.vocab_size for row in rows.values() for t in row)
+        assert np.isfinite(lps).all() and (lps <= 1e-6).all()
+        assert len({tuple(rows[8 * gidx + j]) for gidx in range(4) for j in range(8)}) > 8   # group members sample differently
+        runs.append(rows)
+    assert runs[0] == runs[1]
