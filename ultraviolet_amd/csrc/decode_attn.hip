@@ -149,6 +149,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   constexpr int IPB = 4 / WPR;  // items per block
   __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
   __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
+  __shared__ float sh_post[4][80];  // epilogue operands of the item whose first wave this is: v_hat[64], gate[8], xsa[8]
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wsub = wave % WPR;
@@ -172,6 +173,15 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   const uint32_t qmask = head < G ? 0xffffffffu : 0u;
   const uint16_t* qp = (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + (head < G ? head : G - 1)) * P.sqh + 16 * g;
   const uint4 qw0 = *(const uint4*)qp, qw1 = *(const uint4*)(qp + 8);
+  // Operands of the fused epilogue are requested now, with q, and parked in LDS once q has arrived, so that the
+  // epilogue at the end of the workgroup's life does not start with a round trip to memory.  Unconditional loads (from
+  // q when there is no epilogue) keep the control flow uniform.
+  const bool has_post = P.post_vhat != nullptr;
+  const int hsafe = h * G + (head < G ? head : G - 1);
+  const float* pv_src = has_post ? P.post_vhat + ((int64_t)b * P.KH + h) * 64 + lane : (const float*)P.q + lane;
+  const float* pg_src = has_post && P.post_gate ? P.post_gate + (int64_t)b * P.H + hsafe : (const float*)P.q;
+  const float* px_src = has_post && P.post_xsa ? P.post_xsa + hsafe : (const float*)P.q;
+  const float pv_val = *pv_src, pg_val = *pg_src, px_val = *px_src;
   const RowPlan rp = plan_row(P, b);
   const bool live = live_item && sid < rp.nsplit;
   if (WPR == 1 && !live) return;
@@ -352,6 +362,10 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
     load_tile(slot, TA);
     __builtin_amdgcn_sched_barrier(0);
     prep_q();
+    if (wsub == 0) {
+      sh_post[wave][lane] = pv_val;
+      if (lane < 16) sh_post[wave][64 + lane] = lane < 8 ? pg_val : px_val;  // lanes 8..15 carry head lane - 8 too
+    }
     if (has) {
       while (true) {
         slot = next_slot(slot, tb);
@@ -435,10 +449,13 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
         auto rnd = [&](float x, int dt) -> float {
           return dt == UVMI_F32 ? x : (dt == UVMI_BF16 ? bf16_to_float(float_to_bf16(x)) : (float)(half_t)x);
         };
-        const float4* vp = (const float4*)(P.post_vhat + ((int64_t)b * P.KH + h) * 64 + 16 * g);
-        const float4 v0 = vp[0], v1 = vp[1], v2 = vp[2], v3 = vp[3];
-        const float vv[16] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
-        const float gate = P.post_gate ? P.post_gate[(int64_t)b * P.H + h * G + head] : 1.0f;
+        float vv[16];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const float4 x = *(const float4*)&sh_post[wave][16 * g + 4 * i];
+          vv[4 * i] = x.x; vv[4 * i + 1] = x.y; vv[4 * i + 2] = x.z; vv[4 * i + 3] = x.w;
+        }
+        const float gate = P.post_gate ? sh_post[wave][64 + head] : 1.0f;
         UVMI_TS(4, 1);
         float proj = 0.f;
 #pragma unroll
@@ -448,7 +465,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
         }
         if (P.post_xsa) {
           proj = xsum32(xsum16(proj));
-          const float ah = P.post_xsa[h * G + head] * proj;
+          const float ah = sh_post[wave][72 + head] * proj;
 #pragma unroll
           for (int i = 0; i < 16; i++) o[i] = rnd(o[i] - ah * vv[i], QDT);
         }
@@ -784,7 +801,7 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
     // per item would need more wave slots than the device has at this kernel's occupancy (4 per SIMD), 2 per item keep
     // the whole launch resident in one round instead of two (measured: 2000 rows x ~230 keys, 15.6 us against 18.9 us).
     const int ctx = a->window > 0 && a->window < a->S ? a->window : a->S;
-    int wpr = ctx >= 512 ? 4 : (ctx >= 128 ? 2 : 1);
+    int wpr = ctx >= 256 ? 4 : (ctx >= 128 ? 2 : 1);
     {
       int cus = uvmi_device_cus();
       if (cus <= 0) cus = 256;
