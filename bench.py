@@ -146,12 +146,16 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
     lib = L.lib()
     g = make_rollout(False)
     g._admit()
+    fused = eng.fuse_qkv
+    if fused:   # keep each layer's projection of the sampled step, so that the re-issued launches are the step's own
+        eng.qkvx_keep = [torch.empty_like(eng.buf["qkvx"][:g.B]) for _ in range(cfg.n_layers)]
     layers = list(range(cfg.n_layers))
     ring_layers = [l for l in layers if not cfg.is_global(l)]
     n_glob = len(layers) - len(ring_layers)
     scratch = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
     stream = torch.cuda.current_stream().cuda_stream
     samples = []   # (events A, events B, bytes global, bytes ring)
+    ev_plain = []  # events of the attention-only kernel's sequence A (when the step runs the fused kernel)
 
     def timed_seq(args_list):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -171,9 +175,16 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
             torch.cuda.synchronize()
             n = g.bucket_for(g.n_active_host)
             act, pos, starts = g.act[:n], g.pos_c[:n], g.starts_c[:n]
-            built = {l: eng.cache_attention_args(l, g.st, pos, starts, n, rows=act) for l in layers}
+            if fused:
+                built = {l: eng.fused_attention_args(l, eng.qkvx_keep[l], g.tok_c[:n], g.st, pos, starts, n, rows=act) for l in layers}
+            else:
+                built = {l: eng.cache_attention_args(l, g.st, pos, starts, n, rows=act) for l in layers}
             evA = timed_seq([built[l][0] for l in layers])
             evB = timed_seq([built[l][0] for l in ring_layers])
+            if fused:   # the attention-only kernel on the same caches and positions (q and the epilogue inputs are whatever
+                        # the engine's buffers hold: only the timing is used)
+                plain = {l: eng.cache_attention_args(l, g.st, pos, starts, n, rows=act) for l in layers}
+                ev_plain.append(timed_seq([plain[l][0] for l in layers]))
             torch.cuda.synchronize()
             live = act.cpu().numpy() >= 0
             p, st = pos.cpu().numpy()[live], starts.cpu().numpy()[live]   # what the kernels saw (padding rows: no keys)
@@ -186,6 +197,7 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
             ta, tb = a0.elapsed_time(a1) * 1e3 / reps, b0.elapsed_time(b1) * 1e3 / reps
             print(f"# sample {i}: global {gbts / 1e6:.1f} MB {(ta - tb) / n_glob:.2f} us, ring {rbts / 1e6:.1f} MB {tb / len(ring_layers):.2f} us",
                   file=sys.stderr)
+    eng.qkvx_keep = None
     tA = sum(a.elapsed_time(b) for (a, b), _, _, _ in samples) * 1e3 / reps      # us, all layers, summed over samples
     tB = sum(a.elapsed_time(b) for _, (a, b), _, _ in samples) * 1e3 / reps      # us, ring layers only
     ns = len(samples)
@@ -199,15 +211,23 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
     gb, rb, ab = glob_bytes / glob_us / 1e3, ring_bytes / ring_us / 1e3, all_bytes / all_us / 1e3
     # The headline figure covers every decode-attention launch of the step (sequence A as timed: two global-layer and
     # eight ring-layer launches of the same kernel); the split by layer kind (A - B, B) is reported beside it.
+    extra = {}
+    if ev_plain:
+        plain_us = sum(a.elapsed_time(b) for a, b in ev_plain) * 1e3 / reps / (n_all * ns)
+        extra["attention_only_kernel"] = {
+            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=false> (the same launches without the fused QKV post-processing, which then "
+                      "costs a separate ~10 us launch per layer)",
+            "achieved": round(all_bytes / plain_us / 1e3, 1), "frac": round(all_bytes / plain_us / 1e3 / HBM_PEAK_GBS, 4),
+            "avg_launch_us": round(plain_us, 2), "launches_timed": n_all * ns * reps}
     return {"bound": "hbm", "achieved": round(ab, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ab / HBM_PEAK_GBS, 4),
             "traffic": int(all_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
-            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR> (bf16 q, bf16 out; all ten layers' launches of a step; WPR = 2 waves per row "
-                      "while 4 would not fit the device in one round, else 4 on the global layers)",
+            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=true> (bf16; all ten layers' launches of a step; the kernel also does the "
+                      "row's QKV post-processing and int8 append; WPR = 2 waves per row while 4 would not fit the device in one round, else 4)",
             "avg_launch_us": round(all_us, 2), "bytes_per_launch": int(all_bytes), "steps_sampled": ns, "launches_timed": n_all * ns * reps,
             "global_layers": {"achieved": round(gb, 1), "frac": round(gb / HBM_PEAK_GBS, 4), "avg_launch_us": round(glob_us, 2),
                               "bytes_per_launch": int(glob_bytes), "launches_timed": n_glob * ns * reps},
             "ring_layers": {"achieved": round(rb, 1), "frac": round(rb / HBM_PEAK_GBS, 4), "avg_launch_us": round(ring_us, 2),
-                            "bytes_per_launch": int(ring_bytes), "launches_timed": len(ring_layers) * ns * reps}}
+                            "bytes_per_launch": int(ring_bytes), "launches_timed": len(ring_layers) * ns * reps}, **extra}
 
 
 def cpu_baseline_c5(cfg, prompts, limits, budget_s=15.0, rows=32):

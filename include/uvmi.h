@@ -83,6 +83,7 @@ int uvmi_kv_append(const uvmi_kv_append_args* a, void* stream);
  * Ragged single-query decode attention.  Replaces decode_attention / mathk::decode_attn
  * (ultraviolet/kernels/decode_attn.py:174-230, kernels/decode_attn_cuda.py:273-309).
  * ---------------------------------------------------------------------------------------------------------- */
+struct uvmi_attn_qkv_fuse;
 typedef struct uvmi_attn_args {
   const void* q; int q_dtype;              /* (B, H, hd) F16 or BF16, inner stride 1 */
   int64_t sqb, sqh;
@@ -113,7 +114,28 @@ typedef struct uvmi_attn_args {
   const float* post_gate;                  /* (B, H) fp32 gate values (uvmi_qkv_post gate_out), or NULL */
   const float* post_xsa;                   /* (H,) tanh(alpha) fp32, or NULL */
   int post_round_dtype;                    /* activation dtype whose rounding the epilogue follows (F16 / BF16 / F32) */
+  const struct uvmi_attn_qkv_fuse* fuse;   /* optional: take q and the row's own key from the projection output (below) */
 } uvmi_attn_args;
+
+/* Fused QKV post-processing for decode rows (uvmi_attn_args.fuse).  The attention kernel then does what uvmi_qkv_post
+ * does for the row's own token (QK-norm, partial rotation, value embedding, int8 append at pos[b] - the reference's
+ * Attention.qkv + fast_decode.py:291-294, 315-317) and attends the cached range lo..pos-1 plus that key from registers,
+ * so the step needs no separate post-processing launch.  `qkv` is the output of the projection GEMM, (B, row_stride)
+ * in the q dtype: H*64 q values, KH*64 k, KH*64 v, then at column ext_col the H gate logits (W_gate[h] . xn[:gate_ch],
+ * formed by appending the gate rows to the projection weight) and the KH value-embedding gate logits.  q / sqb / sqh of
+ * the attention arguments are ignored; k_cache, v_cache and the scales are written at the rows' positions.  The XSA /
+ * gate epilogue is always applied (post_vhat and post_gate are ignored: the kernel forms them; post_xsa may be NULL).
+ * Needs the MFMA path (head_dim 64, int8 cache), num_splits == 1, q dtype = activation dtype, n_pairs 16 when rope. */
+typedef struct uvmi_attn_qkv_fuse {
+  const void* qkv; int64_t row_stride;     /* elements */
+  int ext_col;                             /* first gate-logit column */
+  int has_gate;                            /* gate logits present (else gate = 1) */
+  const void* tok;                         /* (B,) token ids (idx_dtype of the attention arguments), for the value embedding */
+  const void* ve_table; int64_t vocab;     /* (vocab, KH, 64) value embedding in the q dtype, or NULL (has_ve = 0) */
+  int has_ve;
+  const float* inv_freq; int n_pairs; int rope;
+  float eps, xsa_eps;
+} uvmi_attn_qkv_fuse;
 
 /* Keys attended by row b: absolute positions max(starts[b], pos[b]-window+1, 0) .. pos[b]; a row with no valid
  * key yields zeros.  fp32 accumulation; int8 caches are dequantised in registers (K scale on the score column,

@@ -259,3 +259,72 @@ def test_patch_model_binds_the_reference_entry_points():
     from ultraviolet_amd import _lib as L
     with pytest.raises(L.UvmiError):
         fd.patch_model(_StubModel(cfg, params), kv_dtype="fp16")
+
+
+def _fused_vs_unfused(cfg, eng, steps=40, resync=True):
+    """Run the same teacher-forced decode with and without the fused QKV path from identical prefilled states; after every
+    step the fused state's caches are overwritten with the unfused ones so that differences do not accumulate.  Returns
+    per-step hidden differences, argmax agreement of the logits and per-layer cache statistics."""
+    from ultraviolet_amd.engine import KVState
+    prompts = _prompts(cfg, (5, 40, 17, 33, 1, 26), seed=11)
+    B = len(prompts)
+    cont = np.random.default_rng(12).integers(1, cfg.vocab_size, size=(B, steps))
+    sts = [KVState(cfg, B, 96, DEV) for _ in range(2)]
+    for st in sts:
+        eng.prefill(prompts, list(range(B)), st)
+    hdiff, agree, cmax, cfrac, sfrac = [], [], np.zeros(cfg.n_layers), np.zeros(cfg.n_layers), np.zeros(cfg.n_layers)
+    for t in range(steps):
+        tok = torch.as_tensor(cont[:, t]).to(DEV)
+        h0 = eng.decode_step(tok, sts[0], fuse=False).clone()
+        h1 = eng.decode_step(tok, sts[1], fuse=True).clone()
+        assert torch.isfinite(h1.float()).all()
+        hdiff.append(float((h0.float() - h1.float()).abs().max()))
+        agree.append(float((eng.logits(h0).argmax(-1) == eng.logits(h1).argmax(-1)).float().mean()))
+        for l in range(cfg.n_layers):
+            for a, b_, sa, sb in ((sts[0].k[l], sts[1].k[l], sts[0].k_scale[l], sts[1].k_scale[l]),
+                                  (sts[0].v[l], sts[1].v[l], sts[0].v_scale[l], sts[1].v_scale[l])):
+                d = (a.int() - b_.int()).abs()
+                cmax[l] = max(cmax[l], int(d.max()))
+                cfrac[l] = max(cfrac[l], float((d > 0).float().sum()) / (B * cfg.n_kv_heads * cfg.head_dim))   # of the bytes written this step
+                sfrac[l] = max(sfrac[l], float((sa.view(torch.int16) != sb.view(torch.int16)).float().sum()) / (B * cfg.n_kv_heads))
+                if resync:
+                    b_.copy_(a)
+                    sb.copy_(sa)
+    assert sts[0].pos.tolist() == sts[1].pos.tolist()
+    return hdiff, agree, cmax, cfrac, sfrac
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("gate_ch", [0, 128])
+def test_fused_qkv_single_layer_is_exact(dtype, gate_ch):
+    """One layer isolates the fused kernel from error propagation: QK-norm, rotation, value embedding and the quantiser
+    must reproduce the separate post-processing kernel bit for bit (identical int8 bytes and fp16 scales at every step,
+    through ring wrap-around), and the layer output - own key merged from registers instead of streamed, gate logits from
+    the projection instead of a separate dot product - must agree to a unit or two in the last place."""
+    cfg, params, eng, _ = _setup("uv-test", dtype=dtype, perturb=0.05, window=32, n_layers=1, global_every=0, ve_every=1,
+                                 attn_gate_channels=gate_ch)
+    assert eng.fuse_qkv and cfg.has_ve(0)
+    hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng)
+    assert cmax.max() == 0 and sfrac.max() == 0
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    assert max(hdiff) <= 4 * 2 * ulp, max(hdiff)      # |h| < 4 after the final norm: one ulp there is 2 * ulp(1)
+    cfg, params, eng, _ = _setup("uv-test", dtype=dtype, perturb=0.05, window=0, n_layers=1, global_every=1, ve_every=0,
+                                 attn_gate_channels=gate_ch)   # a global layer (no rotation, linear cache), no value embedding
+    hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng)
+    assert cmax.max() == 0 and sfrac.max() == 0 and max(hdiff) <= 4 * 2 * ulp
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("name,over", [("uv-test", dict(window=32)), ("uv-50m-alpha", dict())])
+def test_fused_qkv_decode_matches_unfused(dtype, name, over):
+    """Whole models: layer 0 appends identical bytes; deeper layers see inputs that differ in the last place of the
+    activation type, which moves int8 codes near a rounding boundary by a step or two; the final hidden states stay within
+    a few units in the last place and the logits' argmax agrees."""
+    cfg, params, eng, _ = _setup(name, dtype=dtype, perturb=0.05, **over)
+    assert eng.fuse_qkv
+    hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=24)
+    assert cmax[0] == 0 and sfrac[0] == 0
+    assert (cmax <= 1 + np.arange(cfg.n_layers)).all(), cmax     # the perturbation grows layer by layer (bf16 activations)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
+    assert np.mean(agree) > 0.9, np.mean(agree)

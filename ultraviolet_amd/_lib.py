@@ -38,7 +38,14 @@ class AttnArgs(C.Structure):
                 ("B", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("S", C.c_int), ("hd", C.c_int),
                 ("scale", C.c_float), ("window", C.c_int), ("ring", C.c_int), ("num_splits", C.c_int),
                 ("chunk_keys", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
-                ("post_vhat", C.c_void_p), ("post_gate", C.c_void_p), ("post_xsa", C.c_void_p), ("post_round_dtype", C.c_int)]
+                ("post_vhat", C.c_void_p), ("post_gate", C.c_void_p), ("post_xsa", C.c_void_p), ("post_round_dtype", C.c_int),
+                ("fuse", C.c_void_p)]
+
+
+class AttnQkvFuse(C.Structure):
+    _fields_ = [("qkv", C.c_void_p), ("row_stride", C.c_int64), ("ext_col", C.c_int), ("has_gate", C.c_int), ("tok", C.c_void_p),
+                ("ve_table", C.c_void_p), ("vocab", C.c_int64), ("has_ve", C.c_int), ("inv_freq", C.c_void_p), ("n_pairs", C.c_int),
+                ("rope", C.c_int), ("eps", C.c_float), ("xsa_eps", C.c_float)]
 
 
 class PrefillAttnArgs(C.Structure):

@@ -51,12 +51,17 @@ struct AttnParams {
   float scale_log2;
   // optional fused epilogue (Attention.post of the reference, model.py:321-333)
   const float* post_vhat; const float* post_gate; const float* post_xsa; int post_dt;
+  // optional fused QKV post-processing of the row's own token (model.py:302-319, fast_decode.py:291-294, 315-317)
+  const void* f_qkv; const void* f_tok; const void* f_ve; const float* f_inv_freq;
+  int64_t f_sqkv, f_vocab;
+  int f_ext, f_rope, f_has_ve, f_has_gate;
+  float f_eps, f_xsa_eps;
 };
 
 // Key range of a row and how it is cut.  The span starts at lo rounded down to 32 so tiles stay aligned to the
 // slot grid; each work item gets `chunk` keys (a multiple of 32, at least chunk_keys, and large enough that at most
 // `splits` items cover the span).  A row with a single chunk is written directly, without partials.
-struct RowPlan { int lo, p, a0, chunk, nsplit, cb; };
+struct RowPlan { int lo, p, a0, chunk, nsplit, cb, pc; };  // p: last streamed position; pc: the row's own position
 // Low 32 bits of element i of an I32 / I64 index array (positions, starts and row ids fit 31 bits; -1 keeps its sign),
 // for a wave-uniform i: one 4-byte scalar load whatever the width (constant address space: the arrays are inputs of the
 // launch), so the three loads of a plan have no branches between them and go out together.
@@ -64,16 +69,20 @@ __device__ __forceinline__ int load_idx32(const void* p, int is64, int64_t i) {
   typedef const int32_t __attribute__((address_space(4))) * cptr32;
   return *(cptr32)((uintptr_t)p + (uintptr_t)(i * (is64 ? 8 : 4)));
 }
-__device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b) {
+// own_key_apart: the key at the row's own position is not in the cache yet (the kernel forms it itself), so the streamed
+// range ends one position earlier.
+__device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b, bool own_key_apart = false) {
   RowPlan r;
   const int pv = load_idx32(P.pos, P.idx64, b);
   const int st = load_idx32(P.starts, P.idx64, b);
   const int rv = load_idx32(P.rows ? P.rows : P.pos, P.idx64, b);
   r.cb = P.rows ? rv : b;               // cache row of this query row
-  const int p = r.cb < 0 ? -1 : pv;     // padding row of a compacted batch: no keys, output zeros
+  const int pc = r.cb < 0 ? -1 : pv;    // padding row of a compacted batch: no keys, output zeros
   if (r.cb < 0) r.cb = 0;               // (dead rows have no keys; keep addresses valid)
   int lo = st > 0 ? st : 0;
-  if (P.window > 0 && p - P.window + 1 > lo) lo = p - P.window + 1;
+  if (P.window > 0 && pc - P.window + 1 > lo) lo = pc - P.window + 1;
+  const int p = own_key_apart ? pc - 1 : pc;
+  r.pc = pc;
   r.lo = lo;
   r.p = p;
   r.a0 = lo & ~31;
@@ -140,8 +149,11 @@ __device__ unsigned long long g_attn_tim[1 << 15][8];
 #define UVMI_TS(k, force) do { } while (0)
 #endif
 
-template <int QDT, int ODT, int WPR>
-__global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
+// FUSE: the row's own token is taken from the projection output (q, k, v, gate logits) instead of from q and the cache:
+// the kernel normalises and rotates q and k, adds the value embedding to v, quantises k and v into the cache, and attends
+// the streamed cache range lo..pos-1 plus the own key from registers; the XSA / gate epilogue uses the own v directly.
+template <int QDT, int ODT, int WPR, bool FUSE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void attn_mfma_i8_hd64(AttnParams P) {
 #ifdef UVMI_ATTN_TIMING
   unsigned long long tim_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   UVMI_TS(0, 0);
@@ -150,6 +162,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
   __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
   __shared__ float sh_post[4][80];  // epilogue operands of the item whose first wave this is: v_hat[64], gate[8], xsa[8]
+  __shared__ float sh_cur[FUSE ? 4 : 1][72];  // own key of that item: score per head [8], dequantised v [64]
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wsub = wave % WPR;
@@ -171,18 +184,31 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   // (no branch around the loads: lanes of absent heads read head G-1 and are masked to zero when the operands are
   // formed, which keeps the control flow, and with it every row-derived scalar, wave-uniform)
   const uint32_t qmask = head < G ? 0xffffffffu : 0u;
-  const uint16_t* qp = (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + (head < G ? head : G - 1)) * P.sqh + 16 * g;
+  const uint16_t* qp = FUSE ? (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv + (h * G + (head < G ? head : G - 1)) * 64 + 16 * g
+                            : (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + (head < G ? head : G - 1)) * P.sqh + 16 * g;
   const uint4 qw0 = *(const uint4*)qp, qw1 = *(const uint4*)(qp + 8);
+  // FUSE: the row's gate logits go out with q (the raw k, v and value-embedding row are read by the item's first wave
+  // when it forms the own key: holding them from here on would cost a wave slot per SIMD)
+  uint16_t glog = 0, vlog = 0;
+  int64_t own_tok = 0;
+  if constexpr (FUSE) {
+    const uint16_t* rowp = (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv;
+    glog = rowp[P.f_ext + (P.f_has_gate ? h * G + (head < G ? head : G - 1) : 0)];
+    vlog = rowp[P.f_ext + P.H + h];
+    own_tok = P.f_has_ve ? (int64_t)load_idx32(P.f_tok, P.idx64, b) : 0;
+    own_tok = own_tok < 0 ? 0 : (own_tok >= P.f_vocab ? P.f_vocab - 1 : own_tok);
+  }
   // Operands of the fused epilogue are requested now, with q, and parked in LDS once q has arrived, so that the
   // epilogue at the end of the workgroup's life does not start with a round trip to memory.  Unconditional loads (from
   // q when there is no epilogue) keep the control flow uniform.
-  const bool has_post = P.post_vhat != nullptr;
+  const bool has_post = FUSE || P.post_vhat != nullptr;
   const int hsafe = h * G + (head < G ? head : G - 1);
-  const float* pv_src = has_post ? P.post_vhat + ((int64_t)b * P.KH + h) * 64 + lane : (const float*)P.q + lane;
-  const float* pg_src = has_post && P.post_gate ? P.post_gate + (int64_t)b * P.H + hsafe : (const float*)P.q;
-  const float* px_src = has_post && P.post_xsa ? P.post_xsa + hsafe : (const float*)P.q;
+  const float* anyf = FUSE ? (const float*)P.f_qkv : (const float*)P.q;  // a readable address for the unused cases
+  const float* pv_src = !FUSE && has_post ? P.post_vhat + ((int64_t)b * P.KH + h) * 64 + lane : anyf + lane;
+  const float* pg_src = !FUSE && has_post && P.post_gate ? P.post_gate + (int64_t)b * P.H + hsafe : anyf;
+  const float* px_src = has_post && P.post_xsa ? P.post_xsa + hsafe : anyf;
   const float pv_val = *pv_src, pg_val = *pg_src, px_val = *px_src;
-  const RowPlan rp = plan_row(P, b);
+  const RowPlan rp = plan_row(P, b, FUSE);
   const bool live = live_item && sid < rp.nsplit;
   if (WPR == 1 && !live) return;
   const int s0 = rp.a0 + sid * rp.chunk;
@@ -196,10 +222,62 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   const uint32_t mA = strm == 0 ? qmask : 0u, mB = strm == 0 ? 0u : qmask;
   h8 QA0, QA1, QB0, QB1;
   float cinit;
+  // helpers of the fused path: 16 values of the activation type <-> fp32, rounding to the activation type, RMS norm over
+  // the 64 dims of a head (4 lane groups) and the partial rotation (dims 0..15 pair with 16..31: lane groups 0 and 1)
+  auto unpack16 = [&](const uint4& a, const uint4& b2, float (&x)[16]) {
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b2.x, b2.y, b2.z, b2.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if (QDT == UVMI_BF16) { x[2 * i] = __uint_as_float(w[i] << 16); x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+      else { x[2 * i] = half_bits_to_float(w[i] & 0xffff); x[2 * i + 1] = half_bits_to_float(w[i] >> 16); }
+    }
+  };
+  auto rq = [&](float v) -> float { return QDT == UVMI_BF16 ? bf16_to_float(float_to_bf16(v)) : (float)(half_t)v; };
+  float rcs[16], rsn[16];  // cos / sin of the row's position per frequency (wave-uniform, rounded to the activation type)
+  auto norm_rope = [&](float (&x)[16]) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) ss += x[i] * x[i];
+    ss = xsum32(xsum16(ss));
+    const float rs = rsqrtf(ss * (1.0f / 64.0f) + P.f_eps);
+#pragma unroll
+    for (int i = 0; i < 16; i++) x[i] = rq(x[i] * rs);
+    if (P.f_rope) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        // the partner dim lives in the neighbouring lane group: after the swap r[0] holds groups (0, 0, 2, 2) and r[1]
+        // groups (1, 1, 3, 3) of x[i]
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x[i]), __float_as_uint(x[i]), false, false);
+        const float y = __uint_as_float((g & 1) ? r[0] : r[1]);
+        if (g == 0) x[i] = rq(x[i] * rcs[i] - y * rsn[i]);
+        else if (g == 1) x[i] = rq(y * rsn[i] + x[i] * rcs[i]);
+      }
+    }
+  };
+  uint32_t qr[8];
   auto prep_q = [&]() {
-    uint32_t qr[8];
     float qsum = 0.f;
-    const uint32_t w[8] = {qw0.x, qw0.y, qw0.z, qw0.w, qw1.x, qw1.y, qw1.z, qw1.w};
+    uint32_t w[8] = {qw0.x, qw0.y, qw0.z, qw0.w, qw1.x, qw1.y, qw1.z, qw1.w};
+    if constexpr (FUSE) {
+      if (P.f_rope) {
+        const float th = (float)rp.pc * P.f_inv_freq[m];
+        const float cl = rq(cosf(th)), sl = rq(sinf(th));
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+          rcs[j] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(cl), j));
+          rsn[j] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(sl), j));
+        }
+      }
+      float x[16];
+      unpack16(qw0, qw1, x);
+      norm_rope(x);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {  // back to the packed activation type: the conversion below is shared with the unfused path
+        const uint32_t lo16 = QDT == UVMI_BF16 ? float_to_bf16(x[2 * i]) : float_to_half_bits(x[2 * i]);
+        const uint32_t hi16 = QDT == UVMI_BF16 ? float_to_bf16(x[2 * i + 1]) : float_to_half_bits(x[2 * i + 1]);
+        w[i] = lo16 | (hi16 << 16);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       float f0, f1;
@@ -213,6 +291,98 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
     QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA); QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
     QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB); QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
     cinit = qmask ? -1152.0f * qsum : 0.f;
+  };
+
+  // FUSE, first wave of the item: k (norm, rotation), v (value embedding), int8 append at the row's position, and what the
+  // end of the kernel needs from them - the own key's score per head and dequantised value (merged into the softmax after
+  // the streamed range), v_hat and the gate for the epilogue - parked in LDS.  Arithmetic and roundings follow the
+  // standalone post-processing kernel (uvmi_qkv_post).
+  constexpr int VW = WPR > 1 ? 1 : 0;  // the wave of an item that forms the own value (the first wave forms the own key)
+  const int iw = wave - wsub;          // LDS slot of the item: its first wave
+  // quantise 16 values per lane of a 64-dim row spread over the 4 lane groups (the arithmetic of the standalone
+  // quantizer: fp16 scale, IEEE division, round half to even, clamp); returns the scale as fp32
+  auto quant = [&](const float (&x)[16], float (&qv)[16], uint16_t& sb) -> float {
+    float am = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) am = fmaxf(am, fabsf(x[i]));
+    am = xmax32(xmax16(am));
+    sb = float_to_half_bits(__fdiv_rn(am, 127.0f));
+    const float sf = fmaxf(half_bits_to_float(sb), 1e-30f);
+#pragma unroll
+    for (int i = 0; i < 16; i++) qv[i] = fminf(fmaxf(__builtin_rintf(__fdiv_rn(x[i], sf)), -127.0f), 127.0f);
+    return half_bits_to_float(sb);
+  };
+  auto pack = [&](const float (&qv)[16]) -> uint4 {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      w[i] = ((uint32_t)(int)qv[4 * i] & 0xffu) | (((uint32_t)(int)qv[4 * i + 1] & 0xffu) << 8) | (((uint32_t)(int)qv[4 * i + 2] & 0xffu) << 16) |
+             (((uint32_t)(int)qv[4 * i + 3] & 0xffu) << 24);
+    return uint4{w[0], w[1], w[2], w[3]};
+  };
+  // own_k (first wave of the item): k -> norm, rotation -> int8 append; the own key's score per head (q as the fp16
+  // operand holds it . k_int8 * k scale, in the units of the streamed scores) and the gate values go to LDS.
+  auto own_k = [&](const uint4& a0, const uint4& a1) {
+    float kx[16], kq[16];
+    uint16_t sbk;
+    unpack16(a0, a1, kx);
+    norm_rope(kx);
+    const float ksf = quant(kx, kq, sbk);
+    const int slot = P.ring ? rp.pc % P.S : rp.pc;
+    if (slot < P.S && m == 0) {  // one lane per group writes its 16 bytes of the row; lane 0 the scale
+      *(uint4*)((int8_t*)P.kc + (int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + 16 * g) = pack(kq);
+      if (g == 0) ((uint16_t*)P.ks)[(int64_t)rp.cb * P.ssb + (int64_t)h * P.ssh + slot] = sbk;
+    }
+    float dq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      dq += half_bits_to_float(qr[i] & 0xffff) * kq[2 * i] + half_bits_to_float(qr[i] >> 16) * kq[2 * i + 1];
+    dq = xsum32(xsum16(dq)) * ksf;
+    if (lane < 8) {
+      sh_cur[iw][lane] = dq;
+      const float lg = QDT == UVMI_BF16 ? bf16_to_float(glog) : half_bits_to_float(glog);
+      sh_post[iw][64 + lane] = P.f_has_gate ? rq(2.0f * rq(1.0f / (1.0f + __expf(-lg)))) : 1.0f;
+    }
+    if (lane >= 8 && lane < 16) sh_post[iw][64 + lane] = px_val;
+  };
+  // own_v (second wave of the item when there is one): v (+ value embedding) -> int8 append; the dequantised own value
+  // and v_hat for the XSA epilogue go to LDS.  Arithmetic and roundings follow uvmi_qkv_post.
+  auto own_v = [&](const uint4& a0, const uint4& a1, const uint4& e0, const uint4& e1) {
+    float vx[16], vq[16];
+    uint16_t sbv;
+    unpack16(a0, a1, vx);
+    if (P.f_has_ve) {
+      float ve[16];
+      unpack16(e0, e1, ve);
+      const float dot = QDT == UVMI_BF16 ? bf16_to_float(vlog) : half_bits_to_float(vlog);
+      const float gv = rq(2.0f * rq(1.0f / (1.0f + __expf(-dot))));
+#pragma unroll
+      for (int i = 0; i < 16; i++) vx[i] = rq(vx[i] + rq(gv * ve[i]));
+    }
+    float vv2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) vv2 += vx[i] * vx[i];
+    const float nv = fmaxf(sqrtf(xsum32(xsum16(vv2))), P.f_xsa_eps);
+    const float vsf = quant(vx, vq, sbv);
+    const int slot = P.ring ? rp.pc % P.S : rp.pc;
+    if (m == 0) {
+      if (slot < P.S) {
+        *(uint4*)((int8_t*)P.vc + (int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + 16 * g) = pack(vq);
+        if (g == 0) ((uint16_t*)P.vs)[(int64_t)rp.cb * P.stb + (int64_t)h * P.sth + slot] = sbv;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        sh_cur[iw][8 + 16 * g + i] = vsf * vq[i];
+        sh_post[iw][16 * g + i] = vx[i] / nv;
+      }
+    }
+  };
+  // raw inputs of own_k / own_v: every lane of a 16-lane group g reads dims 16g..16g+15 of the row's k (first wave) or v
+  // and value-embedding row (second wave); requested right after the first tile, used after q is ready
+  const uint16_t* own_row = (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv;
+  auto own_src = [&](bool v_part) -> const uint16_t* { return own_row + (P.H + (v_part ? P.KH : 0) + h) * 64 + 16 * g; };
+  auto own_ve = [&](const uint16_t* fallback) -> const uint16_t* {
+    return P.f_has_ve ? (const uint16_t*)P.f_ve + (own_tok * P.KH + h) * 64 + 16 * g : fallback;
   };
 
   AttnState st;
@@ -357,14 +527,35 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
       return sl;
     };
     // The first tile is requested unconditionally (a wave without a pipelined tile reads slot 0 and drops it; the
-    // descriptor bounds the access), so that the q conversion, which waits for q only, follows it on every path.
+    // descriptor bounds the access), so that the q conversion - and, on the fused path, the forming of the row's own key -
+    // follows it on every path and waits for q only.  (Requesting two tiles here was measured: the second tile's
+    // registers, live across the own-key arithmetic, push the fused kernel into spills.)
     Tile TA, TB;
     load_tile(slot, TA);
+    uint4 aw0, aw1, ew0, ew1;
+    if constexpr (FUSE) {
+      const uint16_t* ap = own_src(WPR > 1 && wsub == VW);
+      const uint16_t* ep = own_ve(ap);
+      aw0 = *(const uint4*)ap; aw1 = *(const uint4*)(ap + 8);
+      ew0 = *(const uint4*)ep; ew1 = *(const uint4*)(ep + 8);
+    }
     __builtin_amdgcn_sched_barrier(0);
     prep_q();
-    if (wsub == 0) {
-      sh_post[wave][lane] = pv_val;
-      if (lane < 16) sh_post[wave][64 + lane] = lane < 8 ? pg_val : px_val;  // lanes 8..15 carry head lane - 8 too
+    if constexpr (!FUSE) {
+      if (wsub == 0) {
+        sh_post[wave][lane] = pv_val;
+        if (lane < 16) sh_post[wave][64 + lane] = lane < 8 ? pg_val : px_val;  // lanes 8..15 carry head lane - 8 too
+      }
+    } else if (live && rp.pc >= 0) {
+      if (WPR > 1) {
+        if (wsub == 0) own_k(aw0, aw1);
+        else if (wsub == VW) own_v(aw0, aw1, ew0, ew1);
+      } else {  // one wave per item forms both; the value's inputs are read here
+        own_k(aw0, aw1);
+        const uint16_t* vp = own_src(true);
+        const uint16_t* ep = own_ve(vp);
+        own_v(*(const uint4*)vp, *(const uint4*)(vp + 8), *(const uint4*)ep, *(const uint4*)(ep + 8));
+      }
     }
     if (has) {
       while (true) {
@@ -441,21 +632,33 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
   }
   if (strm == 0 && head < G) {
     if (rp.nsplit == 1) {
+      if constexpr (FUSE) {
+        if (rp.pc >= 0) {  // the own key joins the softmax after the streamed range
+          const float s2 = sh_cur[wave][head] * c;
+          const float mnew = fmaxf(mfin, s2);
+          const float wa = mfin == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mfin - mnew), wb = __builtin_amdgcn_exp2f(s2 - mnew);
+          lfin = lfin * wa + wb;
+#pragma unroll
+          for (int i = 0; i < 16; i++) o[i] = o[i] * wa + wb * sh_cur[wave][8 + 16 * g + i];
+          mfin = mnew;
+        }
+      }
       const float inv = lfin > 0.f ? 1.0f / lfin : 0.f;
       const int64_t off = (int64_t)b * P.sob + (int64_t)(h * G + head) * P.soh + 16 * g;
-      if (P.post_vhat) {
+      if (has_post) {
         // z (rounded to the q dtype, as the attention output tensor would be) -> XSA -> gate, written in the output type.
         // All lanes of a head column (n, g = 0..3) are active here, so the cross-group swaps are well defined.
         auto rnd = [&](float x, int dt) -> float {
           return dt == UVMI_F32 ? x : (dt == UVMI_BF16 ? bf16_to_float(float_to_bf16(x)) : (float)(half_t)x);
         };
+        const bool dead = FUSE && rp.pc < 0;  // padding row of the fused path: nothing was parked for it, the output is zero
         float vv[16];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const float4 x = *(const float4*)&sh_post[wave][16 * g + 4 * i];
-          vv[4 * i] = x.x; vv[4 * i + 1] = x.y; vv[4 * i + 2] = x.z; vv[4 * i + 3] = x.w;
+          vv[4 * i] = dead ? 0.f : x.x; vv[4 * i + 1] = dead ? 0.f : x.y; vv[4 * i + 2] = dead ? 0.f : x.z; vv[4 * i + 3] = dead ? 0.f : x.w;
         }
-        const float gate = P.post_gate ? sh_post[wave][64 + head] : 1.0f;
+        const float gate = dead ? 0.f : (FUSE || P.post_gate ? sh_post[wave][64 + head] : 1.0f);
         UVMI_TS(4, 1);
         float proj = 0.f;
 #pragma unroll
@@ -465,7 +668,7 @@ __global__ __launch_bounds__(256) void attn_mfma_i8_hd64(AttnParams P) {
         }
         if (P.post_xsa) {
           proj = xsum32(xsum16(proj));
-          const float ah = sh_post[wave][72 + head] * proj;
+          const float ah = dead ? 0.f : sh_post[wave][72 + head] * proj;
 #pragma unroll
           for (int i = 0; i < 16; i++) o[i] = rnd(o[i] - ah * vv[i], QDT);
         }
@@ -780,7 +983,22 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   P.scale_log2 = a->scale * LOG2E;
   P.ws_o = P.ws_m = P.ws_l = nullptr;
   P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa; P.post_dt = a->post_round_dtype;
-  if (a->post_vhat) {
+  P.f_qkv = nullptr;
+  if (const uvmi_attn_qkv_fuse* f = a->fuse) {
+    UVMI_REQUIRE(mfma_ok(a) && a->num_splits == 1, UVMI_EUNSUPPORTED,
+                 "uvmi_decode_attn: fused QKV post-processing needs the MFMA kernel (head_dim 64, int8 cache, aligned rows) and num_splits == 1");
+    UVMI_REQUIRE(a->out_dtype == a->q_dtype, UVMI_EUNSUPPORTED, "uvmi_decode_attn: fused QKV post-processing writes the q dtype");
+    UVMI_REQUIRE(f->qkv && ((uintptr_t)f->qkv % 16) == 0 && f->row_stride % 8 == 0 && f->ext_col >= (a->H + 2 * a->KH) * 64 &&
+                     f->row_stride >= f->ext_col + a->H + a->KH, UVMI_EINVAL, "uvmi_decode_attn: bad fused qkv layout");
+    UVMI_REQUIRE(!f->rope || (f->n_pairs == 16 && f->inv_freq), UVMI_EUNSUPPORTED, "uvmi_decode_attn: fused rotation needs n_pairs == 16");
+    UVMI_REQUIRE(!f->has_ve || (f->ve_table && f->tok && f->vocab > 0 && ((uintptr_t)f->ve_table % 16) == 0), UVMI_EINVAL,
+                 "uvmi_decode_attn: fused value embedding needs ve_table, tok and vocab");
+    P.f_qkv = f->qkv; P.f_sqkv = f->row_stride; P.f_ext = f->ext_col; P.f_has_gate = f->has_gate ? 1 : 0;
+    P.f_tok = f->tok; P.f_ve = f->ve_table; P.f_vocab = f->vocab; P.f_has_ve = f->has_ve ? 1 : 0;
+    P.f_inv_freq = f->inv_freq; P.f_rope = f->rope ? 1 : 0; P.f_eps = f->eps; P.f_xsa_eps = f->xsa_eps;
+    P.post_vhat = nullptr; P.post_gate = nullptr;
+  }
+  if (a->post_vhat && !a->fuse) {
     UVMI_REQUIRE(mfma_ok(a) && a->num_splits == 1, UVMI_EUNSUPPORTED,
                  "uvmi_decode_attn: the fused post epilogue needs the MFMA kernel (head_dim 64, int8 cache) and num_splits == 1");
     UVMI_REQUIRE(is_float_dtype(a->post_round_dtype) && ((uintptr_t)a->post_vhat % 16) == 0, UVMI_EINVAL, "uvmi_decode_attn: bad post arguments");
@@ -813,19 +1031,28 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
     if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
     const int ipb = 4 / wpr;
     const dim3 grid((unsigned)((P.n_items + ipb - 1) / ipb)), blk(256);
-#define UVMI_L(QD, OD)                                                                         \
-  do {                                                                                         \
-    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 4>), grid, blk, 0, st, P);      \
-    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2>), grid, blk, 0, st, P); \
-    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1>), grid, blk, 0, st, P);               \
+#define UVMI_L(QD, OD)                                                                                \
+  do {                                                                                                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 4, false>), grid, blk, 0, st, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2, false>), grid, blk, 0, st, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1, false>), grid, blk, 0, st, P);               \
+  } while (0)
+#define UVMI_LF(QD)                                                                                   \
+  do {                                                                                                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true>), grid, blk, 0, st, P);       \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true>), grid, blk, 0, st, P);  \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true>), grid, blk, 0, st, P);                \
   } while (0)
     const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
-    if (a->q_dtype == UVMI_F16) {
+    if (a->fuse) {
+      if (a->q_dtype == UVMI_F16) UVMI_LF(UVMI_F16); else UVMI_LF(UVMI_BF16);
+    } else if (a->q_dtype == UVMI_F16) {
       if (od == UVMI_F16) UVMI_L(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(UVMI_F16, UVMI_BF16); else UVMI_L(UVMI_F16, UVMI_F32);
     } else {
       if (od == UVMI_F16) UVMI_L(UVMI_BF16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(UVMI_BF16, UVMI_BF16); else UVMI_L(UVMI_BF16, UVMI_F32);
     }
 #undef UVMI_L
+#undef UVMI_LF
   } else {
     const dim3 grid((unsigned)P.n_items), blk(64);
     const size_t sh = ((size_t)P.G * a->hd + (size_t)P.G * 64) * 4;

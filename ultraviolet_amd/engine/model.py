@@ -16,7 +16,7 @@ import torch
 from torch import Tensor
 
 from .. import _lib as L
-from ..kernels.decode_attn import build_attn_args, decode_attention, decode_attention_post
+from ..kernels.decode_attn import build_attn_args, build_fused_args, decode_attention, decode_attention_fused, decode_attention_post
 from ..kernels.varlen_attn import packed_attention
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
@@ -82,6 +82,12 @@ class UVEngine:
         self.buf = dict(x=e(n, d), xn=e(n, d), h=e(n, d), qkv=e(n, (H + 2 * K) * hd), q=e(n, H, hd, dtype=self.q_dtype),
                         k=e(n, K, hd), v=e(n, K, hd), zg=e(n, H * hd), a=e(n, d), gu=e(n, 2 * f), act=e(n, f), m=e(n, d),
                         vhat=e(n, K, hd, dtype=torch.float32), gate=e(n, H, dtype=torch.float32))
+        # decode steps of a 16-bit engine take q, k, v and the gate logits from one extended projection and leave the
+        # post-processing to the attention kernel (one launch less per layer)
+        self.fuse_qkv = dt in (torch.bfloat16, torch.float16) and cfg.n_heads // cfg.n_kv_heads <= 8 and cfg.n_pairs in (0, 16)
+        self.qkvx_keep = None
+        if self.fuse_qkv:
+            self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
         self.pf_ws = torch.empty(L.lib().uvmi_prefill_attn_workspace_bytes(n), dtype=torch.uint8, device=dev)  # fails now if the library is missing
 
     # ------------------------------------------------------------------------------------------------ kernels
@@ -159,6 +165,40 @@ class UVEngine:
             return None
         return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, num_splits=1, **kw)
 
+    def fused_layer_ok(self, l: int, st: KVState) -> bool:
+        """Whether layer l's decode attention can take the fused path: the MFMA kernel streams 32-key tiles."""
+        S = st.k[l].size(2)
+        return self.fuse_qkv and S % 32 == 0 and S >= 32
+
+    def _fuse_dict(self, l: int, tok: Tensor) -> dict:
+        cfg = self.cfg
+        glob = cfg.is_global(l)
+        has_ve = cfg.has_ve(l)
+        return dict(ext_col=(cfg.n_heads + 2 * cfg.n_kv_heads) * cfg.head_dim, has_gate=cfg.gate_ch > 0, tok=tok if has_ve else None,
+                    ve_table=self.w.value_embed if has_ve else None, vocab=cfg.vocab_size, inv_freq=self.w.inv_freq, n_pairs=cfg.n_pairs,
+                    rope=((not glob) or cfg.global_rope) and cfg.n_pairs > 0, eps=self.eps, xsa_eps=cfg.xsa_eps)
+
+    def fused_cache_attention(self, l: int, tok: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
+        """Decode attention of layer l straight from buf qkvx (the extended projection of the n rows): QK-norm, rotation,
+        value embedding, int8 append, attention over lo..pos, XSA and gate in one launch; writes buf zg."""
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        glob = cfg.is_global(l)
+        out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
+        decode_attention_fused(b["qkvx"][:n], cfg.n_heads, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0 if glob else cfg.window,
+                               ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], xsa=W["xsa"], out=out,
+                               fuse=self._fuse_dict(l, tok), rows=rows)
+
+    def fused_attention_args(self, l: int, qkvx: Tensor, tok: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int,
+                             rows: Tensor | None = None):
+        """The uvmi_attn_args struct fused_cache_attention launches for layer l, on a given copy of that layer's extended
+        projection (qkvx_keep): lets a benchmark re-issue exactly the step's launches through the C ABI.  Re-issuing it
+        on the step's own positions rewrites the same K/V bytes."""
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        glob = cfg.is_global(l)
+        out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
+        return build_fused_args(qkvx[:n], cfg.n_heads, st.k[l], st.v[l], pos, starts, cfg.attn_scale, 0 if glob else cfg.window, not glob,
+                                st.k_scale[l], st.v_scale[l], W["xsa"], out, self._fuse_dict(l, tok), rows)
+
     def cache_attention_args(self, l: int, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
         """The uvmi_attn_args struct cache_attention would launch for layer l on the engine's buffers (fused path only):
         lets a benchmark re-issue exactly the step's attention launches through the C ABI without the Python wrapper."""
@@ -169,7 +209,8 @@ class UVEngine:
                                st.k_scale[l], st.v_scale[l], 1, out, 0, rows,
                                (b["vhat"][:n], None if W["attn_gate"] is None else b["gate"][:n], W["xsa"], out.dtype))
 
-    def _trunk(self, tok: Tensor, pos: Tensor, n: int, attn, rows=None, last_pos=None, st: KVState | None = None) -> Tensor:
+    def _trunk(self, tok: Tensor, pos: Tensor, n: int, attn, rows=None, last_pos=None, st: KVState | None = None,
+               fused_attn=None) -> Tensor:
         """n token rows through all layers; attn(l, q (n, H, hd)) -> z (n, H, hd) (or None when it wrote the post-processed
         result to buf zg itself) runs after K/V of the layer have been appended to the cache and written unquantized to
         buf k / v.  Returns the final normed hidden (n, d) (a buffer)."""
@@ -178,11 +219,19 @@ class UVEngine:
         self._embed_norm(tok, n)
         x, xn = b["x"][:n], b["xn"][:n]
         for l, W in enumerate(self.w.layers):
-            torch.mm(xn, W["wqkv"].t(), out=b["qkv"][:n])
-            self._qkv_post(l, tok, pos, rows, last_pos, st, n)
-            z = attn(l, b["q"][:n])
-            if z is not None:   # None: the attention kernel already applied XSA + gate and wrote buf zg
-                self._attn_post(l, z, n)
+            if fused_attn is not None and self.fused_layer_ok(l, st):
+                # decode rows of a 16-bit engine: the projection also forms the gate logits, and fused_attn(l) does the
+                # post-processing, the cache append, the attention and its epilogue in one launch (writes buf zg)
+                torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
+                if self.qkvx_keep is not None:   # a benchmark re-issues this layer's launch later on the same projection
+                    self.qkvx_keep[l][:n].copy_(b["qkvx"][:n])
+                fused_attn(l)
+            else:
+                torch.mm(xn, W["wqkv"].t(), out=b["qkv"][:n])
+                self._qkv_post(l, tok, pos, rows, last_pos, st, n)
+                z = attn(l, b["q"][:n])
+                if z is not None:   # None: the attention kernel already applied XSA + gate and wrote buf zg
+                    self._attn_post(l, z, n)
             torch.mm(b["zg"][:n], W["wo"].t(), out=b["a"][:n])
             # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
             self._add_norm(x, b["a"][:n], W["resid_attn"], W["post_attn"], n, b["h"], b["xn"])
@@ -204,7 +253,7 @@ class UVEngine:
 
     # ------------------------------------------------------------------------------------------------ decode
     @torch.no_grad()
-    def decode_step(self, tok: Tensor, st: KVState, num_splits: dict | None = None) -> Tensor:
+    def decode_step(self, tok: Tensor, st: KVState, num_splits: dict | None = None, fuse: bool = True) -> Tensor:
         """One token for all B rows at per-row st.pos (reference: decode_step_fast, fast_decode.py:272-334): append K/V
         at pos first, attend lo..pos, then st.pos += 1.  Returns the final normed hidden (B, d)."""
         cfg = self.cfg
@@ -220,7 +269,10 @@ class UVEngine:
             return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0 if glob else cfg.window, ring=not glob,
                                     k_scale=st.k_scale[l], v_scale=st.v_scale[l], num_splits=ns[key])
 
-        h = self._trunk(tok, pos, B, attn, st=st)
+        fused = None
+        if self.fuse_qkv and not num_splits and fuse:
+            fused = lambda l: self.fused_cache_attention(l, tok, st, pos, starts, B)
+        h = self._trunk(tok, pos, B, attn, st=st, fused_attn=fused)
         st.pos.add_(1)
         return h
 

@@ -249,7 +249,8 @@ class Rollout:
         def attn(l, q):
             return self._attention(l, q, st, pos, starts, n, act)
 
-        h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st)
+        fused = (lambda l: e.fused_cache_attention(l, self.tok_c[:n], st, pos, starts, n, rows=act)) if e.fuse_qkv else None
+        h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st, fused_attn=fused)
         x = e.head(h)
         if self.T > 0:
             tok, lp = fused_sample_seeded(x, self.seed, self.req_c[:n], self.cnt_c[:n], cfg.softcap, self.T)

@@ -70,6 +70,12 @@ class UVWeights:
         self.inv_freq = ((1.0 / cfg.rope_base) ** torch.linspace(0, 1, n_pairs, dtype=torch.float32)).to(self.device) \
             if n_pairs else torch.zeros(1, device=self.device)
 
+    @staticmethod
+    def qkv_ext_rows(cfg: UVConfig) -> int:
+        """Rows of the extended projection weight: q, k, v columns, then n_heads + n_kv_heads gate logits, padded to 16."""
+        n = (cfg.n_heads + 2 * cfg.n_kv_heads) * cfg.head_dim + cfg.n_heads + cfg.n_kv_heads
+        return (n + 15) // 16 * 16
+
     def _fuse(self, params: dict):
         """The reference's fuse_for_inference (model.py:289-300, 384-386) on a name -> array mapping."""
         cfg, dtype, dev = self.cfg, self.dtype, self.device
@@ -98,6 +104,17 @@ class UVWeights:
                 "attn_gate": t(params[a + "attn_gate"]).to(dtype).float().to(dev).contiguous() if cfg.gate_ch else None,
                 "xsa": torch.tanh(t(params[a + "xsa_alpha"])).to(dev).contiguous() if cfg.xsa else None,
             }
+            if dtype in (torch.bfloat16, torch.float16):
+                # Projection with the gate rows appended (decode steps): columns [q | k | v | H attention-gate logits |
+                # K value-embedding gate logits | zero padding to a multiple of 16].  The gates are linear in the same
+                # normed input (F.linear(x[..., :C], w), model.py:312, 330), so the GEMM forms their logits for free.
+                d, C_g, C_v = cfg.d_model, cfg.gate_ch, cfg.ve_gate_channels
+                ext = torch.zeros(self.qkv_ext_rows(cfg) - wqkv.size(0), d)
+                if cfg.gate_ch:
+                    ext[:cfg.n_heads, :C_g] = t(params[a + "attn_gate"]).to(dtype).float()
+                if cfg.has_ve(l):
+                    ext[cfg.n_heads:cfg.n_heads + cfg.n_kv_heads, :C_v] = t(params[a + "ve_gate"]).to(dtype).float()
+                L["wqkv_ext"] = torch.cat([wqkv.to(dtype), ext.to(dtype)]).to(dev).contiguous()
             # the four residual scalars are cast to the activation dtype before use (model.py:568-571)
             for s in ("resid_attn", "post_attn", "resid_mlp", "post_mlp"):
                 L[s] = float(torch.tensor(float(params[f"blocks.{l}.{s}"])).to(dtype).float())

@@ -38,7 +38,7 @@ def supported(q: Tensor, k_cache: Tensor) -> bool:
 
 
 def build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0,
-                    rows=None, post=None):
+                    rows=None, post=None, fuse=None):
     """Fill a uvmi_attn_args struct for these tensors.  Returns (args, keepalive): the struct holds raw pointers, so the
     caller keeps `keepalive` (and the tensors) alive until the launch has been enqueued."""
     B, H, hd = q.shape
@@ -79,13 +79,27 @@ def build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_sca
         if xsa is not None:
             assert xsa.dtype == torch.float32 and xsa.is_contiguous()
             a.post_xsa = xsa.data_ptr()
-    return a, (ws, rows)
+    f = None
+    if fuse is not None:
+        # fuse: dict(qkv (B, row) projection output, ext_col, has_gate, tok, ve_table, vocab, inv_freq, n_pairs, rope, eps, xsa_eps)
+        qkv = fuse["qkv"]
+        assert qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.dtype == q.dtype
+        f = L.AttnQkvFuse()
+        f.qkv, f.row_stride, f.ext_col, f.has_gate = qkv.data_ptr(), qkv.stride(0), int(fuse["ext_col"]), int(bool(fuse["has_gate"]))
+        ve, tok = fuse.get("ve_table"), fuse.get("tok")
+        if ve is not None:
+            assert tok is not None and tok.dtype == pos.dtype and tok.is_contiguous() and ve.is_contiguous() and ve.dtype == q.dtype
+            f.tok, f.ve_table, f.vocab, f.has_ve = tok.data_ptr(), ve.data_ptr(), int(fuse["vocab"]), 1
+        f.inv_freq, f.n_pairs, f.rope = fuse["inv_freq"].data_ptr(), int(fuse["n_pairs"]), int(bool(fuse["rope"]))
+        f.eps, f.xsa_eps = float(fuse["eps"]), float(fuse["xsa_eps"])
+        a.fuse = C.addressof(f)
+    return a, (ws, rows, f)
 
 
 def _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys=0, rows=None,
-            post=None):
+            post=None, fuse=None):
     a, keep = build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out, chunk_keys,
-                              rows, post)
+                              rows, post, fuse)
     L.check(L.lib().uvmi_decode_attn(C.byref(a), L.stream_ptr(q)), "uvmi_decode_attn")
     del keep
     return out
@@ -159,3 +173,33 @@ def decode_attention_post(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tens
         rows = rows.to(pos.dtype).contiguous()
     return _launch(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window), bool(ring), k_scale,
                    v_scale, 1, out, 0, rows, (vhat, gate, xsa, out.dtype))
+
+
+def decode_attention_fused(qkv: Tensor, H: int, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float, *,
+                           window: int, ring: bool, k_scale: Tensor, v_scale: Tensor, xsa: Tensor | None, out: Tensor,
+                           fuse: dict, rows: Tensor | None = None) -> Tensor:
+    """A decode step's attention straight from the projection output: the kernel normalises and rotates q and k of each
+    row's token, adds the value embedding to v, appends k and v (int8) to the cache at pos, attends lo..pos and applies
+    the XSA / gate epilogue (ultraviolet/model.py:302-333, kernels/fast_decode.py:291-325 of the reference in one launch).
+    qkv (B, row) holds H*64 q, K*64 k, K*64 v and, from column fuse["ext_col"], the H gate logits and K value-embedding
+    gate logits; see uvmi_attn_qkv_fuse in include/uvmi.h for the other entries of `fuse`.  The caches are written."""
+    a, keep = build_fused_args(qkv, H, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, xsa, out, fuse, rows)
+    L.check(L.lib().uvmi_decode_attn(C.byref(a), L.stream_ptr(qkv)), "uvmi_decode_attn")
+    del keep
+    return out
+
+
+def build_fused_args(qkv, H, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, xsa, out, fuse, rows=None):
+    """The uvmi_attn_args struct (and what must stay alive with it) of decode_attention_fused."""
+    L.require_cuda(qkv, k_cache, pos)
+    B = qkv.size(0)
+    q = qkv.as_strided((B, H, 64), (qkv.stride(0), 64, 1))   # the q columns, for the shape / alignment checks
+    if rows is not None:
+        rows = rows.to(pos.dtype).contiguous()
+    a, keep = build_attn_args(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window), bool(ring), k_scale,
+                              v_scale, 1, out, 0, rows, None, dict(fuse, qkv=qkv))
+    a.post_round_dtype = L.dtype_code(out.dtype)
+    if xsa is not None:
+        assert xsa.dtype == torch.float32 and xsa.is_contiguous()
+        a.post_xsa = xsa.data_ptr()
+    return a, (keep, q, xsa)
