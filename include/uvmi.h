@@ -133,9 +133,15 @@ typedef struct uvmi_attn_qkv_fuse {
   const void* tok;                         /* (B,) token ids (idx_dtype of the attention arguments), for the value embedding */
   const void* ve_table; int64_t vocab;     /* (vocab, KH, 64) value embedding in the q dtype, or NULL (has_ve = 0) */
   int has_ve;
-  const float* inv_freq; int n_pairs; int rope;
+  const float* rope_table; int rope_positions; /* uvmi_rope_table output for n_pairs = 16 (128-byte aligned) and its row count:
+                                                 every pos[b] must be below it */
+  int n_pairs; int rope;
   float eps, xsa_eps;
 } uvmi_attn_qkv_fuse;
+/* The rotation table of the fused path: out (n_positions, 2 * n_pairs) fp32, row p = cos(p * inv_freq[j]) for j <
+ * n_pairs, then sin, each rounded to round_dtype - the values uvmi_qkv_post forms per token (the reference keeps the same
+ * table as a buffer of the model, ultraviolet/model.py:198-226). */
+int uvmi_rope_table(const float* inv_freq, int n_pairs, int64_t n_positions, int round_dtype, float* out, void* stream);
 
 /* Keys attended by row b: absolute positions max(starts[b], pos[b]-window+1, 0) .. pos[b]; a row with no valid
  * key yields zeros.  fp32 accumulation; int8 caches are dequantised in registers (K scale on the score column,

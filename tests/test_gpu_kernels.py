@@ -389,3 +389,23 @@ def test_error_paths_are_loud():
     p = torch.zeros(2, dtype=torch.long, device=DEV)
     with pytest.raises(L.UvmiError):
         decode_attention(q, kc, kc, p, p, 0.1, k_scale=sc, v_scale=sc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_rope_table_matches_rounded_cos_sin(dtype):
+    """uvmi_rope_table: row p = cos(p * inv_freq) then sin(p * inv_freq), each rounded to the activation type - compared with
+    float64 cos / sin of the fp32 angle (the reference's Rotary buffers, ultraviolet/model.py:198-226): at most one unit
+    in the last place of the rounding type apart (fp32 cosf against float64), and exactly representable in that type."""
+    from ultraviolet_amd.kernels.decode_attn import rope_table
+    inv = ((1.0 / 1024.0) ** torch.linspace(0, 1, 16, dtype=torch.float32)).cuda()
+    n = 2336
+    tab = rope_table(inv, n, dtype)
+    assert tab.shape == (n, 32) and tab.dtype == torch.float32
+    assert torch.equal(tab.to(dtype).float(), tab)
+    ang = (torch.arange(n, dtype=torch.float32, device="cuda")[:, None] * inv[None, :]).double()
+    ref = torch.cat([ang.cos(), ang.sin()], 1)
+    ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -23}[dtype]
+    assert float((tab.double() - ref).abs().max()) <= ulp
+    exact = ref.float().to(dtype).float()
+    assert float((tab != exact).float().mean()) < 1e-3   # the rounding differs only where fp32 cosf lands across a tie

@@ -44,8 +44,8 @@ class AttnArgs(C.Structure):
 
 class AttnQkvFuse(C.Structure):
     _fields_ = [("qkv", C.c_void_p), ("row_stride", C.c_int64), ("ext_col", C.c_int), ("has_gate", C.c_int), ("tok", C.c_void_p),
-                ("ve_table", C.c_void_p), ("vocab", C.c_int64), ("has_ve", C.c_int), ("inv_freq", C.c_void_p), ("n_pairs", C.c_int),
-                ("rope", C.c_int), ("eps", C.c_float), ("xsa_eps", C.c_float)]
+                ("ve_table", C.c_void_p), ("vocab", C.c_int64), ("has_ve", C.c_int), ("rope_table", C.c_void_p), ("rope_positions", C.c_int),
+                ("n_pairs", C.c_int), ("rope", C.c_int), ("eps", C.c_float), ("xsa_eps", C.c_float)]
 
 
 class PrefillAttnArgs(C.Structure):
@@ -140,6 +140,7 @@ def lib() -> C.CDLL:
         L.uvmi_sched_admit.argtypes = [C.POINTER(SchedState), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_void_p]
         L.uvmi_sched_expand.argtypes = [C.POINTER(SchedState), C.c_int, C.c_int] + [C.c_void_p] * 8
+        L.uvmi_rope_table.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 
@@ -166,4 +167,4 @@ EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu",
-           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand"]
+           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_rope_table"]

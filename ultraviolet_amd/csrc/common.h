@@ -84,6 +84,13 @@ inline int dtype_bytes(int dt) {
 }
 
 // wave64 butterfly reductions (ds_bpermute based; used off the hot loops)
+// One element of the partial rotation: x cos - y sin for the first half of a pair, x cos + y sin for the second, as one
+// fma on the rounded product y sin.  Every kernel that rotates q or k goes through here, so they round alike.
+__device__ __forceinline__ float rope_rot(float x, float y, float c, float s, bool first) {
+  const float t = __fmul_rn(y, s);
+  return __builtin_fmaf(x, c, first ? -t : t);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
   return v;

@@ -52,9 +52,9 @@ struct AttnParams {
   // optional fused epilogue (Attention.post of the reference, model.py:321-333)
   const float* post_vhat; const float* post_gate; const float* post_xsa; int post_dt;
   // optional fused QKV post-processing of the row's own token (model.py:302-319, fast_decode.py:291-294, 315-317)
-  const void* f_qkv; const void* f_tok; const void* f_ve; const float* f_inv_freq;
+  const void* f_qkv; const void* f_tok; const void* f_ve; const float* f_rope_tab;
   int64_t f_sqkv, f_vocab;
-  int f_ext, f_rope, f_has_ve, f_has_gate;
+  int f_ext, f_rope, f_rope_n, f_has_ve, f_has_gate;
   float f_eps, f_xsa_eps;
 };
 
@@ -124,6 +124,37 @@ __device__ __forceinline__ float xsum32(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Butterfly reductions over the 64 lanes with the pairing order of wave_sum / wave_max (lane ^ 32, 16, 8, 4, 2, 1), so
+// that a sum formed here rounds exactly as the one in the standalone post-processing kernel; the steps use the lane-swap,
+// DPP and swizzle forms instead of six LDS permutes.
+__device__ __forceinline__ float lane_xor16(float v) {  // value of lane l ^ 16
+  return __uint_as_float((uint32_t)__builtin_amdgcn_ds_swizzle((int)__float_as_uint(v), 0x401f));
+}
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_mov_dpp((int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_xor4(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_ds_swizzle((int)__float_as_uint(v), 0x101f));
+}
+__device__ __forceinline__ float bfly_sum(float v) {
+  v = xsum32(v);
+  v = xsum16(v);
+  v += dpp_mov<0x128>(v);  // row_ror:8 == lane ^ 8 inside a row of 16
+  v += lane_xor4(v);
+  v += dpp_mov<0x4e>(v);   // quad_perm [2, 3, 0, 1] == lane ^ 2
+  v += dpp_mov<0xb1>(v);   // quad_perm [1, 0, 3, 2] == lane ^ 1
+  return v;
+}
+__device__ __forceinline__ float bfly_max(float v) {
+  v = xmax32(v);
+  v = xmax16(v);
+  v = fmaxf(v, dpp_mov<0x128>(v));
+  v = fmaxf(v, lane_xor4(v));
+  v = fmaxf(v, dpp_mov<0x4e>(v));
+  v = fmaxf(v, dpp_mov<0xb1>(v));
+  return v;
+}
+
 struct Tile {             // one 32-key super-tile as loaded from HBM (26 dwords per lane)
   uint4 kA, kB;           // key m of stream A / B, bytes 16g..16g+15
   uint32_t vA[4], vB[4];  // keys 4g+j of stream A / B, bytes 4m..4m+3
@@ -163,6 +194,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
   __shared__ float sh_post[4][80];  // epilogue operands of the item whose first wave this is: v_hat[64], gate[8], xsa[8]
   __shared__ float sh_cur[FUSE ? 4 : 1][72];  // own key of that item: score per head [8], dequantised v [64]
+  __shared__ __attribute__((aligned(16))) uint16_t sh_q[FUSE ? 4 : 1][8][64];  // the item's q as fp16 operand words
+  __shared__ float sh_qs[FUSE ? 4 : 1][8];                                      // and their sum per head
+  __shared__ float sh_kq[FUSE ? 4 : 1][64];   // the own key's int8 codes (as floats), for its score against every head
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wsub = wave % WPR;
@@ -184,17 +218,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   // (no branch around the loads: lanes of absent heads read head G-1 and are masked to zero when the operands are
   // formed, which keeps the control flow, and with it every row-derived scalar, wave-uniform)
   const uint32_t qmask = head < G ? 0xffffffffu : 0u;
-  const uint16_t* qp = FUSE ? (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv + (h * G + (head < G ? head : G - 1)) * 64 + 16 * g
+  // (FUSE: q is normalised and rotated once per item, by its first wave, eight dims per lane - lane (hh, cc) = dims
+  // 8cc..8cc+7 of head hh, the standalone post-processing kernel's layout and reduction order - and reaches the operand
+  // layout of every wave of the item through LDS)
+  const int hh = lane >> 3, cc = lane & 7;
+  const uint16_t* qp = FUSE ? (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv + (h * G + (hh < G ? hh : G - 1)) * 64 + 8 * cc
                             : (const uint16_t*)P.q + (int64_t)b * P.sqb + (int64_t)(h * G + (head < G ? head : G - 1)) * P.sqh + 16 * g;
-  const uint4 qw0 = *(const uint4*)qp, qw1 = *(const uint4*)(qp + 8);
-  // FUSE: the row's gate logits go out with q (the raw k, v and value-embedding row are read by the item's first wave
-  // when it forms the own key: holding them from here on would cost a wave slot per SIMD)
-  uint16_t glog = 0, vlog = 0;
+  const uint4 qw0 = *(const uint4*)qp, qw1 = FUSE ? qw0 : *(const uint4*)(qp + 8);
+  // FUSE: the row's gate logits and its raw k / v go out with q.  k and v are read one dim per lane: the item's first wave
+  // takes k, its second wave v (a lone wave takes both)
+  constexpr int VW = WPR > 1 ? 1 : 0;  // the wave of an item that forms the own value (the first wave forms the own key)
+  uint16_t glog = 0, vlog = 0, raw_a = 0, raw_v = 0;
   int64_t own_tok = 0;
   if constexpr (FUSE) {
     const uint16_t* rowp = (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv;
     glog = rowp[P.f_ext + (P.f_has_gate ? h * G + (head < G ? head : G - 1) : 0)];
     vlog = rowp[P.f_ext + P.H + h];
+    raw_a = rowp[(P.H + (WPR > 1 && wsub == VW ? P.KH : 0) + h) * 64 + lane];
+    if (WPR == 1) raw_v = rowp[(P.H + P.KH + h) * 64 + lane];
     own_tok = P.f_has_ve ? (int64_t)load_idx32(P.f_tok, P.idx64, b) : 0;
     own_tok = own_tok < 0 ? 0 : (own_tok >= P.f_vocab ? P.f_vocab - 1 : own_tok);
   }
@@ -209,6 +250,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   const float* px_src = has_post && P.post_xsa ? P.post_xsa + hsafe : anyf;
   const float pv_val = *pv_src, pg_val = *pg_src, px_val = *px_src;
   const RowPlan rp = plan_row(P, b, FUSE);
+  // FUSE: the row of the rotation table (cos / sin of the row's position per frequency, already rounded to the activation
+  // type): prep_q reads its 32 values as scalars, the lane that owns dim d of the own key reads its own pair
+  const int rope_row = rp.pc < 0 ? 0 : (rp.pc < P.f_rope_n ? rp.pc : P.f_rope_n - 1);
   const bool live = live_item && sid < rp.nsplit;
   if (WPR == 1 && !live) return;
   const int s0 = rp.a0 + sid * rp.chunk;
@@ -222,62 +266,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   const uint32_t mA = strm == 0 ? qmask : 0u, mB = strm == 0 ? 0u : qmask;
   h8 QA0, QA1, QB0, QB1;
   float cinit;
-  // helpers of the fused path: 16 values of the activation type <-> fp32, rounding to the activation type, RMS norm over
-  // the 64 dims of a head (4 lane groups) and the partial rotation (dims 0..15 pair with 16..31: lane groups 0 and 1)
-  auto unpack16 = [&](const uint4& a, const uint4& b2, float (&x)[16]) {
-    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b2.x, b2.y, b2.z, b2.w};
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      if (QDT == UVMI_BF16) { x[2 * i] = __uint_as_float(w[i] << 16); x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
-      else { x[2 * i] = half_bits_to_float(w[i] & 0xffff); x[2 * i + 1] = half_bits_to_float(w[i] >> 16); }
-    }
-  };
   auto rq = [&](float v) -> float { return QDT == UVMI_BF16 ? bf16_to_float(float_to_bf16(v)) : (float)(half_t)v; };
-  float rcs[16], rsn[16];  // cos / sin of the row's position per frequency (wave-uniform, rounded to the activation type)
-  auto norm_rope = [&](float (&x)[16]) {
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) ss += x[i] * x[i];
-    ss = xsum32(xsum16(ss));
-    const float rs = rsqrtf(ss * (1.0f / 64.0f) + P.f_eps);
-#pragma unroll
-    for (int i = 0; i < 16; i++) x[i] = rq(x[i] * rs);
-    if (P.f_rope) {
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        // the partner dim lives in the neighbouring lane group: after the swap r[0] holds groups (0, 0, 2, 2) and r[1]
-        // groups (1, 1, 3, 3) of x[i]
-        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x[i]), __float_as_uint(x[i]), false, false);
-        const float y = __uint_as_float((g & 1) ? r[0] : r[1]);
-        if (g == 0) x[i] = rq(x[i] * rcs[i] - y * rsn[i]);
-        else if (g == 1) x[i] = rq(y * rsn[i] + x[i] * rcs[i]);
-      }
-    }
-  };
+  const int iw = wave - wsub;  // LDS slot of the item: its first wave
   uint32_t qr[8];
+  float qsum;
+  auto set_q = [&]() {
+    QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA); QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
+    QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB); QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
+    cinit = qmask ? -1152.0f * qsum : 0.f;
+  };
+  // unfused: q arrives normalised and rotated, 16 dims per lane in the operand layout
   auto prep_q = [&]() {
-    float qsum = 0.f;
-    uint32_t w[8] = {qw0.x, qw0.y, qw0.z, qw0.w, qw1.x, qw1.y, qw1.z, qw1.w};
-    if constexpr (FUSE) {
-      if (P.f_rope) {
-        const float th = (float)rp.pc * P.f_inv_freq[m];
-        const float cl = rq(cosf(th)), sl = rq(sinf(th));
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-          rcs[j] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(cl), j));
-          rsn[j] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(sl), j));
-        }
-      }
-      float x[16];
-      unpack16(qw0, qw1, x);
-      norm_rope(x);
-#pragma unroll
-      for (int i = 0; i < 8; i++) {  // back to the packed activation type: the conversion below is shared with the unfused path
-        const uint32_t lo16 = QDT == UVMI_BF16 ? float_to_bf16(x[2 * i]) : float_to_half_bits(x[2 * i]);
-        const uint32_t hi16 = QDT == UVMI_BF16 ? float_to_bf16(x[2 * i + 1]) : float_to_half_bits(x[2 * i + 1]);
-        w[i] = lo16 | (hi16 << 16);
-      }
-    }
+    const uint32_t w[8] = {qw0.x, qw0.y, qw0.z, qw0.w, qw1.x, qw1.y, qw1.z, qw1.w};
+    qsum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       float f0, f1;
@@ -288,101 +289,117 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       qsum += half_bits_to_float(l16) + half_bits_to_float(h16);
     }
     qsum = xsum32(xsum16(qsum));  // all 64 dims of this head
-    QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA); QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
-    QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB); QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
-    cinit = qmask ? -1152.0f * qsum : 0.f;
+    set_q();
+  };
+  // FUSE, first wave of the item: QK-norm and partial rotation of the 8 heads (uvmi_qkv_post's arithmetic: RMS over the
+  // head's 8 lanes by xor 1, 2, 4; rotation partner dims 8cc.. <-> 8(cc ^ 2)..), then the fp16 operand words and their
+  // sum per head go to LDS
+  auto prep_q_item = [&](const float4& c0, const float4& c1, const float4& s0, const float4& s1) {
+    const uint32_t w[4] = {qw0.x, qw0.y, qw0.z, qw0.w};
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      if (QDT == UVMI_BF16) { x[2 * i] = __uint_as_float(w[i] << 16); x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+      else { x[2 * i] = half_bits_to_float(w[i] & 0xffff); x[2 * i + 1] = half_bits_to_float(w[i] >> 16); }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+    ss += dpp_mov<0xb1>(ss); ss += dpp_mov<0x4e>(ss); ss += lane_xor4(ss);
+    const float rs = rsqrtf(ss * (1.0f / 64.0f) + P.f_eps);
+#pragma unroll
+    for (int j = 0; j < 8; j++) x[j] = rq(x[j] * rs);
+    if (P.f_rope) {  // 16 pairs: dims 0..15 (cc 0, 1) with 16..31 (cc 2, 3); frequency index of dim 8cc + j is 8(cc & 1) + j
+      const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w}, sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+      const bool first = cc < 2, rot = cc < 4;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const float v = rq(rope_rot(x[j], dpp_mov<0x4e>(x[j]), cs[j], sn[j], first));
+        x[j] = rot ? v : x[j];
+      }
+    }
+    uint32_t o[4];
+    float qs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint16_t l16 = float_to_half_bits(x[2 * i]), h16 = float_to_half_bits(x[2 * i + 1]);
+      o[i] = (uint32_t)l16 | ((uint32_t)h16 << 16);
+      qs += half_bits_to_float(l16) + half_bits_to_float(h16);
+    }
+    qs += dpp_mov<0xb1>(qs); qs += dpp_mov<0x4e>(qs); qs += lane_xor4(qs);
+    *(uint4*)&sh_q[iw][hh][8 * cc] = uint4{o[0], o[1], o[2], o[3]};
+    if (cc == 0) sh_qs[iw][hh] = qs;
+  };
+  // FUSE, every wave of the item, after the barrier that follows prep_q_item: its operand words from LDS
+  auto fetch_q = [&]() {
+    const uint4 o0 = *(const uint4*)&sh_q[iw][head][16 * g], o1 = *(const uint4*)&sh_q[iw][head][16 * g + 8];
+    qr[0] = o0.x; qr[1] = o0.y; qr[2] = o0.z; qr[3] = o0.w; qr[4] = o1.x; qr[5] = o1.y; qr[6] = o1.z; qr[7] = o1.w;
+    qsum = sh_qs[iw][head];
+    set_q();
   };
 
-  // FUSE, first wave of the item: k (norm, rotation), v (value embedding), int8 append at the row's position, and what the
-  // end of the kernel needs from them - the own key's score per head and dequantised value (merged into the softmax after
-  // the streamed range), v_hat and the gate for the epilogue - parked in LDS.  Arithmetic and roundings follow the
-  // standalone post-processing kernel (uvmi_qkv_post).
-  constexpr int VW = WPR > 1 ? 1 : 0;  // the wave of an item that forms the own value (the first wave forms the own key)
-  const int iw = wave - wsub;          // LDS slot of the item: its first wave
-  // quantise 16 values per lane of a 64-dim row spread over the 4 lane groups (the arithmetic of the standalone
-  // quantizer: fp16 scale, IEEE division, round half to even, clamp); returns the scale as fp32
-  auto quant = [&](const float (&x)[16], float (&qv)[16], uint16_t& sb) -> float {
-    float am = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) am = fmaxf(am, fabsf(x[i]));
-    am = xmax32(xmax16(am));
+  // FUSE, the row's own token.  The item's first wave forms k (norm, rotation), its second wave v (value embedding); both
+  // work one dim per lane with the arithmetic, roundings and reduction order of the standalone post-processing kernel
+  // (uvmi_qkv_post), append the int8 row at the row's position, and park in LDS what the end of the kernel needs: the own
+  // key's score per head and dequantised value (merged into the softmax after the streamed range), v_hat and the gates.
+  auto cvt_in = [&](uint16_t w) -> float { return QDT == UVMI_BF16 ? bf16_to_float(w) : half_bits_to_float(w); };
+  // int8 code (as a float) of this lane's element of a 64-dim row, and the row's fp16 scale: fp16 scale, IEEE division,
+  // round half to even, clamp - the standalone quantizer's arithmetic
+  auto quant1 = [&](float x, uint16_t& sb) -> float {
+    const float am = bfly_max(fabsf(x));
     sb = float_to_half_bits(__fdiv_rn(am, 127.0f));
     const float sf = fmaxf(half_bits_to_float(sb), 1e-30f);
-#pragma unroll
-    for (int i = 0; i < 16; i++) qv[i] = fminf(fmaxf(__builtin_rintf(__fdiv_rn(x[i], sf)), -127.0f), 127.0f);
-    return half_bits_to_float(sb);
+    return fminf(fmaxf(__builtin_rintf(__fdiv_rn(x, sf)), -127.0f), 127.0f);
   };
-  auto pack = [&](const float (&qv)[16]) -> uint4 {
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-      w[i] = ((uint32_t)(int)qv[4 * i] & 0xffu) | (((uint32_t)(int)qv[4 * i + 1] & 0xffu) << 8) | (((uint32_t)(int)qv[4 * i + 2] & 0xffu) << 16) |
-             (((uint32_t)(int)qv[4 * i + 3] & 0xffu) << 24);
-    return uint4{w[0], w[1], w[2], w[3]};
-  };
-  // own_k (first wave of the item): k -> norm, rotation -> int8 append; the own key's score per head (q as the fp16
-  // operand holds it . k_int8 * k scale, in the units of the streamed scores) and the gate values go to LDS.
-  auto own_k = [&](const uint4& a0, const uint4& a1) {
-    float kx[16], kq[16];
-    uint16_t sbk;
-    unpack16(a0, a1, kx);
-    norm_rope(kx);
-    const float ksf = quant(kx, kq, sbk);
-    const int slot = P.ring ? rp.pc % P.S : rp.pc;
-    if (slot < P.S && m == 0) {  // one lane per group writes its 16 bytes of the row; lane 0 the scale
-      *(uint4*)((int8_t*)P.kc + (int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + 16 * g) = pack(kq);
-      if (g == 0) ((uint16_t*)P.ks)[(int64_t)rp.cb * P.ssb + (int64_t)h * P.ssh + slot] = sbk;
+  auto own_k = [&](uint16_t raw, float kcs, float ksn) {
+    float k = cvt_in(raw);
+    const float rs = rsqrtf(bfly_sum(k * k) * (1.0f / 64.0f) + P.f_eps);
+    k = rq(k * rs);
+    if (P.f_rope) {
+      const float kr = rq(rope_rot(k, lane_xor16(k), kcs, ksn, lane < 16));
+      k = lane < 32 ? kr : k;
     }
+    uint16_t sbk;
+    const float kq = quant1(k, sbk);
+    const int slot = P.ring ? rp.pc % P.S : rp.pc;
+    if (slot < P.S) {
+      ((int8_t*)P.kc)[(int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + lane] = (int8_t)(int)kq;
+      if (lane == 0) ((uint16_t*)P.ks)[(int64_t)rp.cb * P.ssb + (int64_t)h * P.ssh + slot] = sbk;
+    }
+    // score of the own key against every head: q as the fp16 operand holds it (lane (head, g): dims 16g..16g+15) . the
+    // int8 codes * k scale, in the units of the streamed scores
+    sh_kq[iw][lane] = kq;
+    __builtin_amdgcn_wave_barrier();
     float dq = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; i++)
-      dq += half_bits_to_float(qr[i] & 0xffff) * kq[2 * i] + half_bits_to_float(qr[i] >> 16) * kq[2 * i + 1];
-    dq = xsum32(xsum16(dq)) * ksf;
+    for (int i = 0; i < 4; i++) {
+      const float4 c4 = *(const float4*)&sh_kq[iw][16 * g + 4 * i];
+      dq += half_bits_to_float(qr[2 * i] & 0xffff) * c4.x + half_bits_to_float(qr[2 * i] >> 16) * c4.y;
+      dq += half_bits_to_float(qr[2 * i + 1] & 0xffff) * c4.z + half_bits_to_float(qr[2 * i + 1] >> 16) * c4.w;
+    }
+    dq = xsum32(xsum16(dq)) * half_bits_to_float(sbk);
     if (lane < 8) {
       sh_cur[iw][lane] = dq;
-      const float lg = QDT == UVMI_BF16 ? bf16_to_float(glog) : half_bits_to_float(glog);
-      sh_post[iw][64 + lane] = P.f_has_gate ? rq(2.0f * rq(1.0f / (1.0f + __expf(-lg)))) : 1.0f;
+      sh_post[iw][64 + lane] = P.f_has_gate ? rq(2.0f * rq(1.0f / (1.0f + __expf(-cvt_in(glog))))) : 1.0f;
     }
     if (lane >= 8 && lane < 16) sh_post[iw][64 + lane] = px_val;
   };
-  // own_v (second wave of the item when there is one): v (+ value embedding) -> int8 append; the dequantised own value
-  // and v_hat for the XSA epilogue go to LDS.  Arithmetic and roundings follow uvmi_qkv_post.
-  auto own_v = [&](const uint4& a0, const uint4& a1, const uint4& e0, const uint4& e1) {
-    float vx[16], vq[16];
-    uint16_t sbv;
-    unpack16(a0, a1, vx);
+  auto own_v = [&](uint16_t raw, uint16_t raw_ve) {
+    float v = cvt_in(raw);
     if (P.f_has_ve) {
-      float ve[16];
-      unpack16(e0, e1, ve);
-      const float dot = QDT == UVMI_BF16 ? bf16_to_float(vlog) : half_bits_to_float(vlog);
-      const float gv = rq(2.0f * rq(1.0f / (1.0f + __expf(-dot))));
-#pragma unroll
-      for (int i = 0; i < 16; i++) vx[i] = rq(vx[i] + rq(gv * ve[i]));
+      const float gv = rq(2.0f * rq(1.0f / (1.0f + __expf(-cvt_in(vlog)))));
+      v = rq(v + rq(gv * cvt_in(raw_ve)));
     }
-    float vv2 = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) vv2 += vx[i] * vx[i];
-    const float nv = fmaxf(sqrtf(xsum32(xsum16(vv2))), P.f_xsa_eps);
-    const float vsf = quant(vx, vq, sbv);
+    const float nv = fmaxf(sqrtf(bfly_sum(v * v)), P.f_xsa_eps);
+    uint16_t sbv;
+    const float vq = quant1(v, sbv);
     const int slot = P.ring ? rp.pc % P.S : rp.pc;
-    if (m == 0) {
-      if (slot < P.S) {
-        *(uint4*)((int8_t*)P.vc + (int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + 16 * g) = pack(vq);
-        if (g == 0) ((uint16_t*)P.vs)[(int64_t)rp.cb * P.stb + (int64_t)h * P.sth + slot] = sbv;
-      }
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        sh_cur[iw][8 + 16 * g + i] = vsf * vq[i];
-        sh_post[iw][16 * g + i] = vx[i] / nv;
-      }
+    if (slot < P.S) {
+      ((int8_t*)P.vc)[(int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + lane] = (int8_t)(int)vq;
+      if (lane == 0) ((uint16_t*)P.vs)[(int64_t)rp.cb * P.stb + (int64_t)h * P.sth + slot] = sbv;
     }
-  };
-  // raw inputs of own_k / own_v: every lane of a 16-lane group g reads dims 16g..16g+15 of the row's k (first wave) or v
-  // and value-embedding row (second wave); requested right after the first tile, used after q is ready
-  const uint16_t* own_row = (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv;
-  auto own_src = [&](bool v_part) -> const uint16_t* { return own_row + (P.H + (v_part ? P.KH : 0) + h) * 64 + 16 * g; };
-  auto own_ve = [&](const uint16_t* fallback) -> const uint16_t* {
-    return P.f_has_ve ? (const uint16_t*)P.f_ve + (own_tok * P.KH + h) * 64 + 16 * g : fallback;
+    sh_cur[iw][8 + lane] = half_bits_to_float(sbv) * vq;
+    sh_post[iw][lane] = v / nv;
   };
 
   AttnState st;
@@ -526,35 +543,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
       if (P.ring) while (sl >= S) sl -= S;
       return sl;
     };
+    // What the fused prologue still needs from memory - the rotation table row (q: this lane's 8 frequencies; own key: the
+    // lane's pair) and the value-embedding element - is requested before the tiles: loads complete in order, so anything
+    // requested after a tile could only be used once that tile has arrived.
+    // (unconditional loads from a select of addresses - the row itself when a feature is off - keep this stretch free of
+    // branches, which would make the compiler wait for the loads before it requests the tiles)
+    float kcs = 1.f, ksn = 0.f;
+    uint16_t raw_ve = 0;
+    float4 rc0 = float4{1.f, 1.f, 1.f, 1.f}, rc1 = rc0, rs0 = float4{0.f, 0.f, 0.f, 0.f}, rs1 = rs0;
+    if constexpr (FUSE) {
+      const uint16_t* own_row = (const uint16_t*)P.f_qkv + (int64_t)b * P.f_sqkv;
+      const float* tr = P.f_rope ? P.f_rope_tab + (int64_t)rope_row * 32 : (const float*)own_row;
+      const float* tq = tr + 8 * (cc & 1);
+      rc0 = *(const float4*)tq; rc1 = *(const float4*)(tq + 4); rs0 = *(const float4*)(tq + 16); rs1 = *(const float4*)(tq + 20);
+      kcs = tr[lane & 15]; ksn = tr[16 + (lane & 15)];
+      raw_ve = (P.f_has_ve ? (const uint16_t*)P.f_ve + (own_tok * P.KH + h) * 64 : own_row)[lane];
+    }
     // The first tile is requested unconditionally (a wave without a pipelined tile reads slot 0 and drops it; the
     // descriptor bounds the access), so that the q conversion - and, on the fused path, the forming of the row's own key -
-    // follows it on every path and waits for q only.  (Requesting two tiles here was measured: the second tile's
-    // registers, live across the own-key arithmetic, push the fused kernel into spills.)
+    // follows it on every path and waits for q only.  (Requesting two tiles here was measured on the fused path, with no
+    // spills: 20.5 us against 19.2 us per launch on ~2000 rows x ~215 keys - all waves' first two tiles then leave in
+    // one burst of more than half the launch's bytes.)
     Tile TA, TB;
     load_tile(slot, TA);
-    uint4 aw0, aw1, ew0, ew1;
-    if constexpr (FUSE) {
-      const uint16_t* ap = own_src(WPR > 1 && wsub == VW);
-      const uint16_t* ep = own_ve(ap);
-      aw0 = *(const uint4*)ap; aw1 = *(const uint4*)(ap + 8);
-      ew0 = *(const uint4*)ep; ew1 = *(const uint4*)(ep + 8);
-    }
     __builtin_amdgcn_sched_barrier(0);
-    prep_q();
     if constexpr (!FUSE) {
+      prep_q();
       if (wsub == 0) {
         sh_post[wave][lane] = pv_val;
         if (lane < 16) sh_post[wave][64 + lane] = lane < 8 ? pg_val : px_val;  // lanes 8..15 carry head lane - 8 too
       }
-    } else if (live && rp.pc >= 0) {
-      if (WPR > 1) {
-        if (wsub == 0) own_k(aw0, aw1);
-        else if (wsub == VW) own_v(aw0, aw1, ew0, ew1);
-      } else {  // one wave per item forms both; the value's inputs are read here
-        own_k(aw0, aw1);
-        const uint16_t* vp = own_src(true);
-        const uint16_t* ep = own_ve(vp);
-        own_v(*(const uint4*)vp, *(const uint4*)(vp + 8), *(const uint4*)ep, *(const uint4*)(ep + 8));
+    } else {
+      const bool own = live && rp.pc >= 0;
+      if (wsub == 0) prep_q_item(rc0, rc1, rs0, rs1);
+      else if (WPR > 1 && wsub == VW && own) own_v(raw_a, raw_ve);  // needs no q: done while the first wave prepares it
+      if (WPR > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+      fetch_q();
+      if (own && wsub == 0) {
+        own_k(raw_a, kcs, ksn);
+        if (WPR == 1) own_v(raw_v, raw_ve);
       }
     }
     if (has) {
@@ -983,19 +1010,20 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   P.scale_log2 = a->scale * LOG2E;
   P.ws_o = P.ws_m = P.ws_l = nullptr;
   P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa; P.post_dt = a->post_round_dtype;
-  P.f_qkv = nullptr;
+  P.f_qkv = nullptr; P.f_rope_tab = nullptr; P.f_rope_n = 1; P.f_rope = 0;
   if (const uvmi_attn_qkv_fuse* f = a->fuse) {
     UVMI_REQUIRE(mfma_ok(a) && a->num_splits == 1, UVMI_EUNSUPPORTED,
                  "uvmi_decode_attn: fused QKV post-processing needs the MFMA kernel (head_dim 64, int8 cache, aligned rows) and num_splits == 1");
     UVMI_REQUIRE(a->out_dtype == a->q_dtype, UVMI_EUNSUPPORTED, "uvmi_decode_attn: fused QKV post-processing writes the q dtype");
     UVMI_REQUIRE(f->qkv && ((uintptr_t)f->qkv % 16) == 0 && f->row_stride % 8 == 0 && f->ext_col >= (a->H + 2 * a->KH) * 64 &&
                      f->row_stride >= f->ext_col + a->H + a->KH, UVMI_EINVAL, "uvmi_decode_attn: bad fused qkv layout");
-    UVMI_REQUIRE(!f->rope || (f->n_pairs == 16 && f->inv_freq), UVMI_EUNSUPPORTED, "uvmi_decode_attn: fused rotation needs n_pairs == 16");
+    UVMI_REQUIRE(!f->rope || (f->n_pairs == 16 && f->rope_table && f->rope_positions > 0 && ((uintptr_t)f->rope_table % 128) == 0), UVMI_EUNSUPPORTED,
+                 "uvmi_decode_attn: fused rotation needs n_pairs == 16 and a 128-byte aligned rope_table");
     UVMI_REQUIRE(!f->has_ve || (f->ve_table && f->tok && f->vocab > 0 && ((uintptr_t)f->ve_table % 16) == 0), UVMI_EINVAL,
                  "uvmi_decode_attn: fused value embedding needs ve_table, tok and vocab");
     P.f_qkv = f->qkv; P.f_sqkv = f->row_stride; P.f_ext = f->ext_col; P.f_has_gate = f->has_gate ? 1 : 0;
     P.f_tok = f->tok; P.f_ve = f->ve_table; P.f_vocab = f->vocab; P.f_has_ve = f->has_ve ? 1 : 0;
-    P.f_inv_freq = f->inv_freq; P.f_rope = f->rope ? 1 : 0; P.f_eps = f->eps; P.f_xsa_eps = f->xsa_eps;
+    P.f_rope_tab = f->rope_table; P.f_rope_n = f->rope ? f->rope_positions : 1; P.f_rope = f->rope ? 1 : 0; P.f_eps = f->eps; P.f_xsa_eps = f->xsa_eps;
     P.post_vhat = nullptr; P.post_gate = nullptr;
   }
   if (a->post_vhat && !a->fuse) {

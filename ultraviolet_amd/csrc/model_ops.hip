@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
         for (int j = 0; j < 8; j++) y[j] = __shfl_xor(x[j], pl, 64);  // partner chunk: c <-> c ^ pl inside the head
         if (rot) {
 #pragma unroll
-          for (int j = 0; j < 8; j++) x[j] = first ? round_t<DT>(x[j] * cs[j] - y[j] * sn[j]) : round_t<DT>(y[j] * sn[j] + x[j] * cs[j]);
+          for (int j = 0; j < 8; j++) x[j] = round_t<DT>(rope_rot(x[j], y[j], cs[j], sn[j], first));
         }
       }
       if (h < A.H) {
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       k = round_t<DT>(k * rs);
       if (A.rope) {
         const float other = __shfl_xor(k, np_, 64);
-        if (rot1) k = lane < np_ ? round_t<DT>(k * cs1 - other * sn1) : round_t<DT>(other * sn1 + k * cs1);
+        if (rot1) k = round_t<DT>(rope_rot(k, other, cs1, sn1, lane < np_));
       }
     }
     float v = elem<DT>::ld(A.qkv, base + (A.H + A.KH + kh) * 64 + lane);
@@ -401,6 +401,31 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   const dim3 grid((unsigned)((a->n + 3) / 4)), blk(256);
   dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
   UVMI_CHECK_LAUNCH("uvmi_qkv_post");
+  return UVMI_OK;
+}
+
+// cos / sin of position * inv_freq per frequency, rounded to the activation type as the rotation applies them
+// (round_t(cosf(th)) above), as an fp32 table: row p holds cos[0..n_pairs) then sin[0..n_pairs)
+template <int DT>
+__global__ __launch_bounds__(256) void rope_table_kernel(const float* __restrict__ inv_freq, int n_pairs, int64_t n_pos, float* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_pos * n_pairs) return;
+  const int64_t p = i / n_pairs;
+  const int j = (int)(i % n_pairs);
+  const float th = (float)p * inv_freq[j];
+  out[p * 2 * n_pairs + j] = round_t<DT>(cosf(th));
+  out[p * 2 * n_pairs + n_pairs + j] = round_t<DT>(sinf(th));
+}
+
+extern "C" int uvmi_rope_table(const float* inv_freq, int n_pairs, int64_t n_positions, int round_dtype, float* out, void* stream) {
+  UVMI_REQUIRE(inv_freq && out, UVMI_EINVAL, "uvmi_rope_table: null pointer");
+  UVMI_REQUIRE(n_pairs > 0 && n_positions >= 0 && is_float_dtype(round_dtype), UVMI_EINVAL, "uvmi_rope_table: bad arguments");
+  if (n_positions == 0) return UVMI_OK;
+  const dim3 grid((unsigned)((n_positions * n_pairs + 255) / 256)), blk(256);
+  dispatch_dt(round_dtype, [&](auto DT) {
+    hipLaunchKernelGGL((rope_table_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, inv_freq, n_pairs, n_positions, out);
+  });
+  UVMI_CHECK_LAUNCH("uvmi_rope_table");
   return UVMI_OK;
 }
 

@@ -16,7 +16,8 @@ import torch
 from torch import Tensor
 
 from .. import _lib as L
-from ..kernels.decode_attn import build_attn_args, build_fused_args, decode_attention, decode_attention_fused, decode_attention_post
+from ..kernels.decode_attn import (build_attn_args, build_fused_args, decode_attention, decode_attention_fused, decode_attention_post,
+                                   rope_table)
 from ..kernels.varlen_attn import packed_attention
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
@@ -86,6 +87,7 @@ class UVEngine:
         # post-processing to the attention kernel (one launch less per layer)
         self.fuse_qkv = dt in (torch.bfloat16, torch.float16) and cfg.n_heads // cfg.n_kv_heads <= 8 and cfg.n_pairs in (0, 16)
         self.qkvx_keep = None
+        self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
         self.pf_ws = torch.empty(L.lib().uvmi_prefill_attn_workspace_bytes(n), dtype=torch.uint8, device=dev)  # fails now if the library is missing
@@ -170,13 +172,23 @@ class UVEngine:
         S = st.k[l].size(2)
         return self.fuse_qkv and S % 32 == 0 and S >= 32
 
-    def _fuse_dict(self, l: int, tok: Tensor) -> dict:
+    def rope_table(self, n_positions: int) -> Tensor:
+        """cos / sin of every position below n_positions in the activation type's rounding, built once per size."""
+        t = self._rope_tabs.get(n_positions)
+        if t is None:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("the rotation table must exist before a graph is captured: call rope_table(state.max_len) first")
+            t = self._rope_tabs[n_positions] = rope_table(self.w.inv_freq, n_positions, self.dtype)
+        return t
+
+    def _fuse_dict(self, l: int, tok: Tensor, st: KVState) -> dict:
         cfg = self.cfg
         glob = cfg.is_global(l)
         has_ve = cfg.has_ve(l)
+        rope = ((not glob) or cfg.global_rope) and cfg.n_pairs > 0
         return dict(ext_col=(cfg.n_heads + 2 * cfg.n_kv_heads) * cfg.head_dim, has_gate=cfg.gate_ch > 0, tok=tok if has_ve else None,
-                    ve_table=self.w.value_embed if has_ve else None, vocab=cfg.vocab_size, inv_freq=self.w.inv_freq, n_pairs=cfg.n_pairs,
-                    rope=((not glob) or cfg.global_rope) and cfg.n_pairs > 0, eps=self.eps, xsa_eps=cfg.xsa_eps)
+                    ve_table=self.w.value_embed if has_ve else None, vocab=cfg.vocab_size, rope_table=self.rope_table(st.max_len) if rope else None,
+                    n_pairs=cfg.n_pairs, rope=rope, eps=self.eps, xsa_eps=cfg.xsa_eps)
 
     def fused_cache_attention(self, l: int, tok: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
         """Decode attention of layer l straight from buf qkvx (the extended projection of the n rows): QK-norm, rotation,
@@ -186,7 +198,7 @@ class UVEngine:
         out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
         decode_attention_fused(b["qkvx"][:n], cfg.n_heads, st.k[l], st.v[l], pos, starts, cfg.attn_scale, window=0 if glob else cfg.window,
                                ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], xsa=W["xsa"], out=out,
-                               fuse=self._fuse_dict(l, tok), rows=rows)
+                               fuse=self._fuse_dict(l, tok, st), rows=rows)
 
     def fused_attention_args(self, l: int, qkvx: Tensor, tok: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int,
                              rows: Tensor | None = None):
@@ -197,7 +209,7 @@ class UVEngine:
         glob = cfg.is_global(l)
         out = b["zg"][:n].view(n, cfg.n_heads, cfg.head_dim)
         return build_fused_args(qkvx[:n], cfg.n_heads, st.k[l], st.v[l], pos, starts, cfg.attn_scale, 0 if glob else cfg.window, not glob,
-                                st.k_scale[l], st.v_scale[l], W["xsa"], out, self._fuse_dict(l, tok), rows)
+                                st.k_scale[l], st.v_scale[l], W["xsa"], out, self._fuse_dict(l, tok, st), rows)
 
     def cache_attention_args(self, l: int, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None):
         """The uvmi_attn_args struct cache_attention would launch for layer l on the engine's buffers (fused path only):

@@ -81,7 +81,7 @@ def build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_sca
             a.post_xsa = xsa.data_ptr()
     f = None
     if fuse is not None:
-        # fuse: dict(qkv (B, row) projection output, ext_col, has_gate, tok, ve_table, vocab, inv_freq, n_pairs, rope, eps, xsa_eps)
+        # fuse: dict(qkv (B, row) projection output, ext_col, has_gate, tok, ve_table, vocab, rope_table, n_pairs, rope, eps, xsa_eps)
         qkv = fuse["qkv"]
         assert qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.dtype == q.dtype
         f = L.AttnQkvFuse()
@@ -90,7 +90,11 @@ def build_attn_args(q, k_cache, v_cache, pos, starts, scale, window, ring, k_sca
         if ve is not None:
             assert tok is not None and tok.dtype == pos.dtype and tok.is_contiguous() and ve.is_contiguous() and ve.dtype == q.dtype
             f.tok, f.ve_table, f.vocab, f.has_ve = tok.data_ptr(), ve.data_ptr(), int(fuse["vocab"]), 1
-        f.inv_freq, f.n_pairs, f.rope = fuse["inv_freq"].data_ptr(), int(fuse["n_pairs"]), int(bool(fuse["rope"]))
+        f.n_pairs, f.rope = int(fuse["n_pairs"]), int(bool(fuse["rope"]))
+        if f.rope:  # (positions, 2 * n_pairs) fp32 from rope_table(): every pos must lie inside it
+            tab = fuse["rope_table"]
+            assert tab.dtype == torch.float32 and tab.is_contiguous() and tab.dim() == 2 and tab.size(1) == 2 * f.n_pairs
+            f.rope_table, f.rope_positions = tab.data_ptr(), tab.size(0)
         f.eps, f.xsa_eps = float(fuse["eps"]), float(fuse["xsa_eps"])
         a.fuse = C.addressof(f)
     return a, (ws, rows, f)
@@ -173,6 +177,17 @@ def decode_attention_post(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tens
         rows = rows.to(pos.dtype).contiguous()
     return _launch(q, k_cache, v_cache, pos.contiguous(), starts.contiguous(), float(scale), int(window), bool(ring), k_scale,
                    v_scale, 1, out, 0, rows, (vhat, gate, xsa, out.dtype))
+
+
+def rope_table(inv_freq: Tensor, n_positions: int, round_dtype: torch.dtype) -> Tensor:
+    """(n_positions, 2 * n_pairs) fp32: cos(p * inv_freq) then sin(p * inv_freq), each rounded to round_dtype - the
+    rotation table the fused decode path reads (the reference's Rotary buffers, ultraviolet/model.py:198-226)."""
+    assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and inv_freq.is_cuda
+    out = torch.empty(n_positions, 2 * inv_freq.numel(), dtype=torch.float32, device=inv_freq.device)
+    rc = L.lib().uvmi_rope_table(inv_freq.data_ptr(), inv_freq.numel(), n_positions, L.dtype_code(round_dtype), out.data_ptr(),
+                                 L.stream_ptr(inv_freq))
+    L.check(rc, "uvmi_rope_table")
+    return out
 
 
 def decode_attention_fused(qkv: Tensor, H: int, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float, *,
