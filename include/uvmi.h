@@ -156,6 +156,22 @@ int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus);
 int uvmi_decode_attn_path(const uvmi_attn_args* a);
 
 /* ------------------------------------------------------------------------------------------------------------
+ * Skinny 16-bit GEMM of a small decode step's projections: C (M, N) = A (M, K) . W (N, K)^T, fp32 accumulation, A, W, C
+ * in `dtype` (F16 / BF16), rows contiguous with pitches lda, ldw, ldc (elements).  Replaces the F.linear calls of the
+ * reference's fused inference path (ultraviolet/model.py:302-335 attention projections, 388-391 MLP) when M is a few
+ * hundred rows: the weights are then the traffic, and the kernel requests a workgroup's whole weight strip and its
+ * activation rows in one burst.  K % 64 == 0, K <= 1984; N % 16 == 0.
+ * epilogue UVMI_GEMM_SWIGLU (K <= 960, N % 32 == 0): W holds w_gate and w_up interleaved in slabs of 16 rows ([gate 0..15 |
+ * up 0..15 | gate 16..31 | ...], N = 2 f rows) and C (M, f) = silu(A w_gate^T) * (A w_up^T) with the roundings of the
+ * separate SwiGLU pass (model.py:388-391).
+ * ---------------------------------------------------------------------------------------------------------- */
+#define UVMI_GEMM_STORE 0
+#define UVMI_GEMM_SWIGLU 1
+int uvmi_gemm_tn_supported(int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue);
+int uvmi_gemm_tn(const void* a, const void* w, void* c, int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
+                 int epilogue, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------
  * Packed (cu_seqlens) causal self-attention with an optional sliding window over unquantized K/V: the attention of
  * a packed prefill.  Replaces varlen_attention (ultraviolet/kernels/varlen_attn.py:87-93, forward only) as called
  * by the packed prefill (ultraviolet/kernels/fast_decode.py:117-163, 210-269).

@@ -141,6 +141,9 @@ def lib() -> C.CDLL:
                                        C.c_void_p]
         L.uvmi_sched_expand.argtypes = [C.POINTER(SchedState), C.c_int, C.c_int] + [C.c_void_p] * 8
         L.uvmi_rope_table.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
+        L.uvmi_gemm_tn_supported.argtypes = [C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]
+        L.uvmi_gemm_tn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int64,
+                                   C.c_int64, C.c_int, C.c_void_p]
         _lib = L
     return _lib
 
@@ -167,4 +170,4 @@ EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu",
-           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_rope_table"]
+           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn"]

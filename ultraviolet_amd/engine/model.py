@@ -10,6 +10,7 @@ model.py:1099-1100)."""
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import numpy as np
 import torch
@@ -18,6 +19,7 @@ from torch import Tensor
 from .. import _lib as L
 from ..kernels.decode_attn import (build_attn_args, build_fused_args, decode_attention, decode_attention_fused, decode_attention_post,
                                    rope_table)
+from ..kernels.gemm import SWIGLU, gemm_tn
 from ..kernels.varlen_attn import packed_attention
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
@@ -87,6 +89,10 @@ class UVEngine:
         # post-processing to the attention kernel (one launch less per layer)
         self.fuse_qkv = dt in (torch.bfloat16, torch.float16) and cfg.n_heads // cfg.n_kv_heads <= 8 and cfg.n_pairs in (0, 16)
         self.qkvx_keep = None
+        # Passes of at most this many rows run their K = d_model projections on the skinny GEMM (the MLP's SwiGLU in its
+        # epilogue); above it, and for the down projection, the library GEMM is faster.  Measured on UV-50M decode steps:
+        # 0.544 -> 0.476 ms at 128 rows, 0.551 -> 0.523 at 256, 0.606 -> 0.589 at 384, slower from 512 on.
+        self.skinny_rows = int(os.environ.get("UVMI_SKINNY_ROWS", "384")) if dt in (torch.bfloat16, torch.float16) else 0
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -230,26 +236,31 @@ class UVEngine:
         assert n <= self.max_tokens
         self._embed_norm(tok, n)
         x, xn = b["x"][:n], b["xn"][:n]
+        skinny = n <= self.skinny_rows and cfg.d_model % 64 == 0 and cfg.d_model <= 960 and (cfg.n_heads * cfg.head_dim) % 64 == 0
+        mm = (lambda a, w, out: gemm_tn(a, w, out)) if skinny else (lambda a, w, out: torch.mm(a, w.t(), out=out))
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
                 # decode rows of a 16-bit engine: the projection also forms the gate logits, and fused_attn(l) does the
                 # post-processing, the cache append, the attention and its epilogue in one launch (writes buf zg)
-                torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
+                mm(xn, W["wqkv_ext"], b["qkvx"][:n])
                 if self.qkvx_keep is not None:   # a benchmark re-issues this layer's launch later on the same projection
                     self.qkvx_keep[l][:n].copy_(b["qkvx"][:n])
                 fused_attn(l)
             else:
-                torch.mm(xn, W["wqkv"].t(), out=b["qkv"][:n])
+                mm(xn, W["wqkv"], b["qkv"][:n])
                 self._qkv_post(l, tok, pos, rows, last_pos, st, n)
                 z = attn(l, b["q"][:n])
                 if z is not None:   # None: the attention kernel already applied XSA + gate and wrote buf zg
                     self._attn_post(l, z, n)
-            torch.mm(b["zg"][:n], W["wo"].t(), out=b["a"][:n])
+            mm(b["zg"][:n], W["wo"], b["a"][:n])
             # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
             self._add_norm(x, b["a"][:n], W["resid_attn"], W["post_attn"], n, b["h"], b["xn"])
-            torch.mm(xn, W["gu"].t(), out=b["gu"][:n])
-            self._swiglu(n)
-            torch.mm(b["act"][:n], W["down"].t(), out=b["m"][:n])
+            if skinny and "gu_il" in W:
+                gemm_tn(xn, W["gu_il"], b["act"][:n], epilogue=SWIGLU)
+            else:
+                mm(xn, W["gu"], b["gu"][:n])
+                self._swiglu(n)
+            torch.mm(b["act"][:n], W["down"].t(), out=b["m"][:n])   # (K = d_ff: 26 K-steps per strip, the library is faster)
             # x = resid_mlp * h + post_mlp * m ; xn = rmsnorm(x) (next block's pre-norm, or the final norm)
             self._add_norm(b["h"][:n], b["m"][:n], W["resid_mlp"], W["post_mlp"], n, b["x"], b["xn"])
         return xn

@@ -115,6 +115,12 @@ class UVWeights:
                 if cfg.has_ve(l):
                     ext[cfg.n_heads:cfg.n_heads + cfg.n_kv_heads, :C_v] = t(params[a + "ve_gate"]).to(dtype).float()
                 L["wqkv_ext"] = torch.cat([wqkv.to(dtype), ext.to(dtype)]).to(dev).contiguous()
+                # gate and up rows interleaved in slabs of 16 for the GEMM whose epilogue is the SwiGLU (small decode steps)
+                f = cfg.d_ff
+                if f % 16 == 0:
+                    g16 = gu.to(dtype)
+                    L["gu_il"] = torch.stack([g16[:f].view(f // 16, 16, d), g16[f:].view(f // 16, 16, d)], 1).reshape(2 * f, d) \
+                        .to(dev).contiguous()
             # the four residual scalars are cast to the activation dtype before use (model.py:568-571)
             for s in ("resid_attn", "post_attn", "resid_mlp", "post_mlp"):
                 L[s] = float(torch.tensor(float(params[f"blocks.{l}.{s}"])).to(dtype).float())
