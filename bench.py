@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch / algorithmic bytes per launch of the decode-attention kernel, from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/c5_attention_hbm_counters.md (FETCH_SIZE scaled x2.000 and WRITE_SIZE
 # x1.000 by what they read for a 1 GiB device copy).
-TRAFFIC_PER_ALGORITHMIC_BYTE = 1.09
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.10
 
 
 def _c5_requests(cfg, n_prompts=256, group=8, seed=0):
