@@ -261,15 +261,15 @@ def test_patch_model_binds_the_reference_entry_points():
         fd.patch_model(_StubModel(cfg, params), kv_dtype="fp16")
 
 
-def _fused_vs_unfused(cfg, eng, steps=40, resync=True):
+def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 26), max_len=96):
     """Run the same teacher-forced decode with and without the fused QKV path from identical prefilled states; after every
     step the fused state's caches are overwritten with the unfused ones so that differences do not accumulate.  Returns
     per-step hidden differences, argmax agreement of the logits and per-layer cache statistics."""
     from ultraviolet_amd.engine import KVState
-    prompts = _prompts(cfg, (5, 40, 17, 33, 1, 26), seed=11)
+    prompts = _prompts(cfg, lens, seed=11)
     B = len(prompts)
     cont = np.random.default_rng(12).integers(1, cfg.vocab_size, size=(B, steps))
-    sts = [KVState(cfg, B, 96, DEV) for _ in range(2)]
+    sts = [KVState(cfg, B, max_len, DEV) for _ in range(2)]
     for st in sts:
         eng.prefill(prompts, list(range(B)), st)
     hdiff, agree, cmax, cfrac, sfrac = [], [], np.zeros(cfg.n_layers), np.zeros(cfg.n_layers), np.zeros(cfg.n_layers)
@@ -328,3 +328,18 @@ def test_fused_qkv_decode_matches_unfused(dtype, name, over):
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
     assert np.mean(agree) > 0.9, np.mean(agree)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lens,window,max_len", [((100, 130, 90, 150, 129, 64), 128, 192), ((300, 420, 260, 500, 257, 300), 256, 576)])
+def test_fused_qkv_single_layer_is_exact_with_several_waves_per_row(dtype, lens, window, max_len):
+    """Caches of 128..255 slots run the attention kernel with 2 waves per row and longer ones with 4 (own key formed by the
+    first wave, own value by the second, q handed over through LDS): the appended bytes must still equal the separate
+    post-processing kernel's, on a ring layer (wraps during the run) and on a global layer."""
+    for over in (dict(window=window, global_every=0, ve_every=1), dict(window=0, global_every=1, ve_every=0)):
+        cfg, params, eng, _ = _setup("uv-test", dtype=dtype, perturb=0.05, n_layers=1, attn_gate_channels=128, **over)
+        assert eng.fuse_qkv
+        hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=12, lens=lens, max_len=max_len)
+        assert cmax.max() == 0 and sfrac.max() == 0
+        ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+        assert max(hdiff) <= 4 * 2 * ulp, max(hdiff)
