@@ -216,6 +216,12 @@ typedef struct uvmi_sample_args {
   float cap_a, cap_b, cap_c;       /* softcap a * sigmoid((x + b) / c) */
   float temperature;               /* > 0 draws from softmax(z / T); <= 0 takes argmax (first maximal index) and
                                       logp is log softmax(z)[tok] */
+  /* Truncated sampling, sample() of the reference (ultraviolet/model.py:1194-1211), for T > 0: top_k in 1..V-1 keeps the
+   * tokens whose value is at least the k-th largest; top_p in (0, 1) then keeps the smallest prefix by probability whose
+   * mass reaches top_p (ties of the last kept value all kept).  0 / anything outside (0, 1) switches the filter off.
+   * logp stays the log-prob under the untruncated softmax, as the reference records it (model.py:1161-1169). */
+  int top_k; float top_p;
+  float* thr_out;                  /* optional (B,): the smallest kept exp((z - a) / T) (0 when nothing is filtered) */
 } uvmi_sample_args;
 int uvmi_fused_sample(const uvmi_sample_args* a, void* stream);
 /* Host-side Philox4x32-10 (Random123) for tests and host tooling: out[4] = philox(ctr[4], key[2]). */

@@ -258,7 +258,7 @@ def test_patch_model_binds_the_reference_entry_points():
     assert not hasattr(m, "decode_step")
     from ultraviolet_amd import _lib as L
     with pytest.raises(L.UvmiError):
-        fd.patch_model(_StubModel(cfg, params), kv_dtype="fp16")
+        fd.patch_model(_StubModel(cfg, params), kv_dtype="fp8")
 
 
 def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 26), max_len=96):
@@ -343,3 +343,50 @@ def test_fused_qkv_single_layer_is_exact_with_several_waves_per_row(dtype, lens,
         assert cmax.max() == 0 and sfrac.max() == 0
         ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
         assert max(hdiff) <= 4 * 2 * ulp, max(hdiff)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_unquantized_kv_engine_matches_dense_forward(dtype):
+    """kv_dtype="fp16" (KernelDecodeState's unquantized layout, fast_decode.py:21-57: K/V cached in the compute dtype):
+    prefill + teacher-forced decode steps over the cache must give the logits of the dense causal forward of the whole
+    sequence (the oracle's trunk in the same 16-bit arithmetic) to the bar of the 16-bit engine tests, on global and ring
+    layers through ring wrap-around - and must sit closer to it than the int8-KV engine does."""
+    from ultraviolet_amd.engine import KVState
+    cfg, params, eng, OracleModel = _setup("uv-test", dtype=dtype, perturb=0.06, window=32)
+    m = OracleModel(cfg, params, dtype=dtype)
+    rng = np.random.default_rng(4)
+    L0, steps, B = 20, 40, 4                        # equal prompt lengths: the dense forward needs no padding
+    seqs = rng.integers(1, cfg.vocab_size, size=(B, L0 + steps))
+    hid, _ = m.trunk(torch.as_tensor(seqs))
+    ref = m.logits(hid).float().numpy()[:, L0 - 1:-1]          # logits that predict positions L0 .. L0 + steps - 1
+    errs = {}
+    for kv in ("fp16", "int8"):
+        st = KVState(cfg, B, 96, DEV, kv_dtype=kv, dtype=dtype)
+        assert (st.k[0].dtype == dtype) == (kv == "fp16") and (st.k_scale[0] is None) == (kv == "fp16")
+        outs = [eng.logits(eng.prefill([s[:L0].tolist() for s in seqs], list(range(B)), st)).cpu()]
+        for t in range(steps - 1):
+            outs.append(eng.logits(eng.decode_step(torch.as_tensor(seqs[:, L0 + t]).to(DEV), st)).cpu())
+        got = torch.stack(outs, 1).float().numpy()
+        errs[kv] = np.abs(got - ref)
+        assert (got.argmax(-1) == ref.argmax(-1)).mean() > 0.9
+    assert errs["fp16"].max() < 0.25, errs["fp16"].max()
+    assert errs["fp16"].mean() <= errs["int8"].mean() * 1.05, (errs["fp16"].mean(), errs["int8"].mean())
+
+
+def test_unquantized_kv_rollout_and_patch_model_state():
+    """The continuous-batching driver and the patch_model binding accept the unquantized layout: a greedy rollout over it
+    equals static greedy generation over it, request by request."""
+    from ultraviolet_amd.engine.rollout import Rollout
+    from ultraviolet_amd.kernels import fast_decode as fd
+    cfg, params, eng, _ = _setup("uv-test", dtype=torch.bfloat16, perturb=0.06, window=32)
+    prompts = _prompts(cfg, (9, 30, 4, 17, 25, 12), seed=2)
+    toks = eng.generate(prompts, 20, temperature=0.0, kv_dtype="fp16")
+    g = Rollout(eng, slots=4, max_prompt=32, max_new=20, temperature=0.0, eos_id=None, check_every=4, bucket=4, kv_dtype="fp16")
+    for i, p in enumerate(prompts):
+        g.add(p, i, limit=20)
+    got = {m: row for m, row, _, _ in g.run(max_chunks=500)}
+    same = sum(got[i] == toks[i] for i in range(len(prompts)))
+    assert all(got[i][0] == toks[i][0] for i in range(len(prompts))) and same >= len(prompts) - 1, same   # (a near-tie in the
+    # top-2 logits may flip under another GEMM batch shape)
+    st = fd.KernelDecodeState(cfg, 3, 64, torch.bfloat16, DEV, kv_dtype="fp16")
+    assert st.k[0].dtype == torch.bfloat16 and st.k_scale[0] is None and fd.kv_bytes_per_seq(cfg, 100, "fp16") > fd.kv_bytes_per_seq(cfg, 100)

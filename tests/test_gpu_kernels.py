@@ -470,3 +470,62 @@ def test_skinny_gemm_rejects_what_it_cannot_do():
     a, w = a[:, :1024], w[:, :1024]
     assert gemm_supported(a, w) and not gemm_supported(a, w, SWIGLU)   # the SwiGLU strip needs K <= 960
     assert not gemm_supported(a.float(), w.float())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,V", [(torch.float32, 2048), (torch.bfloat16, 32768), (torch.float16, 16384)])
+@pytest.mark.parametrize("T,top_k,top_p", [(1.0, 50, 1.0), (0.8, 0, 0.9), (1.0, 20, 0.5), (0.7, 1, 1.0), (1.0, 0, 0.05), (1.0, 5000, 0.999)])
+def test_truncated_sampler_matches_oracle(dtype, V, T, top_k, top_p):
+    """Top-k / nucleus sampling (sample(), ultraviolet/model.py:1194-1211) against the float64 oracle: the kept set (read
+    back through the threshold output) is the oracle's except where a token's mass sits within rounding of the nucleus
+    boundary; the token is a kept one, lies in the float64 CDF interval of the kept distribution for the row's uniform and
+    is the oracle's own token almost always; log-probs are those of the untruncated softmax."""
+    from ultraviolet_amd.kernels.fused_sample import sample_filtered
+    fs = _oracle()[1]
+    g = torch.Generator().manual_seed(V + top_k)
+    B = 192
+    x = (torch.randn(B, V, generator=g) * (torch.rand(B, 1, generator=g) * 6 + 0.5)).to(dtype)
+    u = torch.rand(B, generator=g)
+    t, lp, thr = sample_filtered(x.to(DEV), u.to(DEV), SC, T, top_k, top_p, return_threshold=True)
+    t, lp, thr = t.cpu().numpy(), lp.cpu().double().numpy(), thr.cpu().double().numpy()
+    xn = to_np(x).astype(np.float64)
+    tr, lpr, keep = fs.sample_filtered_ref(xn, u.numpy(), SC, T, top_k, top_p)
+    z = SC[0] / (1.0 + np.exp(-(xn + SC[1]) / SC[2]))
+    e = np.exp((z - SC[0]) / T)
+    kept_kernel = e >= thr[:, None] * (1 - 2e-6)
+    same = (kept_kernel == keep).all(1)
+    assert same.mean() >= 0.97, same.mean()
+    for i in np.nonzero(~same)[0]:   # a differing row differs by the tie group at the cut only: its mass straddles top_p
+        diff = kept_kernel[i] != keep[i]
+        assert top_p < 1.0 and np.ptp(e[i][diff]) <= 1e-5 * e[i][diff].max()
+    assert kept_kernel[np.arange(B), t].all()
+    if top_k == 1:
+        assert (t == xn.argmax(1)).all() or (z[np.arange(B), t] == z.max(1)).all()
+    em = np.where(kept_kernel, e, 0.0)
+    cs = em.cumsum(1)
+    S = cs[:, -1]
+    tgt = (1.0 - u.double().numpy()) * S
+    hi = cs[np.arange(B), t]
+    lo = hi - em[np.arange(B), t]
+    assert ((tgt >= lo - 1e-5 * S) & (tgt <= hi + 1e-5 * S)).all()
+    assert (t[same] == tr[same]).mean() > 0.98
+    full = z / T - (z.max(1, keepdims=True) / T + np.log(np.exp((z - z.max(1, keepdims=True)) / T).sum(1, keepdims=True)))
+    assert np.abs(lp - full[np.arange(B), t]).max() < 2e-5
+
+
+@pytest.mark.gpu
+def test_truncated_sampler_off_equals_plain_and_seeded_draw():
+    from ultraviolet_amd.kernels.fused_sample import fused_sample, fused_sample_seeded, sample_filtered
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(64, 4096, generator=g) * 4).bfloat16().to(DEV)
+    u = torch.rand(64, generator=g).to(DEV)
+    t0, l0 = fused_sample(x, u, SC, 0.9)
+    t1, l1 = sample_filtered(x, u, SC, 0.9, 0, 1.0)                      # no filter: the plain kernel runs
+    assert torch.equal(t0, t1) and torch.equal(l0, l1)
+    t2, l2 = sample_filtered(x, u, SC, 0.9, 4095, 0.9999999)             # a filter that keeps everything
+    assert (t0 == t2).float().mean() > 0.98 and (l0 - l2).abs().max() < 2e-5
+    req, ti = torch.arange(64, device=DEV), torch.full((64,), 3, device=DEV)
+    _, _, us = fused_sample_seeded(x, 7, req, ti, SC, 0.9, return_u=True)
+    ta, _ = sample_filtered(x, us, SC, 0.9, 40, 0.8)
+    tb, _ = sample_filtered(x, None, SC, 0.9, 40, 0.8, seed=7, req_id=req, tok_idx=ti)
+    assert torch.equal(ta, tb)

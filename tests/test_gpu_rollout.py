@@ -300,3 +300,45 @@ def test_full_size_rollout_properties():
         assert len({tuple(rows[8 * gidx + j]) for gidx in range(4) for j in range(8)}) > 8   # group members sample differently
         runs.append(rows)
     assert runs[0] == runs[1]
+
+
+def test_rollout_with_truncated_sampling_draws_inside_the_nucleus():
+    """Rollout(top_k, top_p): every generated token lies in the top-k set of its step's distribution (checked by replaying
+    the stream through the engine with teacher forcing), top_k = 1 reproduces the greedy stream, and the behaviour
+    log-probs stay those of the untruncated softmax."""
+    from ultraviolet_amd.engine import KVState, UVEngine, UVWeights, make_config, random_params
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg = make_config("uv-test")
+    eng = UVEngine(UVWeights(cfg, random_params(cfg, 0, perturb=0.06), torch.bfloat16, "cuda"), max_tokens=2048)
+    rng = np.random.default_rng(0)
+    prompts = [rng.integers(1, cfg.vocab_size, size=int(n)).tolist() for n in rng.integers(4, 40, size=12)]
+
+    def run(**kw):
+        g = Rollout(eng, slots=8, max_prompt=64, max_new=24, seed=3, eos_id=None, check_every=4, bucket=8, **kw)
+        for i, p in enumerate(prompts):
+            g.add(p, i, limit=24)
+        out = {}
+        for meta, toks, lps, _ in g.run():
+            out[meta] = (np.asarray(toks), np.asarray(lps))
+        return out
+
+    greedy = run(temperature=0.0)
+    k1 = run(temperature=1.0, top_k=1)
+    assert all((greedy[i][0] == k1[i][0]).all() for i in range(len(prompts)))
+    K = 5
+    outk = run(temperature=1.0, top_k=K, top_p=0.95)
+    plain = run(temperature=1.0)
+    assert any((outk[i][0] != plain[i][0]).any() for i in range(len(prompts)))      # the truncation changes the stream
+    for i, p in enumerate(prompts):
+        toks, lps = outk[i]
+        st = KVState(cfg, 1, 96, "cuda")
+        lg = [eng.logits(eng.prefill([p], [0], st))]
+        for t in toks[:-1]:
+            lg.append(eng.logits(eng.decode_step(torch.tensor([int(t)], device="cuda"), st)))
+        lg = torch.cat(lg).float().cpu()
+        # tokens clearly more likely than the drawn one (the replay runs other GEMM shapes than the rollout did, so its bf16
+        # logits can sit a rounding step away: near-ties at the k-th place are not counted)
+        rank = (lg > lg.gather(1, torch.as_tensor(toks)[:, None]) + 0.06).sum(1)
+        assert int(rank.max()) < K, rank
+        ref_lp = torch.log_softmax(lg, -1).gather(1, torch.as_tensor(toks)[:, None])[:, 0]
+        assert float((ref_lp - torch.as_tensor(lps)).abs().max()) < 5e-2            # bf16 logits: the replay is not bit-identical

@@ -84,3 +84,73 @@ def test_request_uniform_mapping():
     r = philox.philox4x32_10((5, 9, 0, philox.DOMAIN_SAMPLE), (7, 0))
     assert philox.request_uniform(7, 9, 5) == np.float32((int(r[0]) >> 8) * 2.0 ** -24)
     assert philox.request_uniform(7, 9, 5) != philox.request_uniform(7, 9, 5, philox.DOMAIN_RETIRE)
+
+
+# ---- truncated sampling (top-k / nucleus): the oracle's filter against what defines it
+def test_filter_mask_is_a_top_set_with_k_members_and_minimal_nucleus():
+    """Properties that fix sample()'s truncation (ultraviolet/model.py:1200-1209) without restating it: the kept set is a
+    top set by value; top-k keeps exactly k tokens when values are distinct; the nucleus has mass >= top_p and is minimal
+    (dropping its smallest member leaves less than top_p); the most likely token always survives; no filter keeps all."""
+    from oracle.fused_sample import filter_mask
+    rng = np.random.default_rng(0)
+    for V, k, p in [(64, 5, 1.0), (64, 0, 0.7), (512, 40, 0.9), (512, 3, 0.2), (33, 32, 0.999), (128, 1, 0.5), (128, 0, 1e-9)]:
+        z = rng.normal(size=V) * 3
+        keep = filter_mask(z, k, p)
+        assert keep[np.argmax(z)]
+        assert z[keep].min() > z[~keep].max() if (~keep).any() else True
+        pr = np.exp(z - z.max()); pr /= pr.sum()
+        if k and p >= 1.0:
+            assert keep.sum() == k
+        if p < 1.0:
+            base = np.ones(V, bool) if not k else filter_mask(z, k, 1.0)
+            q = np.where(base, pr, 0.0); q /= q.sum()          # the nucleus is taken inside the top-k set, renormalised
+            m = q[keep].sum()
+            assert m >= p - 1e-12 or keep.sum() == base.sum()
+            assert m - q[keep].min() < p                        # minimal: without its smallest member the mass is short
+    assert filter_mask(rng.normal(size=50), 0, 1.0).all()
+
+
+def test_filter_mask_keeps_ties_of_the_cut_value():
+    from oracle.fused_sample import filter_mask
+    z = np.array([3.0, 1.0, 2.0, 2.0, 2.0, 0.0, -1.0])
+    assert filter_mask(z, 2, 1.0).tolist() == [True, False, True, True, True, False, False]      # k-th value 2.0: all three 2.0s stay
+    pr = np.exp(z - 3.0); pr /= pr.sum()
+    p = pr[0] + 1e-6                                                                             # crossing inside the tie group
+    assert filter_mask(z, 0, p).tolist() == [True, False, True, True, True, False, False]
+
+
+def test_filter_mask_brute_force_small():
+    """Every subset rule checked by enumeration on tiny V: the nucleus equals the shortest sorted prefix whose mass reaches
+    top_p, found by trying every prefix length."""
+    from oracle.fused_sample import filter_mask
+    rng = np.random.default_rng(3)
+    for _ in range(200):
+        V = int(rng.integers(2, 9))
+        z = rng.normal(size=V) * 2
+        p = float(rng.uniform(0.05, 0.99))
+        order = np.argsort(-z)
+        pr = np.exp(z - z.max()); pr /= pr.sum()
+        n = next(n for n in range(1, V + 1) if pr[order[:n]].sum() >= p or n == V)
+        want = np.zeros(V, bool); want[order[:n]] = True
+        assert (filter_mask(z, 0, p) == want).all()
+
+
+def test_sample_filtered_ref_draws_only_kept_tokens_in_proportion():
+    from oracle.fused_sample import sample_filtered_ref, fused_sample_ref
+    rng = np.random.default_rng(5)
+    x = rng.normal(size=(1, 32)).astype(np.float32) * 4
+    n = 4000
+    u = rng.random(n)
+    tok, lp, keep = sample_filtered_ref(np.repeat(x, n, 0), u, temperature=0.8, top_k=6, top_p=0.9)
+    assert keep[0, tok].all()
+    z = 23.0 / (1.0 + np.exp(-(x[0].astype(np.float64) + 5.0) / 7.5)) / 0.8
+    q = np.where(keep[0], np.exp(z - z.max()), 0.0); q /= q.sum()
+    cnt = np.bincount(tok, minlength=32)
+    chi = ((cnt - n * q) ** 2 / np.maximum(n * q, 1e-12))[q > 0].sum()
+    assert chi < 40, chi                                    # <= 5 degrees of freedom
+    # log-prob is the untruncated one; no filter reproduces the plain sampler's token
+    t0, l0 = fused_sample_ref(np.repeat(x, 16, 0), u[:16].astype(np.float32), temperature=0.8)
+    t1, l1, _ = sample_filtered_ref(np.repeat(x, 16, 0), u[:16], temperature=0.8)
+    assert (t0 == t1).all() and np.abs(l0 - l1).max() < 1e-5
+    full = z - (z.max() + np.log(np.exp(z - z.max()).sum()))
+    assert np.abs(lp - full[tok]).max() < 1e-12

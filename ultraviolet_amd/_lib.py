@@ -72,7 +72,8 @@ class SampleArgs(C.Structure):
                 ("seed", C.c_uint64), ("req_id", C.c_void_p), ("tok_idx", C.c_void_p),
                 ("tok", C.c_void_p), ("logp", C.c_void_p), ("u_out", C.c_void_p),
                 ("B", C.c_int), ("V", C.c_int),
-                ("cap_a", C.c_float), ("cap_b", C.c_float), ("cap_c", C.c_float), ("temperature", C.c_float)]
+                ("cap_a", C.c_float), ("cap_b", C.c_float), ("cap_c", C.c_float), ("temperature", C.c_float),
+                ("top_k", C.c_int), ("top_p", C.c_float), ("thr_out", C.c_void_p)]
 
 
 class QkvPostArgs(C.Structure):

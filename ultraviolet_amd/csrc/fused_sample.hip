@@ -41,6 +41,7 @@ struct SampleParams {
   float neg_a_over_t_l2;        // -(a/T)*log2(e)
   float neg_a_over_t;           // -(a/T)
   float cap_a, cap_b, cap_c, inv_c;
+  int top_k; float top_p; float* thr_out;
 };
 
 template <int DT>
@@ -153,6 +154,228 @@ __global__ __launch_bounds__(256) void sample_kernel(SampleParams P) {
   }
 }
 
+// Top-k / nucleus sampling (sample() of the reference, ultraviolet/model.py:1194-1211): keep the tokens whose value is at
+// least the k-th largest, then of those the smallest prefix by probability whose mass reaches top_p (the token that
+// crosses it included, ties of the last kept value all kept), and draw from what is kept by inverse CDF in index order.
+// Everything is decided on e = exp((z - a)/T), which is positive and monotone in the logit, so its fp32 bit pattern
+// orders the tokens: both thresholds are found by a radix select over those 32 bits, 8 bits per sweep of the row (the row
+// stays in cache between sweeps).  The nucleus select walks the digits by probability mass; masses are summed as 32.32
+// fixed point in 64-bit integers, so the histogram does not depend on the order in which lanes add to it.  The behaviour
+// log-prob is that of the unfiltered softmax, as the reference records it (model.py:1161-1169).
+template <int DT>
+__global__ __launch_bounds__(256) void sample_filtered_kernel(SampleParams P) {
+  __shared__ float csum[64 + 4];
+  __shared__ unsigned int hcnt[256];
+  __shared__ unsigned long long hmass[256];
+  __shared__ unsigned int sh_prefix, sh_krem;
+  __shared__ unsigned long long sh_mhi, sh_zk;
+  const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tid = threadIdx.x;
+  const char* xr = (const char*)P.x + (int64_t)row * P.stride * (DT == UVMI_F32 ? 4 : 2);
+  const int nchunks = P.V / CHUNK;
+  const int nvec = P.V / 8;
+  auto fix = [](float e) -> unsigned long long { return (unsigned long long)((double)e * 4294967296.0); };
+
+  // ---- unfiltered sum S (for the log-prob), in the order of the unfiltered kernel
+  for (int c = wave; c < nchunks; c += 4) {
+    float v[8];
+    load8<DT>(xr, c * 64 + lane, v);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) s += e_of(v[j], P);
+    s = wave_sum(s);
+    if (lane == 0) csum[c] = s;
+  }
+  __syncthreads();
+  float S = 0.f;
+  for (int c = 0; c < nchunks; c++) S += csum[c];
+  __syncthreads();
+
+  // ---- top-k: the k-th largest key
+  unsigned int thr = 0;  // keep keys >= thr
+  if (P.top_k > 0 && P.top_k < P.V) {
+    unsigned int prefix = 0, mask = 0, krem = (unsigned int)P.top_k;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      hcnt[tid] = 0;
+      __syncthreads();
+      for (int i = tid; i < nvec; i += 256) {
+        float v[8];
+        load8<DT>(xr, i, v);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const unsigned int key = __float_as_uint(e_of(v[j], P));
+          if ((key & mask) == prefix) atomicAdd(&hcnt[(key >> shift) & 255u], 1u);
+        }
+      }
+      __syncthreads();
+      if (tid == 0) {
+        unsigned int c = 0;
+        int d = 255;
+        for (; d > 0; d--) {
+          if (c + hcnt[d] >= krem) break;
+          c += hcnt[d];
+        }
+        sh_prefix = prefix | ((unsigned int)d << shift);
+        sh_krem = krem - c;
+      }
+      __syncthreads();
+      prefix = sh_prefix; krem = sh_krem;
+      mask |= 255u << shift;
+      __syncthreads();
+    }
+    thr = prefix;
+  }
+
+  // ---- nucleus: the smallest key whose mass of strictly larger keys is below top_p * (mass of the top-k set)
+  if (P.top_p < 1.0f) {
+    if (tid == 0) sh_zk = 0;
+    __syncthreads();
+    unsigned long long part = 0;
+    for (int i = tid; i < nvec; i += 256) {
+      float v[8];
+      load8<DT>(xr, i, v);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const float e = e_of(v[j], P);
+        if (__float_as_uint(e) >= thr) part += fix(e);
+      }
+    }
+    atomicAdd(&sh_zk, part);
+    __syncthreads();
+    const double tp = P.top_p > 0.f ? (double)P.top_p : 0.0;
+    const unsigned long long target = (unsigned long long)(tp * (double)sh_zk);
+    unsigned int prefix = 0, mask = 0;
+    unsigned long long mhi = 0;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      hcnt[tid] = 0;
+      hmass[tid] = 0;
+      __syncthreads();
+      for (int i = tid; i < nvec; i += 256) {
+        float v[8];
+        load8<DT>(xr, i, v);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const float e = e_of(v[j], P);
+          const unsigned int key = __float_as_uint(e);
+          if (key >= thr && (key & mask) == prefix) {
+            const unsigned int d = (key >> shift) & 255u;
+            atomicAdd(&hcnt[d], 1u);
+            atomicAdd(&hmass[d], fix(e));
+          }
+        }
+      }
+      __syncthreads();
+      if (tid == 0) {
+        // walk the digits downwards; `run` is the mass above the digit.  The last non-empty digit reached while run <
+        // target holds the cut; when even the largest key fails (top_p = 0) it is kept anyway, as the first token is.
+        unsigned long long run = mhi, above = mhi;
+        int dsel = -1;
+        for (int d = 255; d >= 0; d--) {
+          if (hcnt[d] == 0) continue;
+          if (dsel >= 0 && run >= target) break;
+          dsel = d; above = run;
+          run += hmass[d];
+        }
+        if (dsel < 0) dsel = 0;
+        sh_prefix = prefix | ((unsigned int)dsel << shift);
+        sh_mhi = above;
+      }
+      __syncthreads();
+      prefix = sh_prefix; mhi = sh_mhi;
+      mask |= 255u << shift;
+      __syncthreads();
+    }
+    thr = prefix;  // (a key of the top-k set, so >= the top-k threshold)
+  }
+  auto e_kept = [&](float x) -> float {
+    const float e = e_of(x, P);
+    return __float_as_uint(e) >= thr ? e : 0.f;
+  };
+
+  // ---- draw from the kept tokens: chunk sums, then the chunk, the lane, the element (as the unfiltered kernel)
+  for (int c = wave; c < nchunks; c += 4) {
+    float v[8];
+    load8<DT>(xr, c * 64 + lane, v);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) s += e_kept(v[j]);
+    s = wave_sum(s);
+    if (lane == 0) csum[c] = s;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float incl = lane < nchunks ? csum[lane] : 0.f;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float t = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += t;
+  }
+  const float Sk = __shfl(incl, 63, 64);
+  float u;
+  if (P.u) {
+    u = P.u[row];
+  } else {
+    const uint64_t rid = (uint64_t)P.req_id[row], ti = (uint64_t)P.tok_idx[row];
+    const uint32_t ctr[4] = {(uint32_t)ti, (uint32_t)rid, (uint32_t)(rid >> 32), DOMAIN_SAMPLE};
+    const uint32_t key[2] = {(uint32_t)P.seed, (uint32_t)(P.seed >> 32)};
+    uint32_t o[4];
+    philox4x32_10(ctr, key, o);
+    u = (float)(o[0] >> 8) * 5.9604644775390625e-08f;  // 2^-24
+  }
+  const float target = (1.0f - u) * Sk;
+  const unsigned long long below = __ballot(lane < nchunks && incl < target);
+  int ck = __popcll(below);
+  if (ck > nchunks - 1) ck = nchunks - 1;
+  // (a chunk without kept tokens has the inclusive sum of its predecessor, which is < target whenever it is chosen over,
+  // so the chosen chunk always holds a kept token unless rounding pushed target past the total: then walk back)
+  while (ck > 0 && (ck > 0 ? __shfl(incl, ck - 1, 64) : 0.f) >= Sk) ck--;
+  const float before = ck > 0 ? __shfl(incl, ck - 1, 64) : 0.f;
+  float v[8], e[8];
+  load8<DT>(xr, ck * 64 + lane, v);
+  float ls = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    e[j] = e_kept(v[j]);
+    ls += e[j];
+  }
+  float linc = ls;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float t = __shfl_up(linc, o, 64);
+    if (lane >= o) linc += t;
+  }
+  linc += before;
+  // the lane: the first one whose inclusive sum reaches target and that holds a kept token; when rounding pushed target
+  // past the chunk's total, the last lane that holds one
+  const unsigned long long has = __ballot(ls > 0.f);
+  int ln = __popcll(__ballot(linc < target));
+  {
+    const unsigned long long hi = ln < 64 ? has & ~((1ull << ln) - 1ull) : 0ull;
+    ln = hi ? __ffsll((long long)hi) - 1 : (has ? 63 - __clzll((long long)has) : 0);
+  }
+  // every lane recomputes that lane's walk from broadcast values: the first kept element whose running sum reaches
+  // target, else the lane's last kept element
+  float run = ln > 0 ? __shfl(linc, ln - 1, 64) : before;
+  int sel = ln * 8;
+  float xsel = __shfl(v[0], ln, 64);
+  bool found = false;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const float ej = __shfl(e[j], ln, 64), xj = __shfl(v[j], ln, 64);
+    if (ej > 0.f && !found) {
+      run += ej;
+      sel = ln * 8 + j; xsel = xj;
+      if (run >= target) found = true;
+    }
+  }
+  if (lane == 0) {
+    P.tok[row] = ck * CHUNK + sel;
+    const float E = __builtin_amdgcn_exp2f(fmaf(xsel, P.inv_c_l2, P.b_over_c_l2));
+    P.logp[row] = P.neg_a_over_t * __builtin_amdgcn_rcpf(1.0f + E) - __logf(S);
+    if (P.u_out) P.u_out[row] = u;
+    if (P.thr_out) P.thr_out[row] = __uint_as_float(thr);
+  }
+}
+
 // Greedy: argmax of the raw head output (the softcap is strictly increasing, so argmax z = argmax x), first maximal
 // index; logp = log softmax(z)[tok] at T = 1.
 template <int DT>
@@ -232,6 +455,10 @@ extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
   P.neg_a_over_t = -a->cap_a / T;
   P.neg_a_over_t_l2 = P.neg_a_over_t * l2e;
   P.cap_a = a->cap_a; P.cap_b = a->cap_b; P.cap_c = a->cap_c;
+  P.top_k = a->top_k > 0 && a->top_k < a->V ? a->top_k : 0;
+  P.top_p = a->top_p > 0.f && a->top_p < 1.0f ? a->top_p : 1.0f;
+  P.thr_out = a->thr_out;
+  const bool filtered = !greedy && (P.top_k > 0 || P.top_p < 1.0f);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(a->B), blk(256);
 #define UVMI_S(K)                                                                          \
@@ -240,7 +467,9 @@ extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
     else if (a->x_dtype == UVMI_BF16) hipLaunchKernelGGL((K<UVMI_BF16>), grid, blk, 0, st, P); \
     else hipLaunchKernelGGL((K<UVMI_F32>), grid, blk, 0, st, P);                           \
   } while (0)
-  if (greedy) UVMI_S(argmax_kernel); else UVMI_S(sample_kernel);
+  if (greedy) UVMI_S(argmax_kernel);
+  else if (filtered) UVMI_S(sample_filtered_kernel);
+  else UVMI_S(sample_kernel);
 #undef UVMI_S
   UVMI_CHECK_LAUNCH("uvmi_fused_sample");
   return UVMI_OK;

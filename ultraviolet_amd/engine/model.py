@@ -20,6 +20,7 @@ from .. import _lib as L
 from ..kernels.decode_attn import (build_attn_args, build_fused_args, decode_attention, decode_attention_fused, decode_attention_post,
                                    rope_table)
 from ..kernels.gemm import SWIGLU, gemm_tn
+from ..kernels.kv_quant import kv_write
 from ..kernels.varlen_attn import packed_attention
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
 from .config import UVConfig
@@ -27,30 +28,34 @@ from .weights import UVWeights
 
 
 class KVState:
-    """Slot-indexed int8 KV cache (reference: KernelDecodeState, fast_decode.py:21-57): per layer k, v (B, K, S, hd) int8
+    """Slot-indexed KV cache (reference: KernelDecodeState, fast_decode.py:21-57): per layer k, v (B, K, S, hd) int8
     and k_scale, v_scale (B, K, S) fp16 with S = max_len on global layers and min(window, max_len) on local (ring)
-    layers; pos / starts (B,) int64 on the device.  pos is the next position to write."""
+    layers; pos / starts (B,) int64 on the device.  pos is the next position to write.  kv_dtype "fp16" (the
+    reference's name for "unquantized") keeps k, v in `dtype`, the activation type, with no scales."""
 
-    def __init__(self, cfg: UVConfig, B: int, max_len: int, device="cuda"):
+    def __init__(self, cfg: UVConfig, B: int, max_len: int, device="cuda", kv_dtype: str = "int8", dtype=torch.bfloat16):
         # Global caches are allocated with S rounded up to 32 slots: the MFMA attention kernel streams 32-key tiles and
         # needs S % 4 == 0 for its 8-byte scale loads (other S fall back to the generic kernel).  Ring length is unchanged.
         self.local_len = min(cfg.window, max_len)
         max_len = (max_len + 31) // 32 * 32
         self.cfg, self.B, self.max_len = cfg, B, max_len
+        assert kv_dtype in ("int8", "fp16") and (kv_dtype == "int8" or dtype in (torch.float16, torch.bfloat16))
+        self.kv_dtype, self.quantized = kv_dtype, kv_dtype == "int8"
+        cdt = torch.int8 if self.quantized else dtype
         dev = torch.device(device)
         self.k, self.v, self.k_scale, self.v_scale = [], [], [], []
         for l in range(cfg.n_layers):
             S = max_len if cfg.is_global(l) else self.local_len
             shp = (B, cfg.n_kv_heads, S, cfg.head_dim)
-            self.k.append(torch.zeros(shp, dtype=torch.int8, device=dev))
-            self.v.append(torch.zeros(shp, dtype=torch.int8, device=dev))
-            self.k_scale.append(torch.zeros(shp[:3], dtype=torch.float16, device=dev))
-            self.v_scale.append(torch.zeros(shp[:3], dtype=torch.float16, device=dev))
+            self.k.append(torch.zeros(shp, dtype=cdt, device=dev))
+            self.v.append(torch.zeros(shp, dtype=cdt, device=dev))
+            self.k_scale.append(torch.zeros(shp[:3], dtype=torch.float16, device=dev) if self.quantized else None)
+            self.v_scale.append(torch.zeros(shp[:3], dtype=torch.float16, device=dev) if self.quantized else None)
         self.pos = torch.zeros(B, dtype=torch.long, device=dev)
         self.starts = torch.zeros(B, dtype=torch.long, device=dev)
 
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.k + self.v + self.k_scale + self.v_scale)
+        return sum(t.numel() * t.element_size() for t in self.k + self.v + self.k_scale + self.v_scale if t is not None)
 
 
 def kv_bytes_per_seq(cfg: UVConfig, ctx: int) -> int:
@@ -125,7 +130,7 @@ class UVEngine:
         a.inv_freq = self.w.inv_freq.data_ptr()
         a.q_out, a.q_dtype = b["q"].data_ptr(), L.dtype_code(self.q_dtype)
         a.k_out, a.v_out = b["k"].data_ptr(), b["v"].data_ptr()
-        if st is not None and write_cache:
+        if st is not None and write_cache and st.quantized:
             kc, ks = st.k[l], st.k_scale[l]
             a.k_cache, a.v_cache, a.k_scale, a.v_scale = kc.data_ptr(), st.v[l].data_ptr(), ks.data_ptr(), st.v_scale[l].data_ptr()
             a.scb, a.sch, a.scs, a.ssb, a.ssh = kc.stride(0), kc.stride(1), kc.stride(2), ks.stride(0), ks.stride(1)
@@ -140,6 +145,27 @@ class UVEngine:
         if W["attn_gate"] is not None:
             a.gate_w, a.gate_ch, a.gate_out = W["attn_gate"].data_ptr(), cfg.gate_ch, b["gate"].data_ptr()
         L.check(L.lib().uvmi_qkv_post(C.byref(a), L.stream_ptr(pos)), "uvmi_qkv_post")
+        if st is not None and write_cache and not st.quantized:
+            self._write_kv16(l, pos, rows, last_pos, st, n)
+
+    def _write_kv16(self, l: int, pos: Tensor, rows: Tensor | None, last_pos: Tensor | None, st: KVState, n: int):
+        """Unquantized caches: buf k / v of the n rows go to slot pos (pos % S on a ring) of their cache rows - the two
+        kv_write calls of the reference's step (fast_decode.py:291-294, 315-317).  Dropped, as the int8 append drops them:
+        padding rows, positions past a linear cache, and prompt positions a ring will not keep (older than last_pos - S)."""
+        cfg, b = self.cfg, self.buf
+        K = cfg.n_kv_heads
+        S = st.k[l].size(2)
+        ring = not cfg.is_global(l)
+        row = torch.arange(n, device=pos.device) if rows is None else rows[:n]
+        p = pos[:n]
+        slot = torch.remainder(p, S) if ring else p
+        ok = (row >= 0) & (p >= 0) & (slot < S)
+        if ring and last_pos is not None:
+            ok &= p > last_pos[:n] - S
+        flat = (row[:, None] * K + torch.arange(K, device=pos.device)[None, :]) * S + slot[:, None]
+        flat = torch.where(ok[:, None], flat, torch.full_like(flat, -1)).reshape(-1).contiguous()
+        kv_write(st.k[l], None, flat, b["k"][:n])
+        kv_write(st.v[l], None, flat, b["v"][:n])
 
     def _attn_post(self, l: int, z: Tensor, n: int, off: int = 0):
         """XSA + gate of rows off..off+n of the call (z holds just those rows); writes buf zg[off:off+n]."""
@@ -166,7 +192,7 @@ class UVEngine:
         S = st.k[l].size(2)
         kw = dict(window=0 if glob else cfg.window, ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=rows)
         # the MFMA kernel (which carries the epilogue) streams 32-key tiles: rings need S % 32 == 0, linear caches S % 4 == 0
-        if cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0:
+        if st.quantized and cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0:
             out = b["zg"][off:off + n].view(n, cfg.n_heads, cfg.head_dim)
             decode_attention_post(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, vhat=b["vhat"][off:off + n],
                                   gate=None if W["attn_gate"] is None else b["gate"][off:off + n], xsa=W["xsa"], out=out, **kw)
@@ -176,7 +202,7 @@ class UVEngine:
     def fused_layer_ok(self, l: int, st: KVState) -> bool:
         """Whether layer l's decode attention can take the fused path: the MFMA kernel streams 32-key tiles."""
         S = st.k[l].size(2)
-        return self.fuse_qkv and S % 32 == 0 and S >= 32
+        return self.fuse_qkv and st.quantized and S % 32 == 0 and S >= 32
 
     def rope_table(self, n_positions: int) -> Tensor:
         """cos / sin of every position below n_positions in the activation type's rounding, built once per size."""
@@ -388,14 +414,15 @@ class UVEngine:
     # ------------------------------------------------------------------------------------------------ generation
     @torch.no_grad()
     def generate(self, prompts: list[list[int]], max_new: int, temperature: float = 0.0, seed: int = 0,
-                 max_len: int | None = None, use_graph: bool = False, return_logp: bool = False):
+                 max_len: int | None = None, use_graph: bool = False, return_logp: bool = False, top_k: int = 0,
+                 top_p: float = 1.0, kv_dtype: str = "int8"):
         """Static-batch generation (reference: generate, model.py:1228-1263): packed prefill of all prompts, then
         lockstep decode.  temperature <= 0: greedy.  Otherwise the fused sampler with Philox uniforms keyed by
-        (seed, request = prompt index, token index)."""
+        (seed, request = prompt index, token index), truncated by top_k / top_p as sample() does (model.py:1200-1209)."""
         cfg, dev = self.cfg, self.device
         B = len(prompts)
         T = max(len(p) for p in prompts)
-        st = KVState(cfg, B, max_len or (T + max_new), dev)
+        st = KVState(cfg, B, max_len or (T + max_new), dev, kv_dtype=kv_dtype, dtype=self.dtype)
         req = torch.arange(B, dtype=torch.long, device=dev)
         ti = torch.zeros(B, dtype=torch.long, device=dev)
 
@@ -403,7 +430,7 @@ class UVEngine:
             xh = self.head(hidden)
             if temperature <= 0:
                 return greedy_sample(xh, cfg.softcap)
-            return fused_sample_seeded(xh, seed, req, ti, cfg.softcap, temperature)
+            return fused_sample_seeded(xh, seed, req, ti, cfg.softcap, temperature, top_k=top_k, top_p=top_p)
 
         tok, lp = draw(self.prefill(prompts, list(range(B)), st))
         toks, lps = [tok.clone()], [lp.clone()]

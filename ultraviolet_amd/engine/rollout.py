@@ -29,8 +29,9 @@ class Rollout:
     def __init__(self, engine: UVEngine, slots: int, max_prompt: int, max_new: int, temperature: float = 1.0,
                  seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
                  use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False,
-                 admit_cap: int = 16):
+                 admit_cap: int = 16, top_k: int = 0, top_p: float = 1.0, kv_dtype: str = "int8"):
         self.e, self.cfg = engine, engine.cfg
+        self.top_k, self.top_p = int(top_k), float(top_p)   # truncated sampling (sample(), model.py:1200-1209); off by default
         self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
         self.T, self.seed, self.eos = float(temperature), int(seed), eos_id
         self.ce, self.bucket, self.use_graph = check_every, bucket, use_graph
@@ -40,7 +41,7 @@ class Rollout:
         dev = engine.device
         self.dev = dev
         assert slots <= engine.max_tokens
-        self.st = KVState(self.cfg, slots, max_prompt + max_new + 1, dev)
+        self.st = KVState(self.cfg, slots, max_prompt + max_new + 1, dev, kv_dtype=kv_dtype, dtype=engine.dtype)
         z = lambda *s, dt=torch.long: torch.zeros(*s, dtype=dt, device=dev)
         self.slot_req = torch.full((slots,), -1, dtype=torch.long, device=dev)
         self.slot_cnt, self.slot_limit, self.slot_tok = z(slots), z(slots), z(slots)
@@ -144,7 +145,7 @@ class Rollout:
             tt = lambda a: torch.as_tensor(a, dtype=torch.long, device=self.dev)
             req_t = tt(reqs)
             if self.T > 0:
-                tok, lp = fused_sample_seeded(x, self.seed, req_t, torch.zeros_like(req_t), self.cfg.softcap, self.T)
+                tok, lp = self._sample(x, req_t, torch.zeros_like(req_t))
             else:
                 tok, lp = greedy_sample(x, self.cfg.softcap)
             slot_t, lim_t = tt(slots), tt([b[2] for b in batch])   # named: they must outlive the launch call
@@ -157,7 +158,7 @@ class Rollout:
 
     def _sample(self, x, req, cnt):
         if self.T > 0:
-            return fused_sample_seeded(x, self.seed, req, cnt, self.cfg.softcap, self.T)
+            return fused_sample_seeded(x, self.seed, req, cnt, self.cfg.softcap, self.T, top_k=self.top_k, top_p=self.top_p)
         return greedy_sample(x, self.cfg.softcap)
 
     @torch.no_grad()
@@ -253,7 +254,7 @@ class Rollout:
         h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st, fused_attn=fused)
         x = e.head(h)
         if self.T > 0:
-            tok, lp = fused_sample_seeded(x, self.seed, self.req_c[:n], self.cnt_c[:n], cfg.softcap, self.T)
+            tok, lp = self._sample(x, self.req_c[:n], self.cnt_c[:n])
         else:
             tok, lp = greedy_sample(x, cfg.softcap)
         self.new_tok[:n].copy_(tok)

@@ -4,7 +4,7 @@ UV engine of this package.  patch_model(model) reads model.cfg and model.state_d
 and parameter names), builds the fused device weights once, and binds new_state / prefill / decode_step onto the
 instance exactly as the reference's patch_model does (fast_decode.py:341-364); the model's own forward is untouched.
 
-Only the int8 KV layout is implemented (kv_dtype="int8"); attention-only presets (uv-50m-alpha) only."""
+kv_dtype "int8" (the fast path) or "fp16" (unquantized, in the engine's 16-bit dtype); attention-only presets (uv-50m-alpha) only."""
 from __future__ import annotations
 
 import dataclasses
@@ -45,17 +45,21 @@ class KernelDecodeState(KVState):
     multiple of 32 here) and min(window, max_len) on local ones, plus pos / starts / host_pos."""
 
     def __init__(self, cfg, B: int, max_len: int, dtype=torch.float16, device="cuda", kv_dtype: str = "int8"):
-        if kv_dtype != "int8":
-            raise L.UvmiError(f"kv_dtype {kv_dtype!r}: only the int8 KV layout is implemented")
-        super().__init__(as_uvconfig(cfg), B, max_len, device)
-        self.dtype, self.kv_dtype = dtype, kv_dtype
+        if kv_dtype not in ("int8", "fp16"):
+            raise L.UvmiError(f"kv_dtype {kv_dtype!r}: the KV layouts are 'int8' and 'fp16' (unquantized, in the compute dtype)")
+        super().__init__(as_uvconfig(cfg), B, max_len, device, kv_dtype=kv_dtype, dtype=dtype)
+        self.dtype = dtype
         self.local_len = min(self.cfg.window, self.max_len)
         self.host_pos = np.zeros(B, dtype=np.int64)
 
 
 def kv_bytes_per_seq(cfg, ctx: int, kv_dtype: str = "int8") -> int:
-    assert kv_dtype == "int8"
-    return _kv_bytes(as_uvconfig(cfg), ctx)
+    """Cache bytes of one sequence at context ctx (reference: fast_decode.py:60-67): hd + 2 bytes per key / value row
+    with int8 + fp16 scale, 2 hd unquantized."""
+    c = as_uvconfig(cfg)
+    if kv_dtype == "int8":
+        return _kv_bytes(c, ctx)
+    return sum(2 * c.n_kv_heads * 2 * c.head_dim * (ctx if c.is_global(l) else min(ctx, c.window)) for l in range(c.n_layers))
 
 
 def _engine(model) -> UVEngine:
@@ -107,8 +111,10 @@ def patch_model(model, kv_dtype: str = "int8", num_splits: dict | None = None, b
     """Bind the kernel decode path onto `model` (instance attributes only).  model.cfg and model.state_dict() must use
     the reference's names.  dtype: activation / weight dtype of the engine; max_tokens: largest number of token rows of
     one call (decode rows or packed prefill tokens)."""
-    if kv_dtype != "int8":
-        raise L.UvmiError(f"kv_dtype {kv_dtype!r}: only the int8 KV layout is implemented")
+    if kv_dtype not in ("int8", "fp16"):
+        raise L.UvmiError(f"kv_dtype {kv_dtype!r}: the KV layouts are 'int8' and 'fp16' (unquantized, in the compute dtype)")
+    if kv_dtype == "fp16" and dtype not in (torch.float16, torch.bfloat16):
+        raise L.UvmiError("an unquantized KV cache needs a 16-bit engine dtype")
     cfg = as_uvconfig(model.cfg)
     sd = model.state_dict()
     dev = device or next(iter(sd.values())).device
@@ -117,7 +123,8 @@ def patch_model(model, kv_dtype: str = "int8", num_splits: dict | None = None, b
     eng = UVEngine(UVWeights(cfg, sd, dtype, dev), max_tokens)
 
     def new_state(self, batch, max_len, dtype=torch.float16, device=None):
-        return KernelDecodeState(cfg, batch, max_len, dtype, device or dev, kv_dtype)
+        # (an unquantized cache is kept in the engine's activation dtype, whatever the caller's compute dtype is called)
+        return KernelDecodeState(cfg, batch, max_len, eng.dtype if kv_dtype == "fp16" else dtype, device or dev, kv_dtype)
 
     def decode_step(self, tok, st, g_len=0, skip_attn=False):
         return decode_step_fast(self, tok, st, g_len, skip_attn, num_splits, backend)
