@@ -1054,7 +1054,6 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
       const int64_t slots = (int64_t)cus * 16;
       while (wpr > 1 && P.n_items * wpr > slots && P.n_items * (wpr / 2) <= slots) wpr /= 2;
     }
-    if (const char* e = getenv("UVMI_ATTN_WPR")) { const int v = atoi(e); if (v == 1 || v == 2 || v == 4) wpr = v; }
     P.gran = 32 * wpr;
     if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
     const int ipb = 4 / wpr;
