@@ -390,3 +390,16 @@ def test_unquantized_kv_rollout_and_patch_model_state():
     # top-2 logits may flip under another GEMM batch shape)
     st = fd.KernelDecodeState(cfg, 3, 64, torch.bfloat16, DEV, kv_dtype="fp16")
     assert st.k[0].dtype == torch.bfloat16 and st.k_scale[0] is None and fd.kv_bytes_per_seq(cfg, 100, "fp16") > fd.kv_bytes_per_seq(cfg, 100)
+
+
+@pytest.mark.parametrize("n_kv_heads", [2, 4])
+def test_fused_qkv_single_layer_is_exact_with_grouped_kv_heads(n_kv_heads):
+    """Several KV heads (query groups of 4 and 2 heads per KV head): every KV head's own key / value row, gate logits and
+    value-embedding row are taken from the right columns of the extended projection - identical bytes again."""
+    for over in (dict(window=32, global_every=0, ve_every=1), dict(window=0, global_every=1, ve_every=0)):
+        cfg, params, eng, _ = _setup("uv-test", dtype=torch.bfloat16, perturb=0.05, n_layers=1, attn_gate_channels=128,
+                                     n_kv_heads=n_kv_heads, **over)
+        assert eng.fuse_qkv and cfg.n_heads // cfg.n_kv_heads == 8 // n_kv_heads
+        hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=40)
+        assert cmax.max() == 0 and sfrac.max() == 0
+        assert max(hdiff) <= 4 * 2 * 2.0 ** -7, max(hdiff)
