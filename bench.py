@@ -450,7 +450,7 @@ def main():
     ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy"])
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU only (rollouts shard by sequence with no communication; see DESIGN.md); "
+        print("bench.py: this build measures one GPU only (rollouts shard by sequence with no communication between ranks); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
