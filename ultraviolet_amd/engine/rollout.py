@@ -68,7 +68,6 @@ class Rollout:
         self.act, self.tok_c, self.pos_c = self.row_all[Np:], self.tok_all[Np:], self.pos_all[Np:]
         self.req_c, self.cnt_c = self.req_all[A:], self.cnt_all[A:]
         self.starts_c = z(slots)
-        self.new_tok, self.new_lp = z(slots), z(slots, dt=torch.float32)
         if mixed:
             # admission staging, one host -> device copy per mixed step: [tokens Np | cu A+1 | slot A | start A | limit A | req A]
             self.stage_n = Np + (A + 1) + 3 * A
@@ -80,7 +79,6 @@ class Rollout:
             self.adm_start, o = self.stage_d[o:o + A], o + A
             self.adm_limit, o = self.stage_d[o:o + A], o + A
             self.gather_idx = torch.cat([z(A), Np + torch.arange(slots, device=dev)])   # rows of the hidden that get sampled
-            self.adm_tok, self.adm_lp = z(A), z(A, dt=torch.float32)
             self.adm_slot.fill_(-1)
             self._stage_ev = torch.cuda.Event()
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
@@ -229,14 +227,12 @@ class Rollout:
         h = e.mixed_trunk(self.tok_all, self.pos_all, self.row_all, self.last_all, Np, n, self.adm_cu, self.starts_c[:n], self.st)
         x = e.head(h.index_select(0, self.gather_idx[:A + n]))
         tok, lp = self._sample(x, self.req_all[:A + n], self.cnt_all[:A + n])
-        self.new_tok[:n].copy_(tok[A:])
-        self.new_lp[:n].copy_(lp[A:])
-        self.adm_tok.copy_(tok[:A])
-        self.adm_lp.copy_(lp[:A])
-        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
+        # (the sampler's outputs are read in place: rows 0..A-1 are the prompts' first tokens, the rest the decode rows')
+        tok_d, lp_d = tok[A:], lp[A:]
+        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), tok_d.data_ptr(), lp_d.data_ptr(),
                                       self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
         L.check(lib.uvmi_sched_admit(C.byref(self.sched), A, self.adm_slot.data_ptr(), self.req_all.data_ptr(), self.adm_limit.data_ptr(),
-                                     self.adm_tok.data_ptr(), self.adm_lp.data_ptr(), sp), "uvmi_sched_admit")
+                                     tok.data_ptr(), lp.data_ptr(), sp), "uvmi_sched_admit")
 
     # ------------------------------------------------------------------------------------------------ decode
     def _step_body(self, n: int):
@@ -257,9 +253,7 @@ class Rollout:
             tok, lp = self._sample(x, self.req_c[:n], self.cnt_c[:n])
         else:
             tok, lp = greedy_sample(x, cfg.softcap)
-        self.new_tok[:n].copy_(tok)
-        self.new_lp[:n].copy_(lp)
-        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), self.new_tok.data_ptr(), self.new_lp.data_ptr(),
+        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), tok.data_ptr(), lp.data_ptr(),
                                       self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
 
     def _attention(self, l, q, st, pos, starts, n, act):
