@@ -190,10 +190,18 @@ typedef struct uvmi_prefill_attn_args {
   float scale;
   int window;
   void* workspace; size_t workspace_bytes; /* >= uvmi_prefill_attn_workspace_bytes(N): per-token segment table */
+  int segments_ready;                      /* non-zero: the workspace already holds the table of these cu_seqlens (an earlier
+                                              call with the same workspace, e.g. the previous layer's): skip building it */
+  /* Optional fused epilogue, used when post_vhat != NULL (MFMA kernel only): Attention.post before the output projection
+   * (ultraviolet/model.py:321-333), as in uvmi_attn_args: XSA z -= xsa[h] (z . v_hat) v_hat, then z *= gate[token][h]. */
+  const float* post_vhat;                  /* (N, KH, hd) fp32 normalized v of every token (uvmi_qkv_post vhat_out) */
+  const float* post_gate;                  /* (N, H) fp32 gate values (uvmi_qkv_post gate_out), or NULL */
+  const float* post_xsa;                   /* (H,) tanh(alpha) fp32, or NULL */
 } uvmi_prefill_attn_args;
 /* The MFMA kernel runs when hd == 64, H / KH <= 8, q and k/v share a 16-bit dtype and rows are 16-byte aligned
  * (probabilities are rounded to that dtype for P.V, accumulation is fp32); anything else that uvmi_decode_attn's
- * generic kernel accepts runs there, token by token.  Two launches: the segment table, then the attention. */
+ * generic kernel accepts runs there, token by token.  Two launches: the segment table (unless segments_ready), then the
+ * attention. */
 int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream);
 size_t uvmi_prefill_attn_workspace_bytes(int N);
 /* 1 = MFMA kernel, 0 = generic kernel, negative = unsupported */

@@ -146,3 +146,34 @@ def test_error_paths():
         packed_attention(d(q).float(), d(k), d(v), d(cu), SC)    # fp32 q is not supported
     with pytest.raises(AssertionError):
         packed_attention(d(q), d(k), d(v), d(cu), SC, workspace=torch.empty(64, dtype=torch.uint8, device=DEV))  # too small
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 48])
+def test_packed_attention_fused_post_epilogue(dtype, window):
+    """post=(vhat, gate, xsa): the kernel's epilogue equals Attention.post applied to its own plain output
+    (ultraviolet/model.py:321-333: z -= xsa_h (z . v_hat) v_hat on the output rounded to the activation type, then the
+    per-head gate), evaluated here in float64 from the plain output of the same kernel; reusing the segment table of an
+    earlier call (segments_ready) changes nothing."""
+    from ultraviolet_amd.kernels.varlen_attn import packed_attention
+    g = torch.Generator(device="cuda").manual_seed(5)
+    lens = [37, 1, 160, 64, 5]
+    N, H, K, hd = sum(lens), 8, 2, 64
+    cu = torch.tensor([0] + list(np.cumsum(lens)), device="cuda")
+    q = torch.randn(N, H, hd, device="cuda", generator=g).to(dtype)
+    k = torch.randn(N, K, hd, device="cuda", generator=g).to(dtype)
+    v = torch.randn(N, K, hd, device="cuda", generator=g).to(dtype)
+    vhat = torch.nn.functional.normalize(v.float(), dim=-1).contiguous()
+    gate = (torch.rand(N, H, device="cuda", generator=g) * 2).contiguous()
+    xsa = torch.tanh(torch.randn(H, device="cuda", generator=g)).contiguous()
+    ws = torch.empty(1 << 16, dtype=torch.uint8, device="cuda")
+    plain = packed_attention(q, k, v, cu, 0.125, window, workspace=ws)
+    fused = packed_attention(q, k, v, cu, 0.125, window, workspace=ws, segments_ready=True, post=(vhat, gate, xsa))
+    z = plain.double()
+    vh = vhat.double().repeat_interleave(H // K, dim=1)
+    want = (z - xsa.double()[None, :, None] * (z * vh).sum(-1, keepdim=True) * vh) * gate.double()[:, :, None]
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    err = (fused.double() - want).abs()
+    assert float((err / (want.abs() + 1.0)).max()) <= 3 * ulp, float((err / (want.abs() + 1.0)).max())
+    no_gate = packed_attention(q, k, v, cu, 0.125, window, workspace=ws, post=(vhat, None, None))
+    assert float((no_gate.double() - z).abs().max()) <= 2 * ulp * float(z.abs().max())

@@ -55,7 +55,8 @@ class PrefillAttnArgs(C.Structure):
                 ("cu_seqlens", C.c_void_p), ("idx_dtype", C.c_int), ("n_seg", C.c_int),
                 ("out", C.c_void_p), ("out_dtype", C.c_int), ("son", C.c_int64), ("soh", C.c_int64),
                 ("N", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int),
-                ("scale", C.c_float), ("window", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+                ("scale", C.c_float), ("window", C.c_int), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+                ("segments_ready", C.c_int), ("post_vhat", C.c_void_p), ("post_gate", C.c_void_p), ("post_xsa", C.c_void_p)]
 
 
 class KvAppendArgs(C.Structure):

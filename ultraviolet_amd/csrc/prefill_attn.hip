@@ -48,6 +48,7 @@ struct PrefillParams {
   int N, H, KH, G, window, n_hg;
   int64_t n_items;
   float scale_log2;
+  const float* post_vhat; const float* post_gate; const float* post_xsa;  // fused Attention.post epilogue when post_vhat != null
 };
 
 // seg_start[i] = cu[s] for the last s with cu[s] <= i (empty sequences are skipped); pidx[i] = i.
@@ -272,17 +273,48 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
   }
 
   // ---- normalise and store: lane (row m, group g) holds head dims 16g .. 16g+15 (O[t][i] is dim 16g + 4i + t)
+  // Optional epilogue, as in the decode kernel: z (rounded to the activation type, as the attention output tensor would be)
+  // -> XSA with the token's normalised v -> per-head gate; the 4 lane groups of a row reduce z . v_hat between them.
+  const bool has_post = P.post_vhat != nullptr;
+  float vv[16];
+  if (has_post) {
+    const float* vp = P.post_vhat + ((int64_t)rowc * P.KH + kvh) * 64 + 16 * g;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const float4 x = *(const float4*)(vp + 4 * i);
+      vv[4 * i] = x.x; vv[4 * i + 1] = x.y; vv[4 * i + 2] = x.z; vv[4 * i + 3] = x.w;
+    }
+  }
+  auto rnd = [&](float x) -> float { return DT == UVMI_BF16 ? bf16_to_float(float_to_bf16(x)) : (float)(half_t)x; };
 #pragma unroll
   for (int hh = 0; hh < HPW; hh++) {
     const int hq = hg * HPW + hh;
     const float l = psum32(psum16(lrun[hh]));
-    if (hq >= G || !row_ok) continue;
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     float o[16];
 #pragma unroll
     for (int t = 0; t < 4; t++)
 #pragma unroll
       for (int i = 0; i < 4; i++) o[4 * i + t] = O[hh][t][i] * inv;
+    if (has_post) {  // (every lane takes part in the reduction; lanes of absent heads / rows compute on clamped operands)
+      const int head = kvh * G + (hq < G ? hq : G - 1);
+      float proj = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        o[i] = rnd(o[i]);
+        proj += o[i] * vv[i];
+      }
+      if (P.post_xsa) {
+        proj = psum32(psum16(proj));
+        const float ah = P.post_xsa[head] * proj;
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[i] = rnd(o[i] - ah * vv[i]);
+      }
+      const float gate = P.post_gate ? P.post_gate[(int64_t)rowc * P.H + head] : 1.0f;
+#pragma unroll
+      for (int i = 0; i < 16; i++) o[i] *= gate;
+    }
+    if (hq >= G || !row_ok) continue;
     const int64_t off = (int64_t)row * P.son + (int64_t)(kvh * G + hq) * P.soh + 16 * g;
     if (ODT == UVMI_F32) {
       float* op = (float*)P.out + off;
@@ -356,9 +388,15 @@ extern "C" int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream) 
   hipStream_t st = (hipStream_t)stream;
   int32_t* seg_start = (int32_t*)a->workspace;
   int32_t* pidx = (int32_t*)((char*)a->workspace + ((size_t)a->N * 4 + 255) / 256 * 256);
-  hipLaunchKernelGGL(prefill_segments, dim3((unsigned)((a->N + 255) / 256)), dim3(256), 0, st, a->cu_seqlens, a->idx_dtype == UVMI_I64 ? 1 : 0,
-                     a->n_seg, a->N, seg_start, pidx);
-  UVMI_CHECK_LAUNCH("uvmi_prefill_attn(segments)");
+  if (!a->segments_ready) {
+    hipLaunchKernelGGL(prefill_segments, dim3((unsigned)((a->N + 255) / 256)), dim3(256), 0, st, a->cu_seqlens, a->idx_dtype == UVMI_I64 ? 1 : 0,
+                       a->n_seg, a->N, seg_start, pidx);
+    UVMI_CHECK_LAUNCH("uvmi_prefill_attn(segments)");
+  }
+  if (a->post_vhat) {
+    UVMI_REQUIRE(prefill_mfma_ok(a), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: the fused post epilogue needs the MFMA kernel (head_dim 64, 16-bit q / k / v)");
+    UVMI_REQUIRE(((uintptr_t)a->post_vhat % 16) == 0, UVMI_EINVAL, "uvmi_prefill_attn: post_vhat must be 16-byte aligned");
+  }
   if (!prefill_mfma_ok(a)) {
     // every packed token is a decode row whose "cache" is the packed K / V of the call (batch stride 0)
     uvmi_attn_args d = {};
@@ -378,6 +416,7 @@ extern "C" int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream) 
   P.n_hg = (P.G + HPW - 1) / HPW;
   P.n_items = (int64_t)((a->N + 15) / 16) * a->KH * P.n_hg;
   P.scale_log2 = a->scale * 1.4426950408889634f;
+  P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa;
   UVMI_REQUIRE(P.n_items < (1LL << 31), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: too many work items");
   const unsigned nblk = (unsigned)(((P.n_items + 3) / 4 + 7) / 8 * 8);
   const dim3 grid(nblk), blk(256);

@@ -199,6 +199,22 @@ class UVEngine:
             return None
         return decode_attention(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, num_splits=1, **kw)
 
+    def prompt_attention(self, l: int, q: Tensor, N: int, cu: Tensor):
+        """Causal (windowed on local layers) attention of the N packed prompt tokens at the head of the call's buffers over
+        their own unquantized K / V (buf k, v).  Where the MFMA kernel runs (16-bit engine) XSA and the gate ride in its
+        epilogue - it writes buf zg[:N] and None is returned; otherwise the plain attention output is returned for
+        _attn_post.  The segment table of cu is built by layer 0's call and reused by the other layers of the pass."""
+        cfg, b, W = self.cfg, self.buf, self.w.layers[l]
+        w = 0 if cfg.is_global(l) else cfg.window
+        kw = dict(workspace=self.pf_ws, segments_ready=l > 0)
+        if (cfg.xsa and self.dtype in (torch.bfloat16, torch.float16) and self.q_dtype == self.dtype and cfg.head_dim == 64
+                and cfg.n_heads // cfg.n_kv_heads <= 8):
+            out = b["zg"][:N].view(N, cfg.n_heads, cfg.head_dim)
+            packed_attention(q, b["k"][:N], b["v"][:N], cu, cfg.attn_scale, w, out=out,
+                             post=(b["vhat"][:N], None if W["attn_gate"] is None else b["gate"][:N], W["xsa"]), **kw)
+            return None
+        return packed_attention(q, b["k"][:N], b["v"][:N], cu, cfg.attn_scale, w, **kw)
+
     def fused_layer_ok(self, l: int, st: KVState) -> bool:
         """Whether layer l's decode attention can take the fused path: the MFMA kernel streams 32-key tiles."""
         S = st.k[l].size(2)
@@ -381,9 +397,9 @@ class UVEngine:
         pos_d, rows_d = pos[Np:N], rows[Np:N]
 
         def attn(l, q):
-            w = 0 if cfg.is_global(l) else cfg.window
-            zp = packed_attention(q[:Np], b["k"][:Np], b["v"][:Np], cu, cfg.attn_scale, w, workspace=self.pf_ws)
-            self._attn_post(l, zp, Np)
+            zp = self.prompt_attention(l, q[:Np], Np, cu)
+            if zp is not None:
+                self._attn_post(l, zp, Np)
             zd = self.cache_attention(l, q[Np:N], st, pos_d, starts_d, nd, rows=rows_d, off=Np)
             if zd is not None:
                 self._attn_post(l, zd, nd, off=Np)
@@ -403,9 +419,7 @@ class UVEngine:
         N, b, cfg = pk["N"], self.buf, self.cfg
 
         def attn(l, q):
-            # causal (windowed on local layers) attention of every prompt over its own unquantized K / V of this call
-            w = 0 if cfg.is_global(l) else cfg.window
-            return packed_attention(q, b["k"][:N], b["v"][:N], pk["cu"], cfg.attn_scale, w, workspace=self.pf_ws)
+            return self.prompt_attention(l, q, N, pk["cu"])
 
         h = self._trunk(pk["tok"], pk["pos"], N, attn, rows=pk["row"], last_pos=pk["last"], st=st)
         self.bind_prompts(pk, st)

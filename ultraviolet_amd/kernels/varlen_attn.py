@@ -27,10 +27,14 @@ def _args(q, k, v, cu, scale, window, out, ws):
 
 
 def packed_attention(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, scale: float, window: int | None = None,
-                     out: Tensor | None = None, out_fp32: bool = False, workspace: Tensor | None = None) -> Tensor:
+                     out: Tensor | None = None, out_fp32: bool = False, workspace: Tensor | None = None,
+                     segments_ready: bool = False, post: tuple | None = None) -> Tensor:
     """q (N, H, hd) fp16 / bf16, k / v (N, K, hd) (same dtype for the MFMA kernel; fp32 runs the generic kernel),
     cu_seqlens (S+1,) int32 / int64 on the device.  Returns (N, H, hd) in q's dtype (fp32 with out_fp32), or fills `out`.
-    `workspace` (uint8, >= uvmi_prefill_attn_workspace_bytes(N)) avoids the allocation."""
+    `workspace` (uint8, >= uvmi_prefill_attn_workspace_bytes(N)) avoids the allocation; segments_ready: it already holds
+    the segment table of these cu_seqlens (an earlier call).  post = (vhat (N, K, hd) fp32, gate (N, H) fp32 or None, xsa
+    (H,) fp32 or None) applies Attention.post (XSA, per-head gate; ultraviolet/model.py:321-333) in the kernel's epilogue
+    (MFMA kernel only)."""
     L.require_cuda(q, k, v, cu_seqlens)
     assert q.dim() == 3 and k.dim() == 3 and v.shape == k.shape and k.size(0) == q.size(0) and k.size(2) == q.size(2)
     assert q.size(1) % k.size(1) == 0, "H must be a multiple of K"
@@ -53,6 +57,17 @@ def packed_attention(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, scale:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     assert workspace.dtype == torch.uint8 and workspace.numel() >= need
     a = _args(q, k, v, cu_seqlens, scale, window, out, workspace)
+    a.segments_ready = int(bool(segments_ready))
+    if post is not None:
+        vhat, gate, xsa = post
+        assert vhat.dtype == torch.float32 and vhat.is_contiguous() and vhat.shape == (N, k.size(1), q.size(2))
+        a.post_vhat = vhat.data_ptr()
+        if gate is not None:
+            assert gate.dtype == torch.float32 and gate.is_contiguous() and gate.shape == (N, q.size(1))
+            a.post_gate = gate.data_ptr()
+        if xsa is not None:
+            assert xsa.dtype == torch.float32 and xsa.is_contiguous() and xsa.numel() == q.size(1)
+            a.post_xsa = xsa.data_ptr()
     L.check(L.lib().uvmi_prefill_attn(C.byref(a), L.stream_ptr(q)), "uvmi_prefill_attn")
     return out
 
