@@ -21,7 +21,9 @@ FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Xclang", "-ta
          "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unknown-warning-option",
          # keep MFMA accumulators in VGPRs: the attention kernels rescale them with VALU ops, and the AGPR form costs
          # an accvgpr read/write pair per register per step
-         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+         # the first kernel arguments arrive in SGPRs with the wave instead of through a load at kernel start
+         "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 def _hipcc() -> str:

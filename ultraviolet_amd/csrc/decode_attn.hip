@@ -183,8 +183,15 @@ __device__ unsigned long long g_attn_tim[1 << 15][8];
 // FUSE: the row's own token is taken from the projection output (q, k, v, gate logits) instead of from q and the cache:
 // the kernel normalises and rotates q and k, adds the value embedding to v, quantises k and v into the cache, and attends
 // the streamed cache range lo..pos-1 plus the own key from registers; the XSA / gate epilogue uses the own v directly.
+// The arguments ahead of the parameter block are what a wave needs before it can request anything - the index arrays of
+// the row's plan, the q (or projection) pointer and the item arithmetic: as leading scalar arguments they are preloaded
+// into SGPRs with the wave, so the plan's loads go out without first waiting for a load of the kernel arguments.
 template <int QDT, int ODT, int WPR, bool FUSE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void attn_mfma_i8_hd64(AttnParams P) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_rows, const void* a_q, int64_t a_items, int a_idx64,
+                       int a_splits, int a_kh, AttnParams P) {
+  P.pos = a_pos; P.starts = a_starts; P.rows = a_rows; P.n_items = a_items; P.idx64 = a_idx64; P.splits = a_splits; P.KH = a_kh;
+  if (FUSE) P.f_qkv = a_q; else P.q = a_q;
 #ifdef UVMI_ATTN_TIMING
   unsigned long long tim_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   UVMI_TS(0, 0);
@@ -1058,17 +1065,18 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
     if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
     const int ipb = 4 / wpr;
     const dim3 grid((unsigned)((P.n_items + ipb - 1) / ipb)), blk(256);
+#define UVMI_LEAD P.pos, P.starts, P.rows, (a->fuse ? P.f_qkv : P.q), P.n_items, P.idx64, P.splits, P.KH
 #define UVMI_L(QD, OD)                                                                                \
   do {                                                                                                \
-    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 4, false>), grid, blk, 0, st, P);      \
-    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2, false>), grid, blk, 0, st, P); \
-    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1, false>), grid, blk, 0, st, P);               \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 4, false>), grid, blk, 0, st, UVMI_LEAD, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2, false>), grid, blk, 0, st, UVMI_LEAD, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1, false>), grid, blk, 0, st, UVMI_LEAD, P);               \
   } while (0)
 #define UVMI_LF(QD)                                                                                   \
   do {                                                                                                \
-    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true>), grid, blk, 0, st, P);       \
-    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true>), grid, blk, 0, st, P);  \
-    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true>), grid, blk, 0, st, P);                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true>), grid, blk, 0, st, UVMI_LEAD, P);       \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true>), grid, blk, 0, st, UVMI_LEAD, P);  \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true>), grid, blk, 0, st, UVMI_LEAD, P);                \
   } while (0)
     const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
     if (a->fuse) {
@@ -1080,6 +1088,7 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
     }
 #undef UVMI_L
 #undef UVMI_LF
+#undef UVMI_LEAD
   } else {
     const dim3 grid((unsigned)P.n_items), blk(64);
     const size_t sh = ((size_t)P.G * a->hd + (size_t)P.G * 64) * 4;

@@ -70,8 +70,12 @@ __device__ __forceinline__ float e_of(float x, const SampleParams& P) {
   return __builtin_amdgcn_exp2f(P.neg_a_over_t_l2 * __builtin_amdgcn_rcpf(1.0f + E));
 }
 
+// (the row pointer's ingredients lead the argument list: leading scalar arguments are preloaded into SGPRs with the wave,
+// so the first loads of the row do not wait for a load of the kernel arguments)
 template <int DT>
-__global__ __launch_bounds__(256) void sample_kernel(SampleParams P) {
+__global__ __launch_bounds__(256) void sample_kernel(const void* a_x, int64_t a_stride, int a_V, float a_inv_c_l2, float a_b_over_c_l2,
+                                                     float a_neg_a_over_t_l2, SampleParams P) {
+  P.x = a_x; P.stride = a_stride; P.V = a_V; P.inv_c_l2 = a_inv_c_l2; P.b_over_c_l2 = a_b_over_c_l2; P.neg_a_over_t_l2 = a_neg_a_over_t_l2;
   __shared__ float csum[64 + 4];
   __shared__ int sh_chunk;
   __shared__ float sh_before, sh_total, sh_target;
@@ -469,7 +473,14 @@ extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
   } while (0)
   if (greedy) UVMI_S(argmax_kernel);
   else if (filtered) UVMI_S(sample_filtered_kernel);
-  else UVMI_S(sample_kernel);
+  else {
+    if (a->x_dtype == UVMI_F16)
+      hipLaunchKernelGGL((sample_kernel<UVMI_F16>), grid, blk, 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P);
+    else if (a->x_dtype == UVMI_BF16)
+      hipLaunchKernelGGL((sample_kernel<UVMI_BF16>), grid, blk, 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P);
+    else
+      hipLaunchKernelGGL((sample_kernel<UVMI_F32>), grid, blk, 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P);
+  }
 #undef UVMI_S
   UVMI_CHECK_LAUNCH("uvmi_fused_sample");
   return UVMI_OK;

@@ -68,8 +68,14 @@ constexpr int SK_RING = 16;     // activation K-steps (of 32) in flight per wave
 constexpr int SK_WPASS = 16;    // most passes of the weight-strip load (32 (row, 128-byte segment) units per pass)
 
 // EPI 0: C = A W^T (M, N).  EPI 1 (BN = 32): W rows are [gate 16 | up 16] slabs; C = silu(gate) * up, (M, N / 2).
+// (individual scalar arguments rather than a parameter block: they are preloaded into SGPRs with the wave, so the first
+// loads need not wait for a load of the kernel arguments)
 template <int DT, int BN, int EPI>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyParams P) {
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const void* a_w, void* a_c, uint32_t a_lda2, uint32_t a_ldw2,
+                                                          int a_M, int a_N, int a_K, int a_tiles_m, int a_tiles_n, int64_t a_ldc) {
+  SkinnyParams P;
+  P.a = a_a; P.w = a_w; P.c = a_c; P.lda2 = a_lda2; P.ldw2 = a_ldw2; P.ldc = a_ldc; P.M = a_M; P.N = a_N; P.K = a_K;
+  P.tiles_m = a_tiles_m; P.tiles_n = a_tiles_n;
   extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];  // BN rows of K * 2 + 16 bytes
   constexpr int TN = BN / 16;
   constexpr uint32_t OOB = 0x40000000u;  // added to an offset that must read as zero (every valid offset is below 2^30)
@@ -211,7 +217,9 @@ extern "C" int uvmi_gemm_tn(const void* a, const void* w, void* c, int dtype, in
   const dim3 grid((unsigned)(((T + 7) / 8) * 8)), blk(256);
   const size_t lds = (size_t)BN * ((size_t)K * 2 + 16);  // at most 32 * 1936 = 62 KB, 16 * 3984 = 64 KB
   hipStream_t st = (hipStream_t)stream;
-  auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, blk, lds, st, P); };
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, grid, blk, lds, st, P.a, P.w, P.c, P.lda2, P.ldw2, P.M, P.N, P.K, P.tiles_m, P.tiles_n, P.ldc);
+  };
   if (dtype == UVMI_F16) {
     if (epilogue == UVMI_GEMM_SWIGLU) go(gemm_skinny_kernel<UVMI_F16, 32, 1>);
     else if (BN == 32) go(gemm_skinny_kernel<UVMI_F16, 32, 0>);
