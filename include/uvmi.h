@@ -167,9 +167,28 @@ int uvmi_decode_attn_path(const uvmi_attn_args* a);
  * ---------------------------------------------------------------------------------------------------------- */
 #define UVMI_GEMM_STORE 0
 #define UVMI_GEMM_SWIGLU 1
+#define UVMI_GEMM_RESID 2
 int uvmi_gemm_tn_supported(int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue);
 int uvmi_gemm_tn(const void* a, const void* w, void* c, int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc,
                  int epilogue, void* stream);
+/* The same GEMM with the two fusions that remove the residual-add + norm launch between a block's projections
+ * (ultraviolet/model.py:567-571):
+ *   epilogue UVMI_GEMM_RESID: C = ca * resid + cb * (A W^T), resid (M, N) in `dtype` with pitch ldr - the product is rounded
+ *     to `dtype` first and the sum rounded again, as a GEMM followed by the residual-add kernel would;
+ *   norm_a != 0: A stands for rmsnorm(A) (no weight, epsilon eps): the kernel sums the squares of its rows while they stream
+ *     and scales the product by rsqrt(mean + eps); the normalised rows are neither written nor rounded to `dtype`.
+ * Any epilogue combines with norm_a. */
+typedef struct uvmi_gemm_args {
+  const void* a; const void* w; void* c; int dtype;
+  int64_t M; int N, K;
+  int64_t lda, ldw, ldc;
+  int epilogue;
+  int norm_a; float eps;
+  const void* resid; int64_t ldr; float ca, cb;
+  int config;                              /* 0: built-in choice of the kernel form; 1: 64-row workgroups; 2: 16-row workgroups
+                                              whose waves split K (needs K % 128 == 0, else form 1) - for tuning and tests */
+} uvmi_gemm_args;
+int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------
  * Packed (cu_seqlens) causal self-attention with an optional sliding window over unquantized K/V: the attention of

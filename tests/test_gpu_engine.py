@@ -324,7 +324,8 @@ def test_fused_qkv_decode_matches_unfused(dtype, name, over):
     assert eng.fuse_qkv
     hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=24)
     assert cmax[0] == 0 and sfrac[0] == 0
-    assert (cmax <= 1 + np.arange(cfg.n_layers)).all(), cmax     # the perturbation grows layer by layer (bf16 activations)
+    # the perturbation grows layer by layer (16-bit activations: one unit in the last place of a key is half an int8 code)
+    assert (cmax <= 3 + np.arange(cfg.n_layers)).all(), cmax
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
     assert np.mean(agree) > 0.9, np.mean(agree)

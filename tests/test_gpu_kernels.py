@@ -427,14 +427,15 @@ def test_skinny_gemm_matches_fp32_reference(dtype, M, K, N):
     w_full = (torch.randn(N, K + 16, device="cuda", generator=g) / K ** 0.5).to(dtype)
     a, w = a_full[:, :K], w_full[:, :K]
     assert gemm_supported(a, w)
-    out_full = torch.full((M, N + 4), 7.0, device="cuda", dtype=dtype)
-    out = out_full[:, :N]
-    gemm_tn(a, w, out)
     ref = a.double() @ w.double().t()
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     tol = ulp * ref.abs().clamp_min(1.0) + 1e-5 * K ** 0.5
-    assert bool(((out.double() - ref).abs() <= tol).all()), float((out.double() - ref).abs().max())
-    assert bool((out_full[:, N:] == 7.0).all())   # nothing written past column N
+    for config in (1, 2):     # 64-row workgroups; 16-row workgroups whose waves split K (the latter when K % 128 == 0)
+        out_full = torch.full((M, N + 4), 7.0, device="cuda", dtype=dtype)
+        out = out_full[:, :N]
+        gemm_tn(a, w, out, config=config)
+        assert bool(((out.double() - ref).abs() <= tol).all()), (config, float((out.double() - ref).abs().max()))
+        assert bool((out_full[:, N:] == 7.0).all())   # nothing written past column N
 
 
 @pytest.mark.gpu
@@ -448,14 +449,15 @@ def test_skinny_gemm_swiglu_epilogue(dtype, M, K, f):
     a = torch.randn(M, K, device="cuda", generator=g).to(dtype)
     wg = (torch.randn(f, K, device="cuda", generator=g) / K ** 0.5).to(dtype)
     wu = (torch.randn(f, K, device="cuda", generator=g) / K ** 0.5).to(dtype)
-    out = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU)
-    assert out.shape == (M, f)
     gg = (a.double() @ wg.double().t()).to(dtype).double()
     uu = (a.double() @ wu.double().t()).to(dtype).double()
     ref = (gg * torch.sigmoid(gg)).to(dtype).double() * uu
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     tol = 4 * ulp * ref.abs().clamp_min(1.0) + 4 * ulp * (gg.abs() + uu.abs())   # g and u may each sit one rounding step off
-    assert bool(((out.double() - ref).abs() <= tol).all()), float((out.double() - ref).abs().max())
+    for config in (1, 2):
+        out = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU, config=config)
+        assert out.shape == (M, f)
+        assert bool(((out.double() - ref).abs() <= tol).all()), (config, float((out.double() - ref).abs().max()))
 
 
 @pytest.mark.gpu
@@ -529,3 +531,40 @@ def test_truncated_sampler_off_equals_plain_and_seeded_draw():
     ta, _ = sample_filtered(x, us, SC, 0.9, 40, 0.8)
     tb, _ = sample_filtered(x, None, SC, 0.9, 40, 0.8, seed=7, req_id=req, tok_idx=ti)
     assert torch.equal(ta, tb)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,N", [(5, 640, 656), (128, 640, 3328), (200, 512, 640), (70, 1664, 640)])
+def test_skinny_gemm_norm_and_resid_fusions(dtype, M, K, N):
+    """norm_eps: the product of the RMS-normalised rows, against float64 (rmsnorm(a) @ w.T without intermediate rounding -
+    the kernel applies the norm as an exact row scale); RESID: ca * r + cb * round(a @ w.T), rounded; and both with SwiGLU."""
+    from ultraviolet_amd.kernels.gemm import RESID, SWIGLU, gemm_tn, interleave_gate_up
+    g = torch.Generator(device="cuda").manual_seed(M + N)
+    a = (torch.randn(M, K, device="cuda", generator=g) * 3).to(dtype)
+    w = (torch.randn(N, K, device="cuda", generator=g) / K ** 0.5).to(dtype)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    eps = 1e-6
+    ad = a.double()
+    an = ad * torch.rsqrt((ad * ad).mean(-1, keepdim=True) + eps)
+    ref = an @ w.double().t()
+    tol = ulp * ref.abs().clamp_min(1.0) + 1e-5 * K ** 0.5
+    r = torch.randn(M, N, device="cuda", generator=g).to(dtype)
+    prod = (ad @ w.double().t()).to(dtype).double()
+    want = 0.75 * r.double() + 1.25 * prod
+    tol2 = ulp * want.abs().clamp_min(1.0) + 1.25 * 2 * ulp * prod.abs().clamp_min(1.0)
+    for config in (1, 2):
+        out = gemm_tn(a, w, norm_eps=eps, config=config)
+        assert bool(((out.double() - ref).abs() <= tol).all()), (config, float((out.double() - ref).abs().max()))
+        got = gemm_tn(a, w, epilogue=RESID, resid=r, ca=0.75, cb=1.25, config=config)
+        assert bool(((got.double() - want).abs() <= tol2).all()), (config, float((got.double() - want).abs().max()))
+    if K <= 960 and N % 32 == 0:
+        f = N // 2
+        wg, wu = w[:f].contiguous(), w[f:].contiguous()
+        gg = (an @ wg.double().t()).to(dtype).double()
+        uu = (an @ wu.double().t()).to(dtype).double()
+        ra = (gg * torch.sigmoid(gg)).to(dtype).double() * uu
+        tol3 = 4 * ulp * ra.abs().clamp_min(1.0) + 4 * ulp * (gg.abs() + uu.abs())
+        for config in (1, 2):
+            act = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU, norm_eps=eps, config=config)
+            assert bool(((act.double() - ra).abs() <= tol3).all()), (config, float((act.double() - ra).abs().max()))

@@ -48,6 +48,12 @@ class AttnQkvFuse(C.Structure):
                 ("n_pairs", C.c_int), ("rope", C.c_int), ("eps", C.c_float), ("xsa_eps", C.c_float)]
 
 
+class GemmArgs(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("w", C.c_void_p), ("c", C.c_void_p), ("dtype", C.c_int), ("M", C.c_int64), ("N", C.c_int),
+                ("K", C.c_int), ("lda", C.c_int64), ("ldw", C.c_int64), ("ldc", C.c_int64), ("epilogue", C.c_int), ("norm_a", C.c_int),
+                ("eps", C.c_float), ("resid", C.c_void_p), ("ldr", C.c_int64), ("ca", C.c_float), ("cb", C.c_float), ("config", C.c_int)]
+
+
 class PrefillAttnArgs(C.Structure):
     _fields_ = [("q", C.c_void_p), ("q_dtype", C.c_int), ("sqn", C.c_int64), ("sqh", C.c_int64),
                 ("k", C.c_void_p), ("v", C.c_void_p), ("kv_dtype", C.c_int),
@@ -144,6 +150,7 @@ def lib() -> C.CDLL:
         L.uvmi_sched_expand.argtypes = [C.POINTER(SchedState), C.c_int, C.c_int] + [C.c_void_p] * 8
         L.uvmi_rope_table.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
         L.uvmi_gemm_tn_supported.argtypes = [C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]
+        L.uvmi_gemm_tn_ex.argtypes = [C.POINTER(GemmArgs), C.c_void_p]
         L.uvmi_gemm_tn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int64,
                                    C.c_int64, C.c_int, C.c_void_p]
         _lib = L
@@ -172,4 +179,4 @@ EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu",
-           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn"]
+           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]

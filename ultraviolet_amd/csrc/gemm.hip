@@ -20,7 +20,14 @@
 //     on one XCD and the strip leaves HBM once;
 //   * epilogue SWIGLU: W holds w_gate and w_up interleaved in slabs of 16 rows, so with BN = 32 accumulator 0 is gate and
 //     accumulator 1 is up of the same 16 output columns, and act = silu(g) * u is formed in registers with the roundings
-//     of the separate SwiGLU pass (g, u and silu(g) rounded to the activation type): the (M, 2f) intermediate never exists.
+//     of the separate SwiGLU pass (g, u and silu(g) rounded to the activation type): the (M, 2f) intermediate never exists;
+//   * epilogue RESID: C = ca * R + cb * (A W^T) with a residual input R (M, N), the block's residual update
+//     (ultraviolet/model.py:567-571) in the arithmetic of the separate residual-add kernel (the product rounded to the
+//     activation type first, then the sum rounded);
+//   * NORM: the activation rows are RMS-normalised on the fly.  RMSNorm has no weight here, so norm(a) W^T = rsqrt(mean(a^2)
+//     + eps) * (a W^T): the kernel sums a^2 of its rows as their K-steps pass through the ring and scales the accumulator
+//     once at the end - the normalised activations are never written (nor rounded to the activation type: the result is
+//     the exact row scale of the un-normalised product, a rounding step closer to exact than the two-pass path).
 #include "common.h"
 
 namespace uvmi {
@@ -65,14 +72,28 @@ template <int DT> __device__ __forceinline__ uint32_t gpack(float a, float b) {
 
 constexpr int SK_BM = 64;       // rows per workgroup
 constexpr int SK_RING = 16;     // activation K-steps (of 32) in flight per wave
+// problems of at most this many 16-row x BN tiles split K over the waves of 16-row workgroups (measured on 640 / 1664-deep
+// projections: faster up to ~500 workgroups, two per compute unit; beyond, the weight strips are re-read too often)
+constexpr int SK_KSPLIT_TILES = 512;
 constexpr int SK_WPASS = 16;    // most passes of the weight-strip load (32 (row, 128-byte segment) units per pass)
 
+__device__ __forceinline__ float gxsum16(float v) {  // v + the value of lane l ^ 16
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float gxsum32(float v) {  // v + the value of lane l ^ 32
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // EPI 0: C = A W^T (M, N).  EPI 1 (BN = 32): W rows are [gate 16 | up 16] slabs; C = silu(gate) * up, (M, N / 2).
+// EPI 2: C = ca * R + cb * (A W^T).  NORM: A stands for its RMS-normalised rows.
 // (individual scalar arguments rather than a parameter block: they are preloaded into SGPRs with the wave, so the first
 // loads need not wait for a load of the kernel arguments)
-template <int DT, int BN, int EPI>
+template <int DT, int BN, int EPI, bool NORM>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const void* a_w, void* a_c, uint32_t a_lda2, uint32_t a_ldw2,
-                                                          int a_M, int a_N, int a_K, int a_tiles_m, int a_tiles_n, int64_t a_ldc) {
+                                                          int a_M, int a_N, int a_K, int a_tiles_m, int a_tiles_n, int64_t a_ldc,
+                                                          float a_eps, const void* a_res, int64_t a_ldr, float a_ca, float a_cb) {
   SkinnyParams P;
   P.a = a_a; P.w = a_w; P.c = a_c; P.lda2 = a_lda2; P.ldw2 = a_ldw2; P.ldc = a_ldc; P.M = a_M; P.N = a_N; P.K = a_K;
   P.tiles_m = a_tiles_m; P.tiles_n = a_tiles_n;
@@ -132,12 +153,23 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const
 #pragma unroll
   for (int j = 0; j < TN; j++) acc[j] = gf4{0.f, 0.f, 0.f, 0.f};
   const unsigned char* wop = wlds + r * pitch + 16 * g;  // operand read: row r of a 16-row slab, 16 bytes at k = 8 g
+  float ss = 0.f;  // NORM: sum of squares of this lane's quarter of row r
   auto step = [&](int s, gu4& slot) {
     gu4 w[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) w[j] = *(const gu4*)(wop + 16 * j * pitch + s * 64);
 #pragma unroll
     for (int j = 0; j < TN; j++) acc[j] = gmfma<DT>(w[j], slot, acc[j]);
+    if (NORM) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        float lo, hi;
+        if (DT == UVMI_BF16) { lo = __uint_as_float(slot[i] << 16); hi = __uint_as_float(slot[i] & 0xffff0000u); }
+        else { lo = half_bits_to_float((uint16_t)(slot[i] & 0xffff)); hi = half_bits_to_float((uint16_t)(slot[i] >> 16)); }
+        ss = fmaf(lo, lo, ss);
+        ss = fmaf(hi, hi, ss);
+      }
+    }
     slot = request(s + SK_RING);
   };
   // whole turns of the ring run in a loop whose body has no branches, which keeps the wait before a step at "all but the
@@ -151,9 +183,36 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const
   for (int d = 0; d < SK_RING - 1; d++)
     if (s + d < ns) step(s + d, ring[d]);  // workgroup-uniform
 
-  // accumulator j: lane (r, g) holds C[m0 + 16 wave + r][n0 + 16 j + 4 g + t], t = 0..3
+  // accumulator j: lane (r, g) holds C[m0 + 16 wave + r][n0 + 16 j + 4 g + t], t = 0..3: the same row r whose quarter the
+  // lane summed, so the row scale needs the 4 lane groups' sums and nothing else
+  if (NORM) {
+    ss = gxsum32(gxsum16(ss));
+    const float rn = rsqrtf(ss / (float)P.K + a_eps);
+#pragma unroll
+    for (int j = 0; j < TN; j++) acc[j] *= rn;
+  }
   if (arow >= P.M) return;
-  if (EPI == 0) {
+  if (EPI == 2) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int n = n0 + 16 * j;
+      if (n >= P.N) continue;
+      const gf4 v = acc[j];
+      const uint2 rw = *(const uint2*)((const uint16_t*)a_res + (int64_t)arow * a_ldr + n + 4 * g);
+      float x[4], o[4];
+      if (DT == UVMI_BF16) {
+        x[0] = __uint_as_float(rw.x << 16); x[1] = __uint_as_float(rw.x & 0xffff0000u);
+        x[2] = __uint_as_float(rw.y << 16); x[3] = __uint_as_float(rw.y & 0xffff0000u);
+      } else {
+        x[0] = half_bits_to_float((uint16_t)(rw.x & 0xffff)); x[1] = half_bits_to_float((uint16_t)(rw.x >> 16));
+        x[2] = half_bits_to_float((uint16_t)(rw.y & 0xffff)); x[3] = half_bits_to_float((uint16_t)(rw.y >> 16));
+      }
+#pragma unroll
+      for (int t = 0; t < 4; t++) o[t] = a_ca * x[t] + a_cb * ground<DT>(v[t]);
+      uint16_t* cp = (uint16_t*)P.c + (int64_t)arow * P.ldc + n + 4 * g;
+      *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};
+    }
+  } else if (EPI == 0) {
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       const int n = n0 + 16 * j;
@@ -163,7 +222,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const
       *(uint2*)cp = uint2{gpack<DT>(v[0], v[1]), gpack<DT>(v[2], v[3])};
     }
   } else {
-    static_assert(EPI == 0 || BN == 32, "the SwiGLU epilogue pairs two 16-row slabs");
+    static_assert(EPI != 1 || BN == 32, "the SwiGLU epilogue pairs two 16-row slabs");
     if (n0 < P.N) {
       const gf4 gt = acc[0], up = acc[TN - 1];
       float o[4];
@@ -173,6 +232,164 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const
         o[t] = ground<DT>(gv / (1.0f + __expf(-gv))) * uv;
       }
       uint16_t* cp = (uint16_t*)P.c + (int64_t)arow * P.ldc + (n0 >> 1) + 4 * g;
+      *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};
+    }
+  }
+}
+
+
+// The same product for the smallest steps, where a 64-row workgroup would leave most compute units idle and every wave
+// would walk all of K: a workgroup owns 16 rows x BN columns and its 4 waves split K in quarters.  Each wave requests its
+// quarter of the weight strip (4 consecutive lanes on 64 bytes of a weight row) and of the 16 activation rows in one
+// burst, parks its own strip quarter in its own LDS region (no workgroup barrier before the loop), multiplies, and the four
+// partial accumulators (and, with NORM, partial sums of squares) meet in LDS, where the first wave adds them and runs the
+// epilogue.  K % 128 == 0, K / 4 <= 512.
+template <int DT, int BN, int EPI, bool NORM>
+__global__ __launch_bounds__(256) void gemm_skinny_ksplit_kernel(const void* a_a, const void* a_w, void* a_c, uint32_t a_lda2, uint32_t a_ldw2,
+                                                                 int a_M, int a_N, int a_K, int a_tiles_m, int a_tiles_n, int64_t a_ldc,
+                                                                 float a_eps, const void* a_res, int64_t a_ldr, float a_ca, float a_cb) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];  // 4 x [BN rows of K / 2 + 16 bytes], then the partials
+  constexpr int TN = BN / 16;
+  constexpr int RP = BN / 16;                 // row passes of the strip load (16 rows per pass)
+  constexpr int MAXCP = 16 / RP;              // most chunk passes (4 chunks of 16 bytes per pass)
+  constexpr int MAXS = 16;                    // most K-steps per wave
+  constexpr uint32_t OOB = 0x40000000u;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int T = a_tiles_m * a_tiles_n;
+  const int per = (T + 7) / 8;
+  const int L = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+  if (L >= T) return;
+  const int bn = L / a_tiles_m, bm = L % a_tiles_m;
+  const int m0 = bm * 16, n0 = bn * BN;
+  const int r = lane & 15, g = lane >> 4;
+  const int nsw = a_K / 128;                  // K-steps (of 32) per wave
+  const int kq2 = a_K / 2;                    // bytes of a row's K quarter
+  const uint32_t pitch = (uint32_t)kq2 + 16;
+  const int cps = kq2 / 64;                   // chunk passes: 64 bytes (4 lanes) of a weight row per pass
+  const uint32_t kbase = (uint32_t)wave * (uint32_t)kq2;  // byte offset of this wave's quarter inside a row
+
+  const uint32_t boundA = (uint32_t)(a_M - 1) * a_lda2 + (uint32_t)a_K * 2;
+  const uint32_t boundW = (uint32_t)(a_N - 1) * a_ldw2 + (uint32_t)a_K * 2;
+  const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc((void*)a_a, 0, (int)boundA, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rW = __builtin_amdgcn_make_buffer_rsrc((void*)a_w, 0, (int)boundW, 0x00020000);
+
+  // ---- this wave's quarter of the weight strip: lane -> row (lane / 4) + 16 j, bytes 16 (lane % 4) + 64 i of the quarter
+  const int wr = lane >> 2, wc = lane & 3;
+  gu4 wst[RP][MAXCP];
+#pragma unroll
+  for (int j = 0; j < RP; j++) {
+    const int row = n0 + wr + 16 * j;
+    const uint32_t base = (row < a_N ? 0u : OOB) + (uint32_t)row * a_ldw2 + kbase + 16 * wc;
+#pragma unroll
+    for (int i = 0; i < MAXCP; i++) wst[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rW, base + (i < cps ? (uint32_t)i * 64 : OOB), 0, 0);
+  }
+  // ---- this wave's quarter of the 16 activation rows, in MFMA operand order: lane (r, g) = row r, k = 32 s + 8 g ..
+  const int arow = m0 + r;
+  const uint32_t abase = (arow < a_M ? 0u : OOB) + (uint32_t)arow * a_lda2 + kbase + 16 * g;
+  gu4 av[MAXS];
+#pragma unroll
+  for (int s = 0; s < MAXS; s++) av[s] = __builtin_amdgcn_raw_buffer_load_b128(rA, abase + (s < nsw ? (uint32_t)s * 64 : OOB), 0, 0);
+
+  unsigned char* mine = wlds + (size_t)wave * BN * pitch;
+#pragma unroll
+  for (int j = 0; j < RP; j++)
+#pragma unroll
+    for (int i = 0; i < MAXCP; i++)
+      if (i < cps) *(gu4*)(mine + (wr + 16 * j) * pitch + 64 * i + 16 * wc) = wst[j][i];
+  __builtin_amdgcn_wave_barrier();  // the region is this wave's own: its LDS operations complete in order
+
+  gf4 acc[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) acc[j] = gf4{0.f, 0.f, 0.f, 0.f};
+  float ss = 0.f;
+  const unsigned char* wop = mine + r * pitch + 16 * g;
+#pragma unroll
+  for (int s = 0; s < MAXS; s++) {
+    if (s < nsw) {  // workgroup-uniform
+      gu4 w[TN];
+#pragma unroll
+      for (int j = 0; j < TN; j++) w[j] = *(const gu4*)(wop + 16 * j * pitch + s * 64);
+#pragma unroll
+      for (int j = 0; j < TN; j++) acc[j] = gmfma<DT>(w[j], av[s], acc[j]);
+      if (NORM) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float lo, hi;
+          if (DT == UVMI_BF16) { lo = __uint_as_float(av[s][i] << 16); hi = __uint_as_float(av[s][i] & 0xffff0000u); }
+          else { lo = half_bits_to_float((uint16_t)(av[s][i] & 0xffff)); hi = half_bits_to_float((uint16_t)(av[s][i] >> 16)); }
+          ss = fmaf(lo, lo, ss);
+          ss = fmaf(hi, hi, ss);
+        }
+      }
+    }
+  }
+  // ---- the four partial results meet in LDS; the first wave adds them (in wave order) and finishes
+  float* red = (float*)(wlds + (size_t)4 * BN * pitch);   // [4 waves][TN * 4 + 1][64 lanes]
+  constexpr int RW = TN * 4 + 1;
+#pragma unroll
+  for (int j = 0; j < TN; j++)
+#pragma unroll
+    for (int t = 0; t < 4; t++) red[(wave * RW + j * 4 + t) * 64 + lane] = acc[j][t];
+  if (NORM) red[(wave * RW + TN * 4) * 64 + lane] = ss;
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 1; w < 4; w++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int t = 0; t < 4; t++) acc[j][t] += red[(w * RW + j * 4 + t) * 64 + lane];
+    if (NORM) ss += red[(w * RW + TN * 4) * 64 + lane];
+  }
+  if (NORM) {
+    ss = gxsum32(gxsum16(ss));
+    const float rn = rsqrtf(ss / (float)a_K + a_eps);
+#pragma unroll
+    for (int j = 0; j < TN; j++) acc[j] *= rn;
+  }
+  if (arow >= a_M) return;
+  if (EPI == 2) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int n = n0 + 16 * j;
+      if (n >= a_N) continue;
+      const gf4 v = acc[j];
+      const uint2 rw = *(const uint2*)((const uint16_t*)a_res + (int64_t)arow * a_ldr + n + 4 * g);
+      float x[4], o[4];
+      if (DT == UVMI_BF16) {
+        x[0] = __uint_as_float(rw.x << 16); x[1] = __uint_as_float(rw.x & 0xffff0000u);
+        x[2] = __uint_as_float(rw.y << 16); x[3] = __uint_as_float(rw.y & 0xffff0000u);
+      } else {
+        x[0] = half_bits_to_float((uint16_t)(rw.x & 0xffff)); x[1] = half_bits_to_float((uint16_t)(rw.x >> 16));
+        x[2] = half_bits_to_float((uint16_t)(rw.y & 0xffff)); x[3] = half_bits_to_float((uint16_t)(rw.y >> 16));
+      }
+#pragma unroll
+      for (int t = 0; t < 4; t++) o[t] = a_ca * x[t] + a_cb * ground<DT>(v[t]);
+      uint16_t* cp = (uint16_t*)a_c + (int64_t)arow * a_ldc + n + 4 * g;
+      *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};
+    }
+  } else if (EPI == 0) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int n = n0 + 16 * j;
+      if (n >= a_N) continue;
+      const gf4 v = acc[j];
+      uint16_t* cp = (uint16_t*)a_c + (int64_t)arow * a_ldc + n + 4 * g;
+      *(uint2*)cp = uint2{gpack<DT>(v[0], v[1]), gpack<DT>(v[2], v[3])};
+    }
+  } else {
+    static_assert(EPI != 1 || BN == 32, "the SwiGLU epilogue pairs two 16-row slabs");
+    if (n0 < a_N) {
+      const gf4 gt = acc[0], up = acc[TN - 1];
+      float o[4];
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const float gv = ground<DT>(gt[t]), uv = ground<DT>(up[t]);
+        o[t] = ground<DT>(gv / (1.0f + __expf(-gv))) * uv;
+      }
+      uint16_t* cp = (uint16_t*)a_c + (int64_t)arow * a_ldc + (n0 >> 1) + 4 * g;
       *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};
     }
   }
@@ -190,7 +407,7 @@ static int skinny_bn(int K, int epilogue) {  // widest strip that fits 64 KB of 
 
 extern "C" int uvmi_gemm_tn_supported(int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue) {
   if (dtype != UVMI_F16 && dtype != UVMI_BF16) return 0;
-  if (epilogue != UVMI_GEMM_STORE && epilogue != UVMI_GEMM_SWIGLU) return 0;
+  if (epilogue != UVMI_GEMM_STORE && epilogue != UVMI_GEMM_SWIGLU && epilogue != UVMI_GEMM_RESID) return 0;
   if (M < 0 || M > (1 << 16) || N <= 0 || K <= 0 || K % 64 != 0 || skinny_bn(K, epilogue) == 0) return 0;
   if (N % (epilogue == UVMI_GEMM_SWIGLU ? 32 : 16) != 0) return 0;
   if (lda < K || ldw < K || lda % 8 != 0 || ldw % 8 != 0 || ldc % 4 != 0) return 0;
@@ -199,36 +416,65 @@ extern "C" int uvmi_gemm_tn_supported(int dtype, int64_t M, int N, int K, int64_
   return 1;
 }
 
-extern "C" int uvmi_gemm_tn(const void* a, const void* w, void* c, int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw,
-                            int64_t ldc, int epilogue, void* stream) {
-  UVMI_REQUIRE(a && w && c, UVMI_EINVAL, "uvmi_gemm_tn: null pointer");
-  UVMI_REQUIRE(uvmi_gemm_tn_supported(dtype, M, N, K, lda, ldw, ldc, epilogue), UVMI_EUNSUPPORTED,
+template <int DT, int BN>
+static void launch_skinny(const uvmi_gemm_args* a, const SkinnyParams& P, dim3 grid, size_t lds, hipStream_t st, bool ksplit) {
+  const dim3 blk(256);
+#define UVMI_GO(EPI, NORM)                                                                                                             \
+  do {                                                                                                                                 \
+    if (ksplit)                                                                                                                        \
+      hipLaunchKernelGGL((gemm_skinny_ksplit_kernel<DT, BN, EPI, NORM>), grid, blk, lds, st, P.a, P.w, P.c, P.lda2, P.ldw2, P.M, P.N,  \
+                         P.K, P.tiles_m, P.tiles_n, P.ldc, a->eps, a->resid, a->ldr, a->ca, a->cb);                                    \
+    else                                                                                                                               \
+      hipLaunchKernelGGL((gemm_skinny_kernel<DT, BN, EPI, NORM>), grid, blk, lds, st, P.a, P.w, P.c, P.lda2, P.ldw2, P.M, P.N, P.K,    \
+                         P.tiles_m, P.tiles_n, P.ldc, a->eps, a->resid, a->ldr, a->ca, a->cb);                                         \
+  } while (0)
+  const bool norm = a->norm_a != 0;
+  if (a->epilogue == UVMI_GEMM_RESID) { if (norm) UVMI_GO(2, true); else UVMI_GO(2, false); }
+  else if (a->epilogue == UVMI_GEMM_SWIGLU) {
+    if constexpr (BN == 32) { if (norm) UVMI_GO(1, true); else UVMI_GO(1, false); }
+  } else { if (norm) UVMI_GO(0, true); else UVMI_GO(0, false); }
+#undef UVMI_GO
+}
+
+extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
+  UVMI_REQUIRE(a && a->a && a->w && a->c, UVMI_EINVAL, "uvmi_gemm_tn: null pointer");
+  UVMI_REQUIRE(uvmi_gemm_tn_supported(a->dtype, a->M, a->N, a->K, a->lda, a->ldw, a->ldc, a->epilogue), UVMI_EUNSUPPORTED,
                "uvmi_gemm_tn: unsupported problem (dtype %d, M %lld, N %d, K %d, lda %lld, ldw %lld, ldc %lld, epilogue %d): needs F16 / BF16, "
                "K %% 64 == 0, K <= 1984 (960 with SWIGLU), N %% 16 == 0 (32 with SWIGLU), lda, ldw %% 8 == 0, ldc %% 4 == 0",
-               dtype, (long long)M, N, K, (long long)lda, (long long)ldw, (long long)ldc, epilogue);
-  UVMI_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)c % 8) == 0, UVMI_EINVAL, "uvmi_gemm_tn: misaligned pointer");
-  if (M == 0) return UVMI_OK;
-  const int BN = skinny_bn(K, epilogue);
+               a->dtype, (long long)a->M, a->N, a->K, (long long)a->lda, (long long)a->ldw, (long long)a->ldc, a->epilogue);
+  UVMI_REQUIRE(((uintptr_t)a->a % 16) == 0 && ((uintptr_t)a->w % 16) == 0 && ((uintptr_t)a->c % 8) == 0, UVMI_EINVAL, "uvmi_gemm_tn: misaligned pointer");
+  if (a->epilogue == UVMI_GEMM_RESID)
+    UVMI_REQUIRE(a->resid && ((uintptr_t)a->resid % 8) == 0 && a->ldr % 4 == 0 && a->ldr >= a->N, UVMI_EINVAL,
+                 "uvmi_gemm_tn: the RESID epilogue needs an 8-byte aligned residual with a pitch that is a multiple of 4 and >= N");
+  UVMI_REQUIRE(!a->norm_a || a->eps >= 0.f, UVMI_EINVAL, "uvmi_gemm_tn: negative eps");
+  if (a->M == 0) return UVMI_OK;
+  const int BN = skinny_bn(a->K, a->epilogue);
+  // the smallest problems split K over the waves of a 16-row workgroup (more, shorter workgroups); config forces a form
+  const bool can_split = a->K % 128 == 0;
+  const int64_t t_split = ((a->M + 15) / 16) * ((a->N + BN - 1) / BN);
+  const bool ksplit = a->config == 2 ? can_split : (a->config == 1 ? false : (can_split && t_split <= SK_KSPLIT_TILES));
   SkinnyParams P;
-  P.a = a; P.w = w; P.c = c; P.lda2 = (uint32_t)lda * 2; P.ldw2 = (uint32_t)ldw * 2; P.ldc = ldc; P.M = (int)M; P.N = N; P.K = K;
-  P.tiles_m = (int)((M + SK_BM - 1) / SK_BM);
-  P.tiles_n = (N + BN - 1) / BN;
+  P.a = a->a; P.w = a->w; P.c = a->c; P.lda2 = (uint32_t)a->lda * 2; P.ldw2 = (uint32_t)a->ldw * 2; P.ldc = a->ldc;
+  P.M = (int)a->M; P.N = a->N; P.K = a->K;
+  const int bm = ksplit ? 16 : SK_BM;
+  P.tiles_m = (int)((a->M + bm - 1) / bm);
+  P.tiles_n = (a->N + BN - 1) / BN;
   const int T = P.tiles_m * P.tiles_n;
-  const dim3 grid((unsigned)(((T + 7) / 8) * 8)), blk(256);
-  const size_t lds = (size_t)BN * ((size_t)K * 2 + 16);  // at most 32 * 1936 = 62 KB, 16 * 3984 = 64 KB
+  const dim3 grid((unsigned)(((T + 7) / 8) * 8));
+  // one strip: at most 32 * 1936 = 62 KB, 16 * 3984 = 64 KB; split: the strip in four regions with their own padding + 9 KB
+  const size_t lds = ksplit ? (size_t)4 * BN * ((size_t)a->K / 2 + 16) + (size_t)4 * (BN / 16 * 4 + 1) * 256
+                            : (size_t)BN * ((size_t)a->K * 2 + 16);
   hipStream_t st = (hipStream_t)stream;
-  auto go = [&](auto kern) {
-    hipLaunchKernelGGL(kern, grid, blk, lds, st, P.a, P.w, P.c, P.lda2, P.ldw2, P.M, P.N, P.K, P.tiles_m, P.tiles_n, P.ldc);
-  };
-  if (dtype == UVMI_F16) {
-    if (epilogue == UVMI_GEMM_SWIGLU) go(gemm_skinny_kernel<UVMI_F16, 32, 1>);
-    else if (BN == 32) go(gemm_skinny_kernel<UVMI_F16, 32, 0>);
-    else go(gemm_skinny_kernel<UVMI_F16, 16, 0>);
-  } else {
-    if (epilogue == UVMI_GEMM_SWIGLU) go(gemm_skinny_kernel<UVMI_BF16, 32, 1>);
-    else if (BN == 32) go(gemm_skinny_kernel<UVMI_BF16, 32, 0>);
-    else go(gemm_skinny_kernel<UVMI_BF16, 16, 0>);
-  }
+  if (a->dtype == UVMI_F16) { if (BN == 32) launch_skinny<UVMI_F16, 32>(a, P, grid, lds, st, ksplit); else launch_skinny<UVMI_F16, 16>(a, P, grid, lds, st, ksplit); }
+  else { if (BN == 32) launch_skinny<UVMI_BF16, 32>(a, P, grid, lds, st, ksplit); else launch_skinny<UVMI_BF16, 16>(a, P, grid, lds, st, ksplit); }
   UVMI_CHECK_LAUNCH("uvmi_gemm_tn");
   return UVMI_OK;
+}
+
+extern "C" int uvmi_gemm_tn(const void* a, const void* w, void* c, int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw,
+                            int64_t ldc, int epilogue, void* stream) {
+  uvmi_gemm_args g = {};
+  g.a = a; g.w = w; g.c = c; g.dtype = dtype; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.epilogue = epilogue;
+  UVMI_REQUIRE(epilogue != UVMI_GEMM_RESID, UVMI_EINVAL, "uvmi_gemm_tn: the RESID epilogue takes its residual through uvmi_gemm_tn_ex");
+  return uvmi_gemm_tn_ex(&g, stream);
 }

@@ -19,7 +19,7 @@ from torch import Tensor
 from .. import _lib as L
 from ..kernels.decode_attn import (build_attn_args, build_fused_args, decode_attention, decode_attention_fused, decode_attention_post,
                                    rope_table)
-from ..kernels.gemm import SWIGLU, gemm_tn
+from ..kernels.gemm import RESID, SWIGLU, gemm_tn
 from ..kernels.kv_quant import kv_write
 from ..kernels.varlen_attn import packed_attention
 from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
@@ -280,11 +280,21 @@ class UVEngine:
         x, xn = b["x"][:n], b["xn"][:n]
         skinny = n <= self.skinny_rows and cfg.d_model % 64 == 0 and cfg.d_model <= 960 and (cfg.n_heads * cfg.head_dim) % 64 == 0
         mm = (lambda a, w, out: gemm_tn(a, w, out)) if skinny else (lambda a, w, out: torch.mm(a, w.t(), out=out))
+        # Small passes whose every layer takes the fused attention never need the normalised hidden in memory: the block's
+        # second residual update then rides on the down projection and the next block's pre-norm on its QKV projection (a row
+        # scale of the product), and only the final norm is a launch of its own.
+        lean = (skinny and fused_attn is not None and os.environ.get("UVMI_LEAN", "1") != "0"
+                and all("gu_il" in W and self.fused_layer_ok(l, st) for l, W in enumerate(self.w.layers))
+                and cfg.d_ff % 64 == 0 and cfg.d_ff <= 1984)
+        x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
                 # decode rows of a 16-bit engine: the projection also forms the gate logits, and fused_attn(l) does the
                 # post-processing, the cache append, the attention and its epilogue in one launch (writes buf zg)
-                mm(xn, W["wqkv_ext"], b["qkvx"][:n])
+                if x_is_normed:
+                    mm(xn, W["wqkv_ext"], b["qkvx"][:n])
+                else:
+                    gemm_tn(x, W["wqkv_ext"], b["qkvx"][:n], norm_eps=self.eps)
                 if self.qkvx_keep is not None:   # a benchmark re-issues this layer's launch later on the same projection
                     self.qkvx_keep[l][:n].copy_(b["qkvx"][:n])
                 fused_attn(l)
@@ -294,17 +304,28 @@ class UVEngine:
                 z = attn(l, b["q"][:n])
                 if z is not None:   # None: the attention kernel already applied XSA + gate and wrote buf zg
                     self._attn_post(l, z, n)
-            mm(b["zg"][:n], W["wo"], b["a"][:n])
-            # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
-            self._add_norm(x, b["a"][:n], W["resid_attn"], W["post_attn"], n, b["h"], b["xn"])
             if skinny and "gu_il" in W:
-                gemm_tn(xn, W["gu_il"], b["act"][:n], epilogue=SWIGLU)
+                # the residual update rides on the output projection (h = resid_attn * x + post_attn * a) and the MLP's
+                # pre-norm on the gate-up projection (a row scale of the product), whose epilogue is the SwiGLU: two
+                # launches where the general path has five
+                gemm_tn(b["zg"][:n], W["wo"], b["h"][:n], epilogue=RESID, resid=x, ca=W["resid_attn"], cb=W["post_attn"])
+                gemm_tn(b["h"][:n], W["gu_il"], b["act"][:n], epilogue=SWIGLU, norm_eps=self.eps)
             else:
+                mm(b["zg"][:n], W["wo"], b["a"][:n])
+                # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
+                self._add_norm(x, b["a"][:n], W["resid_attn"], W["post_attn"], n, b["h"], b["xn"])
                 mm(xn, W["gu"], b["gu"][:n])
                 self._swiglu(n)
-            torch.mm(b["act"][:n], W["down"].t(), out=b["m"][:n])   # (K = d_ff: 26 K-steps per strip, the library is faster)
-            # x = resid_mlp * h + post_mlp * m ; xn = rmsnorm(x) (next block's pre-norm, or the final norm)
-            self._add_norm(b["h"][:n], b["m"][:n], W["resid_mlp"], W["post_mlp"], n, b["x"], b["xn"])
+            if lean:
+                # x = resid_mlp * h + post_mlp * m in the down projection's epilogue (in place of the residual-add + norm launch)
+                gemm_tn(b["act"][:n], W["down"], x, epilogue=RESID, resid=b["h"][:n], ca=W["resid_mlp"], cb=W["post_mlp"])
+                x_is_normed = False
+            else:
+                torch.mm(b["act"][:n], W["down"].t(), out=b["m"][:n])   # (K = d_ff: 26 K-steps per strip, the library is faster)
+                # x = resid_mlp * h + post_mlp * m ; xn = rmsnorm(x) (next block's pre-norm, or the final norm)
+                self._add_norm(b["h"][:n], b["m"][:n], W["resid_mlp"], W["post_mlp"], n, b["x"], b["xn"])
+        if not x_is_normed:
+            self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
         return xn
 
     def head(self, hidden: Tensor) -> Tensor:
