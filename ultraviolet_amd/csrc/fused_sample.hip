@@ -72,9 +72,11 @@ __device__ __forceinline__ float e_of(float x, const SampleParams& P) {
 
 // (the row pointer's ingredients lead the argument list: leading scalar arguments are preloaded into SGPRs with the wave,
 // so the first loads of the row do not wait for a load of the kernel arguments)
-template <int DT>
-__global__ __launch_bounds__(256) void sample_kernel(const void* a_x, int64_t a_stride, int a_V, float a_inv_c_l2, float a_b_over_c_l2,
-                                                     float a_neg_a_over_t_l2, SampleParams P) {
+// NT threads per row: 256 when there are rows enough to fill the device, 1024 for small batches (the row's exponentials are
+// the work of the launch; with one small workgroup per row and fewer rows than compute units most of the device would idle)
+template <int DT, int NT>
+__global__ __launch_bounds__(NT) void sample_kernel(const void* a_x, int64_t a_stride, int a_V, float a_inv_c_l2, float a_b_over_c_l2,
+                                                    float a_neg_a_over_t_l2, SampleParams P) {
   P.x = a_x; P.stride = a_stride; P.V = a_V; P.inv_c_l2 = a_inv_c_l2; P.b_over_c_l2 = a_b_over_c_l2; P.neg_a_over_t_l2 = a_neg_a_over_t_l2;
   __shared__ float csum[64 + 4];
   __shared__ int sh_chunk;
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256) void sample_kernel(const void* a_x, int64_t a_
   const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const char* xr = (const char*)P.x + (int64_t)row * P.stride * (DT == UVMI_F32 ? 4 : 2);
   const int nchunks = P.V / CHUNK;  // host guarantees V % 512 == 0 and nchunks <= 64
-  for (int c = wave; c < nchunks; c += 4) {
+  for (int c = wave; c < nchunks; c += NT / 64) {
     float v[8];
     load8<DT>(xr, c * 64 + lane, v);
     float s = 0.f;
@@ -474,12 +476,13 @@ extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
   if (greedy) UVMI_S(argmax_kernel);
   else if (filtered) UVMI_S(sample_filtered_kernel);
   else {
-    if (a->x_dtype == UVMI_F16)
-      hipLaunchKernelGGL((sample_kernel<UVMI_F16>), grid, blk, 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P);
-    else if (a->x_dtype == UVMI_BF16)
-      hipLaunchKernelGGL((sample_kernel<UVMI_BF16>), grid, blk, 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P);
-    else
-      hipLaunchKernelGGL((sample_kernel<UVMI_F32>), grid, blk, 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P);
+#define UVMI_SK(DT, NT) \
+  hipLaunchKernelGGL((sample_kernel<DT, NT>), grid, dim3(NT), 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P)
+    const bool wide = a->B <= 256;  // (the chunk sums are formed per chunk whatever the width: the draw does not depend on it)
+    if (a->x_dtype == UVMI_F16) { if (wide) UVMI_SK(UVMI_F16, 1024); else UVMI_SK(UVMI_F16, 256); }
+    else if (a->x_dtype == UVMI_BF16) { if (wide) UVMI_SK(UVMI_BF16, 1024); else UVMI_SK(UVMI_BF16, 256); }
+    else { if (wide) UVMI_SK(UVMI_F32, 1024); else UVMI_SK(UVMI_F32, 256); }
+#undef UVMI_SK
   }
 #undef UVMI_S
   UVMI_CHECK_LAUNCH("uvmi_fused_sample");
