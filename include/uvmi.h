@@ -311,6 +311,13 @@ int uvmi_attn_post(const void* z, int z_dtype, const void* v, const void* xn, in
 /* SwiGLU after the fused gate/up GEMM (ultraviolet/model.py:388-391): out[r, j] = silu(gu[r, j]) * gu[r, f + j]. */
 int uvmi_swiglu(const void* gu, int dtype, int64_t rows, int f, void* out, void* stream);
 
+/* The same with the MLP's pre-norm folded in (ultraviolet/model.py:570 n = norm(h), then 388-391): gu (rows, 2 f) is the
+ * gate/up product of the UN-normalised hidden h (rows, d); with rn[r] = rsqrt(mean(h[r]^2) + eps),
+ * out[r, j] = silu(rn gu[r, j]) * (rn gu[r, f + j]) - the row scale commutes with the product, so the normalised hidden
+ * is never written.  f % 8 == 0, d % 2 == 0. */
+int uvmi_swiglu_norm(const void* gu, const void* h, int dtype, int64_t rows, int f, int d, float eps, void* out,
+                     void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------
  * On-device continuous batching: the slot table of generate_continuous (ultraviolet/model.py:1283-1350) and
  * StreamGen (scripts/rl_stream.py:55-146) kept in device memory.  All arrays are caller-owned.

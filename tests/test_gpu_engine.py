@@ -114,10 +114,22 @@ def test_greedy_64_tokens_identical_fp32(name, over):
     assert identical >= len(prompts) - 2, identical
 
 
-def test_bf16_engine_close_to_oracle():
+# the decode pass's launch plans by row count, forced here at a few rows: (skinny_rows, fold_qkv_rows, fold_o_rows)
+_TRUNK_PLANS = {"small": None, "large-skinny-attn-block": (0, 1 << 30, 1 << 30), "large-library": (0, 0, 0)}
+
+
+def _force_plan(eng, plan):
+    if _TRUNK_PLANS[plan] is not None:
+        eng.skinny_rows, eng.fold_qkv_rows, eng.fold_o_rows = _TRUNK_PLANS[plan]
+
+
+@pytest.mark.parametrize("plan", list(_TRUNK_PLANS))
+def test_bf16_engine_close_to_oracle(plan):
     """reference bar for the int8 kernel path vs its SDPA path: max |logit diff| < 0.25, argmax agreement > 0.9
-    (tests/test_math_kernels.py:170-172)."""
+    (tests/test_math_kernels.py:170-172) - for each of the decode pass's launch plans (the one for few rows, and the two
+    for many rows: residual updates inside the projections, the MLP's pre-norm inside the SwiGLU launch)."""
     cfg, params, eng, OracleModel = _setup(dtype=torch.bfloat16, window=16)
+    _force_plan(eng, plan)
     prompts = _prompts(cfg, (5, 12, 9, 20, 3, 17))
     cont = np.random.default_rng(1).integers(1, cfg.vocab_size, size=(6, 30))
     lg, _ = _teacher_forced(eng, prompts, cont, 64)
@@ -325,6 +337,21 @@ def test_fused_qkv_decode_matches_unfused(dtype, name, over):
     hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=24)
     assert cmax[0] == 0 and sfrac[0] == 0
     # the perturbation grows layer by layer (16-bit activations: one unit in the last place of a key is half an int8 code)
+    assert (cmax <= 3 + np.arange(cfg.n_layers)).all(), cmax
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
+    assert np.mean(agree) > 0.9, np.mean(agree)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("plan", ["large-skinny-attn-block", "large-library"])
+def test_large_pass_plans_match_unfused(dtype, plan):
+    """The launch plans of passes with many rows (forced here at 6 rows) against the unfused general path, to the same
+    bounds as the small-pass plan above."""
+    cfg, params, eng, _ = _setup("uv-50m-alpha", dtype=dtype, perturb=0.05)
+    _force_plan(eng, plan)
+    hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=24)
+    assert cmax[0] == 0 and sfrac[0] == 0
     assert (cmax <= 3 + np.arange(cfg.n_layers)).all(), cmax
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     assert max(hdiff) < 16 * 2 * ulp, max(hdiff)

@@ -461,6 +461,33 @@ def test_skinny_gemm_swiglu_epilogue(dtype, M, K, f):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,f,d", [(1, 1664, 640), (300, 1664, 640), (37, 24, 10)])
+def test_swiglu_with_folded_prenorm(dtype, rows, f, d):
+    """uvmi_swiglu_norm(gu = h @ W.T, h) equals the SwiGLU of rmsnorm(h) @ W.T with the norm applied as a row scale of the
+    product (ultraviolet/model.py:570, 388-391): restated here with torch in the same rounding order; the row scale may
+    differ in its last fp32 place (summation order), which can move a rounded factor by one place of the activation type."""
+    from ultraviolet_amd import _lib as L
+    g = torch.Generator(device="cuda").manual_seed(rows + f)
+    h = (3.0 * torch.randn(rows, d, device="cuda", generator=g)).to(dtype)
+    gu = torch.randn(rows, 2 * f, device="cuda", generator=g).to(dtype)
+    eps = 1e-6
+    out = torch.full((rows + 1, f), 7.0, device="cuda", dtype=dtype)
+    code = L.dtype_code(dtype)
+    L.check(L.lib().uvmi_swiglu_norm(gu.data_ptr(), h.data_ptr(), code, rows, f, d, eps, out.data_ptr(), L.stream_ptr(gu)), "uvmi_swiglu_norm")
+    rn = torch.rsqrt(h.float().pow(2).mean(-1, keepdim=True) + eps)
+    gv, uv = (gu[:, :f].float() * rn).to(dtype).float(), (gu[:, f:].float() * rn).to(dtype).float()
+    ref = ((gv * torch.sigmoid(gv)).to(dtype).float() * uv).to(dtype)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    err = (out[:rows].float() - ref.float()).abs()
+    assert bool((err <= 4 * ulp * ref.float().abs().clamp_min(0.05)).all()), float(err.max())
+    assert float((out[:rows] != ref).float().mean()) < 0.02
+    assert bool((out[rows] == 7.0).all())
+    with pytest.raises(L.UvmiError):   # f must be a multiple of 8
+        L.check(L.lib().uvmi_swiglu_norm(gu.data_ptr(), h.data_ptr(), code, rows, f + 1, d, eps, out.data_ptr(), L.stream_ptr(gu)), "uvmi_swiglu_norm")
+
+
+@pytest.mark.gpu
 def test_skinny_gemm_rejects_what_it_cannot_do():
     from ultraviolet_amd import _lib as L
     from ultraviolet_amd.kernels.gemm import SWIGLU, gemm_supported, gemm_tn

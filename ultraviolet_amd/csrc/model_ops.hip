@@ -342,6 +342,35 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const void* __restrict__ gu
   }
 }
 
+// SwiGLU on the gate/up product of the UN-normalised hidden h: the block's pre-norm is the row scale rn = rsqrt(mean(h^2) + eps)
+// of that product, so the norm never needs a launch (or a buffer) of its own.  One workgroup per row; every wave sums
+// the row's squares itself (d / 64 elements per lane), which needs no LDS and no barrier.  f % 8 == 0, d % 2 == 0.
+template <int DT>
+__global__ __launch_bounds__(256) void swiglu_norm_kernel(const void* __restrict__ gu, const void* __restrict__ h, void* __restrict__ out, int f,
+                                                          int d, float eps) {
+  const int64_t r = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  float ss = 0.f;
+  for (int i = 2 * lane; i < d; i += 128) {
+    float a, b;
+    ld2<DT>(h, r * d + i, a, b);
+    ss = fmaf(a, a, ss);
+    ss = fmaf(b, b, ss);
+  }
+  const float rn = rsqrtf(wave_sum(ss) / (float)d + eps);
+  for (int j = threadIdx.x * 8; j < f; j += 256 * 8) {
+    float g[8], u[8], o[8];
+    ld8<DT>(gu, r * 2 * f + j, g);
+    ld8<DT>(gu, r * 2 * f + f + j, u);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const float gv = round_t<DT>(g[k] * rn), uv = round_t<DT>(u[k] * rn);
+      o[k] = round_t<DT>(gv / (1.0f + __expf(-gv))) * uv;
+    }
+    st8<DT>(out, r * (int64_t)f + j, o);
+  }
+}
+
 }  // namespace uvmi
 
 using namespace uvmi;
@@ -455,5 +484,17 @@ extern "C" int uvmi_swiglu(const void* gu, int dtype, int64_t rows, int f, void*
   const dim3 grid((unsigned)blocks), blk(256);
   dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((swiglu_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, gu, out, rows, f); });
   UVMI_CHECK_LAUNCH("uvmi_swiglu");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_swiglu_norm(const void* gu, const void* h, int dtype, int64_t rows, int f, int d, float eps, void* out, void* stream) {
+  UVMI_REQUIRE(gu && h && out, UVMI_EINVAL, "uvmi_swiglu_norm: null pointer");
+  UVMI_REQUIRE(is_float_dtype(dtype) && rows >= 0 && rows <= 0x7fffffff && f > 0 && d > 0 && eps >= 0.f, UVMI_EINVAL, "uvmi_swiglu_norm: bad arguments");
+  UVMI_REQUIRE(f % 8 == 0 && d % 2 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)h % 8) == 0, UVMI_EUNSUPPORTED,
+               "uvmi_swiglu_norm: f %% 8, d %% 2 and 16-byte alignment needed");
+  if (rows == 0) return UVMI_OK;
+  const dim3 grid((unsigned)rows), blk(256);
+  dispatch_dt(dtype, [&](auto DT) { hipLaunchKernelGGL((swiglu_norm_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, gu, h, out, f, d, eps); });
+  UVMI_CHECK_LAUNCH("uvmi_swiglu_norm");
   return UVMI_OK;
 }

@@ -98,6 +98,10 @@ class UVEngine:
         # epilogue); above it, and for the down projection, the library GEMM is faster.  Measured on UV-50M decode steps:
         # 0.544 -> 0.476 ms at 128 rows, 0.551 -> 0.523 at 256, 0.606 -> 0.589 at 384, slower from 512 on.
         self.skinny_rows = int(os.environ.get("UVMI_SKINNY_ROWS", "384")) if dt in (torch.bfloat16, torch.float16) else 0
+        # above skinny_rows the skinny kernel still carries the QKV projection (with the pre-norm) and the output projection
+        # (with the residual update) up to these many rows
+        self.fold_qkv_rows = int(os.environ.get("UVMI_FOLD_QKV_ROWS", "2048"))
+        self.fold_o_rows = int(os.environ.get("UVMI_FOLD_O_ROWS", "1024"))
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -286,6 +290,14 @@ class UVEngine:
         lean = (skinny and fused_attn is not None and os.environ.get("UVMI_LEAN", "1") != "0"
                 and all("gu_il" in W and self.fused_layer_ok(l, st) for l, W in enumerate(self.w.layers))
                 and cfg.d_ff % 64 == 0 and cfg.d_ff <= 1984)
+        # Larger passes under the same condition keep the library GEMMs but still never add a launch for a residual update or
+        # for the MLP's pre-norm: both residual updates are the library's own C = alpha A B + beta C on the hidden in place,
+        # and the pre-norm is a row scale inside the SwiGLU launch (7 launches per layer where the general path has 8; 6 while
+        # the QKV projection with the pre-norm in it is still faster on the skinny kernel).
+        folded = (not skinny and fused_attn is not None and os.environ.get("UVMI_FOLD", "1") != "0" and self.dtype != torch.float32
+                  and all(self.fused_layer_ok(l, st) for l in range(cfg.n_layers)) and cfg.d_ff % 8 == 0)
+        if folded:
+            return self._trunk_folded(n, fused_attn)
         x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
@@ -326,6 +338,38 @@ class UVEngine:
                 self._add_norm(b["h"][:n], b["m"][:n], W["resid_mlp"], W["post_mlp"], n, b["x"], b["xn"])
         if not x_is_normed:
             self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
+        return xn
+
+    def _trunk_folded(self, n: int, fused_attn) -> Tensor:
+        """The layers of _trunk for a pass of many rows whose every layer takes the fused attention; buf x and xn hold the
+        embedded rows and their norm on entry."""
+        cfg, b = self.cfg, self.buf
+        x, xn = b["x"][:n], b["xn"][:n]
+        sk_ok = cfg.d_model % 64 == 0 and cfg.d_model <= 960 and (cfg.n_heads * cfg.head_dim) % 64 == 0
+        sk_qkv, sk_o = sk_ok and n <= self.fold_qkv_rows, sk_ok and n <= self.fold_o_rows
+        for l, W in enumerate(self.w.layers):
+            if l == 0:
+                torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
+            elif sk_qkv:
+                gemm_tn(x, W["wqkv_ext"], b["qkvx"][:n], norm_eps=self.eps)
+            else:
+                self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
+                torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
+            if self.qkvx_keep is not None:
+                self.qkvx_keep[l][:n].copy_(b["qkvx"][:n])
+            fused_attn(l)
+            # x <- resid_attn * x + post_attn * (zg @ wo.T), in place (every element is read and written by the same lane)
+            if sk_o:
+                gemm_tn(b["zg"][:n], W["wo"], x, epilogue=RESID, resid=x, ca=W["resid_attn"], cb=W["post_attn"])
+            else:
+                torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
+            torch.mm(x, W["gu"].t(), out=b["gu"][:n])
+            rc = L.lib().uvmi_swiglu_norm(b["gu"].data_ptr(), x.data_ptr(), self.dt_code, n, cfg.d_ff, cfg.d_model, self.eps,
+                                          b["act"].data_ptr(), L.stream_ptr(x))
+            L.check(rc, "uvmi_swiglu_norm")
+            # x <- resid_mlp * x + post_mlp * (act @ down.T)
+            torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
+        self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
         return xn
 
     def head(self, hidden: Tensor) -> Tensor:
