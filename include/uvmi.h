@@ -362,6 +362,15 @@ int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, con
 int uvmi_sched_expand(const uvmi_sched_state* s, int n_adm, int n_tokens, const int64_t* cu_seqlens, const int64_t* adm_slot,
                       const int64_t* adm_start, int64_t* pos_t, int64_t* row_t, int64_t* last_t, int64_t* last_idx, void* stream);
 
+/* Pack the completion records seen .. min(seen + max_rows, counters[1]) - 1 (seen = records the host has already taken)
+ * and the output rows of their slots, so that the host harvests with one copy of the header and one of exactly the
+ * finished tokens.  hdr (4 + 4 max_rows int64): [0..2] = counters[0..2], [3] = k, the records packed; then for packed
+ * record j: request id, slot, token count (clamped to max_new), offset of its tokens in tok_dst / lp_dst (rows back to
+ * back in record order).  tok_dst, lp_dst: max_rows * max_new elements; lp_dst may be NULL.  Replaces the whole-buffer
+ * .cpu() and the host loop over rows of StreamGen.chunk (scripts/rl_stream.py:126-143; ultraviolet/model.py:1321-1335). */
+int uvmi_sched_harvest(const uvmi_sched_state* s, int64_t seen, int max_rows, int64_t* hdr, int32_t* tok_dst,
+                       float* lp_dst, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

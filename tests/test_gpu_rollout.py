@@ -36,6 +36,9 @@ def test_slot_table_kernels_bit_exact(B, bucket, retire_p):
     tt = lambda a, dt=torch.long: torch.as_tensor(np.asarray(a), dtype=dt, device=DEV)
     nxt = 0
     dense = [torch.zeros(bucket, dtype=torch.long, device=DEV) for _ in range(6)]
+    hv_rows, seen, harvested = 5, 0, []
+    hv_hdr = torch.zeros(4 + 4 * hv_rows, dtype=torch.long, device=DEV)
+    hv_tok, hv_lp = torch.zeros(hv_rows * max_new, dtype=torch.int32, device=DEV), torch.zeros(hv_rows * max_new, dtype=torch.float32, device=DEV)
     for step in range(30):
         free = np.nonzero(tab.req < 0)[0]
         k = int(rng.integers(0, len(free) + 1)) if step < 20 else 0
@@ -67,7 +70,27 @@ def test_slot_table_kernels_bit_exact(B, bucket, retire_p):
         assert n_done == len(tab.done)
         got = sorted(zip(t["done_req"][:n_done].tolist(), t["done_slot"][:n_done].tolist(), t["done_cnt"][:n_done].tolist()))
         assert got == sorted(tab.done)
-    assert len(tab.done) > 0
+        # harvest: at most hv_rows records per launch, packed with their output rows (the slots are not refilled before the
+        # next step's admission, so the simulator's rows still hold the finished requests' tokens)
+        while True:
+            L.check(lib.uvmi_sched_harvest(C.byref(s), seen, hv_rows, hv_hdr.data_ptr(), hv_tok.data_ptr(), hv_lp.data_ptr(), None), "harvest")
+            hdr = hv_hdr.cpu().numpy()
+            assert hdr[:3].tolist() == t["counters"][:3].tolist() and hdr[1] == n_done and hdr[3] == min(n_done - seen, hv_rows)
+            k = int(hdr[3])
+            if k == 0:
+                break
+            rec = hdr[4:4 + 4 * k].reshape(k, 4)
+            ring = list(zip(t["done_req"][seen:seen + k].tolist(), t["done_slot"][seen:seen + k].tolist(), t["done_cnt"][seen:seen + k].tolist()))
+            assert [tuple(r[:3]) for r in rec.tolist()] == [(r, sl, min(c, max_new)) for r, sl, c in ring]
+            assert rec[:, 3].tolist() == np.concatenate([[0], np.cumsum(rec[:, 2])[:-1]]).tolist()
+            tk, lp = hv_tok.cpu().numpy(), hv_lp.cpu().numpy()
+            for r, sl, c, o in rec.tolist():
+                assert np.array_equal(tk[o:o + c], tab.out_tok[sl, :c]) and np.array_equal(lp[o:o + c], tab.out_lp[sl, :c])
+                harvested.append((r, sl, c))
+            seen += k
+            if seen >= n_done:
+                break
+    assert len(tab.done) > 0 and sorted(harvested) == sorted((r, sl, min(c, max_new)) for r, sl, c in tab.done)
 
 
 def _engine(dtype=torch.float32, window=16, max_tokens=1024):

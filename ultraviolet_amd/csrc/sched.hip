@@ -7,7 +7,8 @@
 //                  request id / token index into dense arrays of a fixed bucket length (padding rows get slot -1);
 //   sched_commit   scatter the sampled token and its log-prob into the slot's output row, advance count and position,
 //                  retire on EOS / length limit / seeded Bernoulli(p), park retired rows at position 0 and append a
-//                  completion record for the host to harvest asynchronously.
+//                  completion record for the host to harvest asynchronously;
+//   sched_harvest  pack new completion records and their output rows for the host's copy.
 //
 // Both are integer bookkeeping on <= a few thousand slots: latency-bound, one workgroup / one thread per row.
 #include "common.h"
@@ -161,6 +162,45 @@ __global__ __launch_bounds__(256) void sched_expand_kernel(uvmi_sched_state S, i
   last_t[i] = real ? adm_start[lo] + (cu[lo + 1] - cu[lo]) - 1 : 0;
 }
 
+// Completion records seen .. min(seen + max_rows, written) and their output rows, packed back to back for one small
+// device->host copy of the header and one of exactly the finished tokens.  One workgroup per record.
+__global__ __launch_bounds__(256) void sched_harvest_kernel(uvmi_sched_state S, int64_t seen, int max_rows, int64_t* hdr, int32_t* tok_dst,
+                                                            float* lp_dst) {
+  __shared__ int64_t wsum[4];
+  const int j = blockIdx.x, tid = threadIdx.x;
+  int64_t k = (int64_t)S.counters[1] - seen;
+  k = k < 0 ? 0 : (k > max_rows ? max_rows : k);
+  if (j == 0 && tid < 4) hdr[tid] = tid < 3 ? (int64_t)S.counters[tid] : k;
+  if (j >= k) return;
+  auto count_of = [&](int64_t rec) {
+    const int64_t c = S.done_cnt[rec % S.done_cap];
+    return c < 0 ? 0 : (c > S.max_new ? S.max_new : c);
+  };
+  int64_t part = 0;
+  for (int i = tid; i < j; i += 256) part += count_of(seen + i);
+  for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+  if ((tid & 63) == 0) wsum[tid >> 6] = part;
+  __syncthreads();
+  const int64_t off = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+  const int64_t e = (seen + j) % S.done_cap;
+  const int64_t slot = S.done_slot[e];
+  const bool ok = slot >= 0 && slot < S.B;
+  const int64_t cnt = ok ? count_of(seen + j) : 0;
+  if (tid == 0) {
+    int64_t* h = hdr + 4 + 4 * j;
+    h[0] = S.done_req[e];
+    h[1] = slot;
+    h[2] = cnt;
+    h[3] = off;
+  }
+  const int32_t* src_t = S.out_tok + slot * S.max_new;
+  const float* src_l = S.out_lp ? S.out_lp + slot * S.max_new : nullptr;
+  for (int64_t t = tid; t < cnt; t += 256) {
+    tok_dst[off + t] = src_t[t];
+    if (lp_dst && src_l) lp_dst[off + t] = src_l[t];
+  }
+}
+
 static int check_state(const uvmi_sched_state* s, const char* who) {
   UVMI_REQUIRE(s, UVMI_EINVAL, "%s: null state", who);
   UVMI_REQUIRE(s->slot_req && s->slot_cnt && s->slot_limit && s->slot_tok && s->pos && s->starts && s->out_tok && s->counters &&
@@ -215,5 +255,15 @@ extern "C" int uvmi_sched_expand(const uvmi_sched_state* s, int n_adm, int n_tok
   hipLaunchKernelGGL(sched_expand_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_adm, n_tokens, cu_seqlens, adm_slot,
                      adm_start, pos_t, row_t, last_t, last_idx);
   UVMI_CHECK_LAUNCH("uvmi_sched_expand");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_harvest(const uvmi_sched_state* s, int64_t seen, int max_rows, int64_t* hdr, int32_t* tok_dst, float* lp_dst,
+                                  void* stream) {
+  int rc = check_state(s, "uvmi_sched_harvest");
+  if (rc) return rc;
+  UVMI_REQUIRE(seen >= 0 && max_rows > 0 && max_rows <= 65535 && hdr && tok_dst, UVMI_EINVAL, "uvmi_sched_harvest: bad arguments");
+  hipLaunchKernelGGL(sched_harvest_kernel, dim3(max_rows), dim3(256), 0, (hipStream_t)stream, *s, seen, max_rows, hdr, tok_dst, lp_dst);
+  UVMI_CHECK_LAUNCH("uvmi_sched_harvest");
   return UVMI_OK;
 }

@@ -81,6 +81,12 @@ class Rollout:
             self.gather_idx = torch.cat([z(A), Np + torch.arange(slots, device=dev)])   # rows of the hidden that get sampled
             self.adm_slot.fill_(-1)
             self._stage_ev = torch.cuda.Event()
+        # harvest staging: a launch packs up to hv_rows new completion records and their output rows; the host takes the header
+        # and then exactly the finished tokens, through pinned buffers (no indexing launches, no pageable copies)
+        self.hv_rows = min(slots, 128)
+        self.hv_hdr, self.hv_tok, self.hv_lp = z(4 + 4 * self.hv_rows), z(self.hv_rows * max_new, dt=torch.int32), z(self.hv_rows * max_new, dt=torch.float32)
+        self.hv_hdr_h, self.hv_tok_h, self.hv_lp_h = (torch.zeros(t.shape, dtype=t.dtype, pin_memory=True) for t in (self.hv_hdr, self.hv_tok, self.hv_lp))
+        self._hv_ev = torch.cuda.Event()
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.mixed_graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.queue = collections.deque()
@@ -96,7 +102,8 @@ class Rollout:
     # ------------------------------------------------------------------------------------------------ requests
     def add(self, prompt_ids, meta, limit: int | None = None):
         assert 0 < len(prompt_ids) <= self.max_prompt, "prompt longer than max_prompt"
-        self.queue.append((list(prompt_ids), meta, self.max_new if limit is None else min(int(limit), self.max_new)))
+        ids = list(prompt_ids)
+        self.queue.append((ids, meta, self.max_new if limit is None else min(int(limit), self.max_new), np.asarray(ids, dtype=np.int64)))
 
     def n_active(self) -> int:
         return self.B - len(self.free)
@@ -184,7 +191,7 @@ class Rollout:
         self._stage_ev.synchronize()                        # the previous upload has left the pinned buffer
         h = self.stage_h.numpy()
         h[:] = 0
-        h[:ntok] = np.fromiter((t for b in batch for t in b[0]), dtype=np.int64, count=ntok)
+        h[:ntok] = np.concatenate([b[3] for b in batch])
         o = Np
         h[o] = 0
         h[o + 1:o + 1 + na] = np.cumsum(lens)
@@ -312,28 +319,41 @@ class Rollout:
     # ------------------------------------------------------------------------------------------------ harvest
     @torch.no_grad()
     def poll(self):
-        """Read the completion ring (one small device->host copy), return finished requests as
-        (meta, tokens, logp float32 array, start_version) and free their slots."""
-        cnt = self.counters.cpu().numpy()
-        n_done = int(cnt[1])
-        if cnt[2]:
-            raise RuntimeError("active slots exceeded the captured bucket (host bound on active slots was wrong)")
+        """Harvest: a launch packs the new completion records and their output rows, the host copies the header and then
+        exactly the finished tokens; returns finished requests as (meta, tokens, logp float32 array, start_version) and
+        frees their slots."""
         out = []
-        if n_done > self.done_seen:
+        while True:
+            rc = L.lib().uvmi_sched_harvest(C.byref(self.sched), self.done_seen, self.hv_rows, self.hv_hdr.data_ptr(), self.hv_tok.data_ptr(),
+                                            self.hv_lp.data_ptr(), L.stream_ptr(self.hv_hdr))
+            L.check(rc, "uvmi_sched_harvest")
+            self.hv_hdr_h.copy_(self.hv_hdr, non_blocking=True)
+            self._hv_ev.record()
+            self._hv_ev.synchronize()
+            hdr = self.hv_hdr_h.numpy()
+            n_done, k = int(hdr[1]), int(hdr[3])
+            if hdr[2]:
+                raise RuntimeError("active slots exceeded the captured bucket (host bound on active slots was wrong)")
             assert n_done - self.done_seen <= self.done_cap, "completion ring overflow: poll more often"
-            ix = torch.arange(self.done_seen, n_done, device=self.dev) % self.done_cap
-            reqs, slots, cnts = (t.index_select(0, ix).cpu().numpy() for t in (self.done_req, self.done_slot, self.done_cnt))
-            order = np.argsort(reqs, kind="stable")   # arrival order inside one step is not deterministic: sort by request
-            reqs, slots, cnts = reqs[order], slots[order], cnts[order]
-            st = torch.as_tensor(slots, device=self.dev)
-            toks, lps = self.out_tok.index_select(0, st).cpu().numpy(), self.out_lp.index_select(0, st).cpu().numpy()
-            for j, (r, s_, c) in enumerate(zip(reqs, slots, cnts)):
-                c = min(int(c), self.max_new)
-                meta, v0 = self.meta.pop(int(r))
-                out.append((meta, toks[j, :c].tolist(), lps[j, :c].copy(), v0))
+            if k == 0:
+                break
+            rec = hdr[4:4 + 4 * k].reshape(k, 4)
+            total = int(rec[-1, 3] + rec[-1, 2])
+            if total:
+                self.hv_tok_h[:total].copy_(self.hv_tok[:total], non_blocking=True)
+                self.hv_lp_h[:total].copy_(self.hv_lp[:total], non_blocking=True)
+                self._hv_ev.record()
+                self._hv_ev.synchronize()
+            toks, lps = self.hv_tok_h.numpy(), self.hv_lp_h.numpy()
+            # arrival order inside one step is not deterministic: sort by request
+            for r, s_, c, o in rec[np.argsort(rec[:, 0], kind="stable")].tolist():
+                meta, v0 = self.meta.pop(r)
+                out.append((meta, toks[o:o + c].tolist(), lps[o:o + c].copy(), v0))
                 self.n_tokens += c
-                self.free.append(int(s_))
-            self.done_seen = n_done
+                self.free.append(s_)
+            self.done_seen += k
+            if self.done_seen >= n_done:
+                break
         self.n_active_host = self.n_active()
         return out
 
