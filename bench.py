@@ -95,13 +95,18 @@ def bench_c5(args):
     K = min(args.steps, total_steps - W) if args.steps > 0 else total_steps - W
 
     def run_steps(gg, n):
+        """n decode steps with a harvest every check_every steps; the host takes a harvest's results after it has enqueued
+        the following step, so that its share of the work costs no idle GPU time."""
         done = 0
         while done < n:
             m = min(gg.ce, n - done)
-            for _ in range(m):
+            for i in range(m):
                 gg.step()
+                if i == 0 and gg.harvest_pending:
+                    gg.harvest_end()
             done += m
-            gg.poll()
+            gg.harvest_begin()
+        gg.harvest_end()
 
     run_steps(g, W)
     torch.cuda.synchronize()
@@ -377,7 +382,7 @@ def bench_c3(args):
     K = args.steps if args.steps > 0 else 256
     W = args.warmup
     g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + K + W + 64, temperature=1.0, seed=0, eos_id=None, check_every=4, bucket=128,
-                retire_p=0.01, mixed=True, admit_cap=24)
+                retire_p=0.01, mixed=True, admit_cap=24, overlap_harvest=True)
     # running slots with materialised contexts: request ids 0..B-1, one token generated so far
     rows = torch.arange(B, device=dev)
     _fill_cache(g.st, rows, torch.from_numpy(rng.integers(128, 2049, size=B)).to(dev), gen)
@@ -396,6 +401,8 @@ def bench_c3(args):
         s0 = g.n_decode_steps
         while g.n_decode_steps - s0 < n:
             g.chunk()
+        if g.harvest_pending:   # (chunk() leaves its harvest for the next call to take)
+            g.harvest_end()
 
     def generated():
         return int(g.slot_cnt[g.slot_req >= 0].sum()) + g.n_tokens
@@ -415,7 +422,7 @@ def bench_c3(args):
                       "dtype": "bf16", "data": "synthetic",
                       "config": {"workload": "C3 continuous batching: UV-50M bf16, int8 KV, 512 slots, contexts U{128..2048} materialised in the "
                                              "cache, Bernoulli(0.01) retirement per slot and step on the device, 64-token prompts admitted into "
-                                             "freed slots inside decode passes, host poll every 4 steps",
+                                             "freed slots inside decode passes, harvest every 4 steps (its results taken one step later)",
                                  "tokens_timed": gen_tok, "mixed_steps": g.n_mixed_steps - m0, "requests_finished": g.next_req - len(g.meta),
                                  "active_at_end": g.n_active(), "full_slot_tok_per_s": round(B * steps / dt, 1)}}))
 

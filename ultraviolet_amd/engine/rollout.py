@@ -29,7 +29,7 @@ class Rollout:
     def __init__(self, engine: UVEngine, slots: int, max_prompt: int, max_new: int, temperature: float = 1.0,
                  seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
                  use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False,
-                 admit_cap: int = 16, top_k: int = 0, top_p: float = 1.0, kv_dtype: str = "int8"):
+                 admit_cap: int = 16, top_k: int = 0, top_p: float = 1.0, kv_dtype: str = "int8", overlap_harvest: bool = False):
         self.e, self.cfg = engine, engine.cfg
         self.top_k, self.top_p = int(top_k), float(top_p)   # truncated sampling (sample(), model.py:1200-1209); off by default
         self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
@@ -86,7 +86,10 @@ class Rollout:
         self.hv_rows = min(slots, 128)
         self.hv_hdr, self.hv_tok, self.hv_lp = z(4 + 4 * self.hv_rows), z(self.hv_rows * max_new, dt=torch.int32), z(self.hv_rows * max_new, dt=torch.float32)
         self.hv_hdr_h, self.hv_tok_h, self.hv_lp_h = (torch.zeros(t.shape, dtype=t.dtype, pin_memory=True) for t in (self.hv_hdr, self.hv_tok, self.hv_lp))
-        self._hv_ev = torch.cuda.Event()
+        self._hv_ev, self._hv_ev2 = torch.cuda.Event(), torch.cuda.Event()
+        self._hv_stream = torch.cuda.Stream(device=dev)   # default priority; carries only the harvest's device -> host copies
+        self.harvest_pending = False
+        self.overlap_harvest = bool(overlap_harvest)
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.mixed_graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.queue = collections.deque()
@@ -318,18 +321,28 @@ class Rollout:
 
     # ------------------------------------------------------------------------------------------------ harvest
     @torch.no_grad()
-    def poll(self):
-        """Harvest: a launch packs the new completion records and their output rows, the host copies the header and then
-        exactly the finished tokens; returns finished requests as (meta, tokens, logp float32 array, start_version) and
-        frees their slots."""
+    def harvest_begin(self):
+        """Enqueue the harvest: a launch packs the new completion records and their output rows, and the header starts
+        its way to the host.  Nothing waits; harvest_end() takes the results.  Work enqueued in between (a decode step)
+        runs while the host does so - it may not admit requests, since the rows of finished slots must stay untouched."""
+        assert not self.harvest_pending
+        rc = L.lib().uvmi_sched_harvest(C.byref(self.sched), self.done_seen, self.hv_rows, self.hv_hdr.data_ptr(), self.hv_tok.data_ptr(),
+                                        self.hv_lp.data_ptr(), L.stream_ptr(self.hv_hdr))
+        L.check(rc, "uvmi_sched_harvest")
+        self.hv_hdr_h.copy_(self.hv_hdr, non_blocking=True)
+        self._hv_ev.record()
+        self.harvest_pending = True
+
+    @torch.no_grad()
+    def harvest_end(self):
+        """Take the results of harvest_begin(): finished requests as (meta, tokens, logp float32 array, start_version);
+        frees their slots.  The finished tokens come over on a second stream, so they do not queue behind a decode step
+        enqueued since."""
+        assert self.harvest_pending
         out = []
         while True:
-            rc = L.lib().uvmi_sched_harvest(C.byref(self.sched), self.done_seen, self.hv_rows, self.hv_hdr.data_ptr(), self.hv_tok.data_ptr(),
-                                            self.hv_lp.data_ptr(), L.stream_ptr(self.hv_hdr))
-            L.check(rc, "uvmi_sched_harvest")
-            self.hv_hdr_h.copy_(self.hv_hdr, non_blocking=True)
-            self._hv_ev.record()
             self._hv_ev.synchronize()
+            self.harvest_pending = False
             hdr = self.hv_hdr_h.numpy()
             n_done, k = int(hdr[1]), int(hdr[3])
             if hdr[2]:
@@ -340,10 +353,11 @@ class Rollout:
             rec = hdr[4:4 + 4 * k].reshape(k, 4)
             total = int(rec[-1, 3] + rec[-1, 2])
             if total:
-                self.hv_tok_h[:total].copy_(self.hv_tok[:total], non_blocking=True)
-                self.hv_lp_h[:total].copy_(self.hv_lp[:total], non_blocking=True)
-                self._hv_ev.record()
-                self._hv_ev.synchronize()
+                with torch.cuda.stream(self._hv_stream):   # (the packing launch has finished: its header has arrived)
+                    self.hv_tok_h[:total].copy_(self.hv_tok[:total], non_blocking=True)
+                    self.hv_lp_h[:total].copy_(self.hv_lp[:total], non_blocking=True)
+                    self._hv_ev2.record()
+                self._hv_ev2.synchronize()
             toks, lps = self.hv_tok_h.numpy(), self.hv_lp_h.numpy()
             # arrival order inside one step is not deterministic: sort by request
             for r, s_, c, o in rec[np.argsort(rec[:, 0], kind="stable")].tolist():
@@ -354,12 +368,27 @@ class Rollout:
             self.done_seen += k
             if self.done_seen >= n_done:
                 break
+            self.harvest_begin()   # more records than one launch packs
         self.n_active_host = self.n_active()
         return out
 
+    def poll(self):
+        """Harvest now: harvest_begin() + harvest_end()."""
+        if not self.harvest_pending:
+            self.harvest_begin()
+        return self.harvest_end()
+
     def chunk(self):
-        """Fill idle slots from the queue, decode check_every steps, harvest (reference: StreamGen.chunk)."""
-        steps = self.ce
+        """Fill idle slots from the queue, decode check_every steps, harvest (reference: StreamGen.chunk).  With
+        overlap_harvest the harvest is only enqueued here and its results are returned by the next call, which takes them
+        after it has enqueued its first decode step: the host's share of the harvest then costs no idle GPU time, and
+        freed slots are refilled one step later."""
+        steps, out = self.ce, []
+        if self.harvest_pending:
+            if self.n_active() > 0 and steps > 0:
+                self.step()
+                steps -= 1
+            out = self.harvest_end()
         if self.queue and self.free:
             if self.mixed and self.n_active() > 0:
                 while self.queue and self.free and steps > 0 and self._admit_mixed():
@@ -367,10 +396,13 @@ class Rollout:
             else:
                 self._admit()
         if self.n_active() == 0:
-            return []
+            return out
         for _ in range(steps):
             self.step()
-        return self.poll()
+        if self.overlap_harvest:
+            self.harvest_begin()
+            return out
+        return out + self.poll()
 
     def run(self, max_chunks: int = 1 << 30):
         res = []
@@ -378,4 +410,6 @@ class Rollout:
             if self.n_outstanding() == 0:
                 break
             res += self.chunk()
+        if self.harvest_pending:
+            res += self.harvest_end()
         return res
