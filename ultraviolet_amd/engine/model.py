@@ -185,6 +185,13 @@ class UVEngine:
         rc = L.lib().uvmi_swiglu(b["gu"].data_ptr(), self.dt_code, n, self.cfg.d_ff, b["act"].data_ptr(), L.stream_ptr(b["gu"]))
         L.check(rc, "uvmi_swiglu")
 
+    def _swiglu_norm(self, h: Tensor, n: int):
+        """buf act = SwiGLU of rmsnorm(h) @ gu.T, from buf gu = h @ gu.T (the norm as a row scale of the product)."""
+        b = self.buf
+        rc = L.lib().uvmi_swiglu_norm(b["gu"].data_ptr(), h.data_ptr(), self.dt_code, n, self.cfg.d_ff, self.cfg.d_model, self.eps,
+                                      b["act"].data_ptr(), L.stream_ptr(h))
+        L.check(rc, "uvmi_swiglu_norm")
+
     # ------------------------------------------------------------------------------------------------ trunk
     def cache_attention(self, l: int, q: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None,
                         off: int = 0):
@@ -298,6 +305,7 @@ class UVEngine:
                   and all(self.fused_layer_ok(l, st) for l in range(cfg.n_layers)) and cfg.d_ff % 8 == 0)
         if folded:
             return self._trunk_folded(n, fused_attn)
+        fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and os.environ.get("UVMI_FOLD", "1") != "0"
         x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
@@ -322,6 +330,16 @@ class UVEngine:
                 # launches where the general path has five
                 gemm_tn(b["zg"][:n], W["wo"], b["h"][:n], epilogue=RESID, resid=x, ca=W["resid_attn"], cb=W["post_attn"])
                 gemm_tn(b["h"][:n], W["gu_il"], b["act"][:n], epilogue=SWIGLU, norm_eps=self.eps)
+            elif fold_mlp:
+                # 16-bit passes of any size and attention path: both residual updates are the library's C = alpha A B + beta C
+                # on the hidden in place and the MLP's pre-norm is the row scale inside the SwiGLU launch; the block ends
+                # with the norm the next block's projection and post-processing read
+                torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
+                torch.mm(x, W["gu"].t(), out=b["gu"][:n])
+                self._swiglu_norm(x, n)
+                torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
+                self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
+                continue
             else:
                 mm(b["zg"][:n], W["wo"], b["a"][:n])
                 # h = resid_attn * x + post_attn * a ; n = rmsnorm(h)
@@ -364,9 +382,7 @@ class UVEngine:
             else:
                 torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
             torch.mm(x, W["gu"].t(), out=b["gu"][:n])
-            rc = L.lib().uvmi_swiglu_norm(b["gu"].data_ptr(), x.data_ptr(), self.dt_code, n, cfg.d_ff, cfg.d_model, self.eps,
-                                          b["act"].data_ptr(), L.stream_ptr(x))
-            L.check(rc, "uvmi_swiglu_norm")
+            self._swiglu_norm(x, n)
             # x <- resid_mlp * x + post_mlp * (act @ down.T)
             torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
         self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
