@@ -350,6 +350,14 @@ __global__ __launch_bounds__(256) void swiglu_norm_kernel(const void* __restrict
                                                           int d, float eps) {
   const int64_t r = blockIdx.x;
   const int lane = threadIdx.x & 63;
+  // the thread's first 8 gate / up columns are requested before the row's squares, so that both round trips to memory
+  // overlap (f <= 2048: the only ones)
+  int j = threadIdx.x * 8;
+  float g[8], u[8], o[8];
+  if (j < f) {
+    ld8<DT>(gu, r * 2 * f + j, g);
+    ld8<DT>(gu, r * 2 * f + f + j, u);
+  }
   float ss = 0.f;
   for (int i = 2 * lane; i < d; i += 128) {
     float a, b;
@@ -358,16 +366,18 @@ __global__ __launch_bounds__(256) void swiglu_norm_kernel(const void* __restrict
     ss = fmaf(b, b, ss);
   }
   const float rn = rsqrtf(wave_sum(ss) / (float)d + eps);
-  for (int j = threadIdx.x * 8; j < f; j += 256 * 8) {
-    float g[8], u[8], o[8];
-    ld8<DT>(gu, r * 2 * f + j, g);
-    ld8<DT>(gu, r * 2 * f + f + j, u);
+  while (j < f) {
 #pragma unroll
     for (int k = 0; k < 8; k++) {
       const float gv = round_t<DT>(g[k] * rn), uv = round_t<DT>(u[k] * rn);
       o[k] = round_t<DT>(gv / (1.0f + __expf(-gv))) * uv;
     }
     st8<DT>(out, r * (int64_t)f + j, o);
+    j += 256 * 8;
+    if (j < f) {
+      ld8<DT>(gu, r * 2 * f + j, g);
+      ld8<DT>(gu, r * 2 * f + f + j, u);
+    }
   }
 }
 
