@@ -7,8 +7,9 @@ Workload c5 (default; BASELINE.json configs[4], the configuration the metric is 
 256 prompts x group 8 = 2048 concurrent sequences, prompt lengths U{64..256} shared inside a group, T = 1.0 with seeded
 Philox sampling, per-sequence stop length min(Geom(1/600), 2048), random-init (perturbed) UV-50M in bf16 with an int8
 KV cache.  All prompts are prefilled (untimed, reported separately), W decode steps run untimed, then exactly K decode
-steps of the rollout are timed; a step is compact -> 10-layer trunk over the active rows -> tied head -> fused sampler ->
-commit, replayed from a captured graph, with the inputs resident in HBM.  value = tokens generated in the timed steps /
+steps of the rollout are timed; a step is 10-layer trunk over the active rows -> tied head -> fused sampler -> commit,
+replayed from a captured graph (the active rows are compacted again when the bucket shrinks), with the inputs resident
+in HBM.  value = tokens generated in the timed steps /
 seconds.
 
 After the timed region the same rollout is replayed eagerly and, on a subsample of steps, the step's decode-attention
@@ -175,13 +176,14 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
         return e0, e1
 
     for s in range(W + K):
+        sampled = s >= W and (s - W) % every == 0
+        if sampled:   # the step's own rows, tokens and positions (the step leaves the next step's in their place)
+            n, act, tok, pos, starts = (t if isinstance(t, int) else t.clone() for t in g.step_inputs())
         g.step()
-        if s >= W and (s - W) % every == 0:
+        if sampled:
             torch.cuda.synchronize()
-            n = g.bucket_for(g.n_active_host)
-            act, pos, starts = g.act[:n], g.pos_c[:n], g.starts_c[:n]
             if fused:
-                built = {l: eng.fused_attention_args(l, eng.qkvx_keep[l], g.tok_c[:n], g.st, pos, starts, n, rows=act) for l in layers}
+                built = {l: eng.fused_attention_args(l, eng.qkvx_keep[l], tok, g.st, pos, starts, n, rows=act) for l in layers}
             else:
                 built = {l: eng.cache_attention_args(l, g.st, pos, starts, n, rows=act) for l in layers}
             evA = timed_seq([built[l][0] for l in layers])

@@ -348,6 +348,13 @@ int uvmi_sched_compact(const uvmi_sched_state* s, int n_bucket, int64_t* act_slo
  * rl_stream.py:120-143, model.py:1321-1350. */
 int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const int64_t* act_slot, const int64_t* new_tok,
                       const float* new_lp, float retire_p, uint64_t seed, void* stream);
+/* uvmi_sched_commit that also carries the dense arrays of uvmi_sched_compact to the next step: a row that goes on gets
+ * its new token, position + 1 and token index + 1 in place; a row that retires becomes padding where it stands (slot -1,
+ * zeros).  The next step then runs on these arrays without a compaction; padding rows may sit between active ones, so
+ * the bucket only has to be compacted again after an admission or when it is to shrink. */
+int uvmi_sched_commit_dense(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c,
+                            int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, const int64_t* new_tok,
+                            const float* new_lp, float retire_p, uint64_t seed, void* stream);
 /* Bind n freshly prefilled requests to slots and record their first sampled token (model.py:1306-1313,
  * rl_stream.py:86-92). */
 int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, const int64_t* req_ids,

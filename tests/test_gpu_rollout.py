@@ -61,8 +61,19 @@ def test_slot_table_kernels_bit_exact(B, bucket, retire_p):
         assert int(t["counters"][0]) == n_act
         new_tok, new_lp = rng.integers(0, 6, size=bucket), rng.random(bucket, dtype=np.float32)
         nt, nl = tt(new_tok), tt(new_lp, torch.float32)
-        L.check(lib.uvmi_sched_commit(C.byref(s), bucket, dense[0].data_ptr(), nt.data_ptr(), nl.data_ptr(), retire_p, seed, None), "commit")
+        if step % 2:   # the dense form also carries the dense arrays to the next step
+            L.check(lib.uvmi_sched_commit_dense(C.byref(s), bucket, *[d_.data_ptr() for d_ in dense], nt.data_ptr(), nl.data_ptr(), retire_p,
+                                                seed, None), "commit_dense")
+        else:
+            L.check(lib.uvmi_sched_commit(C.byref(s), bucket, dense[0].data_ptr(), nt.data_ptr(), nl.data_ptr(), retire_p, seed, None), "commit")
         tab.commit(slot, new_tok, new_lp, retire_p, seed)
+        if step % 2:   # rows that go on keep their place with the new token / position / index; retired rows are padding
+            on = (slot >= 0) & (tab.req[np.maximum(slot, 0)] >= 0)
+            sl = np.maximum(slot, 0)
+            want = [np.where(on, slot, -1), np.where(on, tab.tok[sl], 0), np.where(on, tab.pos[sl], 0), np.where(on, tab.starts[sl], 0),
+                    np.where(on, tab.req[sl], 0), np.where(on, tab.cnt[sl], 0)]
+            for j, kname in enumerate(("slot", "tok", "pos", "starts", "req", "cnt")):
+                assert np.array_equal(dense[j].cpu().numpy(), want[j]), (step, kname)
         for name, ref in (("slot_req", tab.req), ("slot_cnt", tab.cnt), ("slot_tok", tab.tok), ("pos", tab.pos), ("starts", tab.starts),
                           ("out_tok", tab.out_tok), ("out_lp", tab.out_lp)):
             assert np.array_equal(t[name].cpu().numpy(), ref), (step, name)

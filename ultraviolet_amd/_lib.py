@@ -146,6 +146,7 @@ def lib() -> C.CDLL:
         L.uvmi_sched_compact.argtypes = [C.POINTER(SchedState), C.c_int] + [C.c_void_p] * 7
         L.uvmi_sched_commit.argtypes = [C.POINTER(SchedState), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_uint64,
                                         C.c_void_p]
+        L.uvmi_sched_commit_dense.argtypes = [C.POINTER(SchedState), C.c_int] + [C.c_void_p] * 8 + [C.c_float, C.c_uint64, C.c_void_p]
         L.uvmi_sched_admit.argtypes = [C.POINTER(SchedState), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                        C.c_void_p]
         L.uvmi_sched_expand.argtypes = [C.POINTER(SchedState), C.c_int, C.c_int] + [C.c_void_p] * 8
@@ -181,4 +182,4 @@ EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu", "uvmi_swiglu_norm",
-           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]
+           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_commit_dense", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]

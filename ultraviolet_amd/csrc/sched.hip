@@ -7,7 +7,9 @@
 //                  request id / token index into dense arrays of a fixed bucket length (padding rows get slot -1);
 //   sched_commit   scatter the sampled token and its log-prob into the slot's output row, advance count and position,
 //                  retire on EOS / length limit / seeded Bernoulli(p), park retired rows at position 0 and append a
-//                  completion record for the host to harvest asynchronously;
+//                  completion record for the host to harvest asynchronously; its dense form also carries the step's dense
+//                  arrays to the next step (retired rows become padding where they stand), so that only the first
+//                  step after an admission or a change of bucket needs a compaction;
 //   sched_harvest  pack new completion records and their output rows for the host's copy.
 //
 // Both are integer bookkeeping on <= a few thousand slots: latency-bound, one workgroup / one thread per row.
@@ -75,8 +77,12 @@ __global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S,
   }
 }
 
-__global__ __launch_bounds__(256) void sched_commit_kernel(uvmi_sched_state S, int n_bucket, const int64_t* act_slot,
-                                                           const int64_t* new_tok, const float* new_lp, float retire_p, uint64_t seed) {
+// DENSE: the step's dense arrays are carried to the next step in place of a new compaction - a row that goes on gets its
+// new token, position and token index, a row that retires becomes padding (slot -1, zeros) where it stands.
+template <bool DENSE>
+__global__ __launch_bounds__(256) void sched_commit_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, const int64_t* new_tok,
+                                                           const float* new_lp, float retire_p, uint64_t seed, int64_t* tok_c,
+                                                           int64_t* pos_c, int64_t* starts_c, int64_t* req_c, int64_t* cnt_c) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= n_bucket) return;
   const int64_t slot = act_slot[i];
@@ -104,6 +110,13 @@ __global__ __launch_bounds__(256) void sched_commit_kernel(uvmi_sched_state S, i
     S.slot_req[slot] = -1;
     S.pos[slot] = 0;      // parked: never overruns the cache (model.py:1345-1350)
     S.starts[slot] = 0;
+  }
+  if (DENSE) {
+    act_slot[i] = fin ? -1 : slot;
+    tok_c[i] = fin ? 0 : tok;
+    pos_c[i] = fin ? 0 : pos_c[i] + 1;
+    cnt_c[i] = fin ? 0 : c + 1;
+    if (fin) { starts_c[i] = 0; req_c[i] = 0; }
   }
 }
 
@@ -228,9 +241,22 @@ extern "C" int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const 
   int rc = check_state(s, "uvmi_sched_commit");
   if (rc) return rc;
   UVMI_REQUIRE(n_bucket > 0 && act_slot && new_tok, UVMI_EINVAL, "uvmi_sched_commit: bad arguments");
-  hipLaunchKernelGGL(sched_commit_kernel, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket, act_slot, new_tok,
-                     new_lp, retire_p, seed);
+  hipLaunchKernelGGL(sched_commit_kernel<false>, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket,
+                     const_cast<int64_t*>(act_slot), new_tok, new_lp, retire_p, seed, nullptr, nullptr, nullptr, nullptr, nullptr);
   UVMI_CHECK_LAUNCH("uvmi_sched_commit");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_commit_dense(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c,
+                                       int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, const int64_t* new_tok, const float* new_lp,
+                                       float retire_p, uint64_t seed, void* stream) {
+  int rc = check_state(s, "uvmi_sched_commit_dense");
+  if (rc) return rc;
+  UVMI_REQUIRE(n_bucket > 0 && act_slot && tok_c && pos_c && starts_c && req_c && cnt_c && new_tok, UVMI_EINVAL,
+               "uvmi_sched_commit_dense: bad arguments");
+  hipLaunchKernelGGL(sched_commit_kernel<true>, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket, act_slot,
+                     new_tok, new_lp, retire_p, seed, tok_c, pos_c, starts_c, req_c, cnt_c);
+  UVMI_CHECK_LAUNCH("uvmi_sched_commit_dense");
   return UVMI_OK;
 }
 

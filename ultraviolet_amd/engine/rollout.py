@@ -98,6 +98,7 @@ class Rollout:
         self.next_req = 0
         self.n_active_host = 0                    # upper bound on active slots (exact after each poll / admit)
         self.done_seen = 0
+        self._dense_n = None                      # bucket the dense step arrays are valid for (None: stale, compact first)
         self.version = 0
         self.n_decode_steps = 0
         self.n_tokens = 0
@@ -163,6 +164,7 @@ class Rollout:
             for r, b in zip(reqs, batch):
                 self.meta[r] = (b[1], self.version)
             self.n_active_host += len(batch)
+            self._dense_n = None
 
     def _sample(self, x, req, cnt):
         if self.T > 0:
@@ -219,6 +221,7 @@ class Rollout:
         for r, b in zip(reqs, batch):
             self.meta[r] = (b[1], self.version)
         self.n_active_host += na
+        self._dense_n = None                                # the step's dense arrays predate the admission
         self.n_decode_steps += 1
         self.n_mixed_steps += 1
         return True
@@ -245,12 +248,19 @@ class Rollout:
                                      tok.data_ptr(), lp.data_ptr(), sp), "uvmi_sched_admit")
 
     # ------------------------------------------------------------------------------------------------ decode
+    def _compact(self, n: int):
+        """Dense arrays of the active slots for a bucket of n rows (active slots first, ascending)."""
+        L.check(L.lib().uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                           self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), L.stream_ptr(self.act)),
+                "uvmi_sched_compact")
+        self._dense_n = n
+
     def _step_body(self, n: int):
+        """One decode step on the dense arrays of bucket n (compacted by the caller when they are stale: after an admission,
+        or when the bucket changes); the commit carries them to the next step, so a step has no compaction launch."""
         e, cfg, st = self.e, self.cfg, self.st
         lib = L.lib()
         sp = L.stream_ptr(self.act)
-        L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
-                                       self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
         act, pos, starts = self.act[:n], self.pos_c[:n], self.starts_c[:n]
 
         def attn(l, q):
@@ -263,8 +273,9 @@ class Rollout:
             tok, lp = self._sample(x, self.req_c[:n], self.cnt_c[:n])
         else:
             tok, lp = greedy_sample(x, cfg.softcap)
-        L.check(lib.uvmi_sched_commit(C.byref(self.sched), n, self.act.data_ptr(), tok.data_ptr(), lp.data_ptr(),
-                                      self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit")
+        L.check(lib.uvmi_sched_commit_dense(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                            self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), tok.data_ptr(),
+                                            lp.data_ptr(), self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit_dense")
 
     def _attention(self, l, q, st, pos, starts, n, act):
         return self.e.cache_attention(l, q, st, pos, starts, n, rows=act)
@@ -281,11 +292,14 @@ class Rollout:
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
+            if not mixed:
+                self._compact(n)   # (a bucket below the active count raises the overflow flag: restored with the rest)
             body(n)
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         for t, k in zip(self._mutable(), keep):
             t.copy_(k)
+        self._dense_n = None
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             body(n)
@@ -304,20 +318,33 @@ class Rollout:
                     self._capture(min(n, self.B), mixed=True)
 
     @torch.no_grad()
+    def step_inputs(self):
+        """(n, slot, token, position, start) of the rows the next step() will run: views of the dense step arrays of its
+        bucket of n rows (slot -1: padding).  step() overwrites them with the following step's."""
+        n = self.bucket_for(self.n_active_host)
+        if self._dense_n != n:
+            self._compact(n)
+        return n, self.act[:n], self.tok_c[:n], self.pos_c[:n], self.starts_c[:n]
+
+    @torch.no_grad()
     def step(self):
         """One decode step for every active slot (graph replay of the bucket that covers the active count)."""
         n = self.bucket_for(self.n_active_host)
-        if not self.use_graph:
+        g = (self.graphs.get(n) or self._capture(n)) if self.use_graph else None
+        if self._dense_n != n:
+            self._compact(n)
+        if g is None:
             self._step_body(n)
         else:
-            (self.graphs.get(n) or self._capture(n)).replay()
+            g.replay()
         self.n_decode_steps += 1
 
     def _mutable(self):
         """State a decode step writes.  The KV cache is left out on purpose: the warm-up step writes K/V at the current
         positions, and the real replay rewrites exactly those slots with identical inputs (as in model.py:1126-1127)."""
         return [self.slot_req, self.slot_cnt, self.slot_limit, self.slot_tok, self.st.pos, self.st.starts, self.out_tok, self.out_lp,
-                self.done_req, self.done_slot, self.done_cnt, self.counters]
+                self.done_req, self.done_slot, self.done_cnt, self.counters, self.act, self.tok_c, self.pos_c, self.starts_c, self.req_c,
+                self.cnt_c]
 
     # ------------------------------------------------------------------------------------------------ harvest
     @torch.no_grad()
