@@ -230,6 +230,7 @@ int uvmi_prefill_attn_path(const uvmi_prefill_attn_args* a);
  * Fused softcap + categorical draw + behaviour log-prob.  Replaces fused_sample
  * (ultraviolet/kernels/fused_sample.py:68-77) and the torch.rand call feeding it (ultraviolet/perf.py:595).
  * ---------------------------------------------------------------------------------------------------------- */
+struct uvmi_sample_commit;
 typedef struct uvmi_sample_args {
   const void* x; int x_dtype;      /* (B, V) raw head output before the softcap; F16 / BF16 / F32 */
   int64_t stride;                  /* row stride of x */
@@ -249,6 +250,8 @@ typedef struct uvmi_sample_args {
    * logp stays the log-prob under the untruncated softmax, as the reference records it (model.py:1161-1169). */
   int top_k; float top_p;
   float* thr_out;                  /* optional (B,): the smallest kept exp((z - a) / T) (0 when nothing is filtered) */
+  const struct uvmi_sample_commit* commit; /* optional: the rows are the dense rows of a decode step, and the launch also does
+                                      uvmi_sched_commit_dense for them (declared with the slot table below) */
 } uvmi_sample_args;
 int uvmi_fused_sample(const uvmi_sample_args* a, void* stream);
 /* Host-side Philox4x32-10 (Random123) for tests and host tooling: out[4] = philox(ctr[4], key[2]). */
@@ -355,6 +358,15 @@ int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const int64_t* ac
 int uvmi_sched_commit_dense(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c,
                             int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, const int64_t* new_tok,
                             const float* new_lp, float retire_p, uint64_t seed, void* stream);
+/* uvmi_fused_sample's optional commit: row i of the sampler is dense row i of the step, and the thread that writes the
+ * row's token and log-prob then commits them as uvmi_sched_commit_dense does (same retirement draw), which saves the
+ * step a launch.  req_c / cnt_c may be the sampler's req_id / tok_idx arrays. */
+typedef struct uvmi_sample_commit {
+  const uvmi_sched_state* state;
+  int64_t* act_slot; int64_t* tok_c; int64_t* pos_c; int64_t* starts_c; int64_t* req_c; int64_t* cnt_c;
+  float retire_p; uint64_t seed;
+} uvmi_sample_commit;
+
 /* Bind n freshly prefilled requests to slots and record their first sampled token (model.py:1306-1313,
  * rl_stream.py:86-92). */
 int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, const int64_t* req_ids,

@@ -104,6 +104,59 @@ def test_slot_table_kernels_bit_exact(B, bucket, retire_p):
     assert len(tab.done) > 0 and sorted(harvested) == sorted((r, sl, min(c, max_new)) for r, sl, c in tab.done)
 
 
+@pytest.mark.parametrize("mode", ["sample", "filtered", "greedy"])
+def test_sampler_with_commit_equals_sampler_then_commit(mode):
+    """The sampler launch that also commits its rows leaves the slot table, the dense step arrays and the completion ring
+    exactly as the sampler followed by uvmi_sched_commit_dense does (all three sampler kernels; rows with EOS, length-limit
+    and seeded random retirement, padding rows)."""
+    from ultraviolet_amd import _lib as L
+    from ultraviolet_amd.kernels.fused_sample import fused_sample_seeded, greedy_sample
+    lib = L.lib()
+    B, bucket, max_new, eos, seed, retire_p, V = 96, 128, 12, 3, 1234, 0.1, 1024
+    rng = np.random.default_rng(5)
+    tt = lambda a, dt=torch.long: torch.as_tensor(np.asarray(a), dtype=dt, device=DEV)
+    softcap = (23.0, 5.0, 7.5)
+    states = []
+    for fused in (False, True):
+        t, s = _dev_table(B, max_new, eos)
+        k = 70
+        slots = rng.permutation(B)[:k] if not states else states[0]["slots"]
+        if not states:
+            init = dict(slots=slots, reqs=np.arange(k) + (1 << 33), lim=rng.integers(1, max_new + 1, size=k), ft=rng.integers(0, 8, size=k),
+                        flp=rng.random(k, dtype=np.float32), pos=rng.integers(1, 50, size=k), x=rng.standard_normal((4, bucket, V)).astype(np.float32))
+            init["x"][:, :, :8] += 6.0     # most draws land on tokens 0..7, so EOS (3) is hit now and then
+        else:
+            init = states[0]["init"]
+        t["pos"][tt(slots)] = tt(init["pos"])
+        a = [tt(slots), tt(init["reqs"]), tt(init["lim"]), tt(init["ft"]), tt(init["flp"], torch.float32)]
+        L.check(lib.uvmi_sched_admit(C.byref(s), k, *[v.data_ptr() for v in a], None), "admit")
+        dense = [torch.zeros(bucket, dtype=torch.long, device=DEV) for _ in range(6)]
+        L.check(lib.uvmi_sched_compact(C.byref(s), bucket, *[d.data_ptr() for d in dense], None), "compact")
+        commit = L.SampleCommit(C.pointer(s), *[d.data_ptr() for d in dense], retire_p, seed)
+        for step in range(4):
+            x = tt(init["x"][step], torch.bfloat16)
+            kw = dict(commit=commit) if fused else {}
+            if mode == "greedy":
+                tok, lp = greedy_sample(x, softcap, **kw)
+            else:
+                tok, lp = fused_sample_seeded(x, seed, dense[4], dense[5], softcap, 1.0, top_k=5 if mode == "filtered" else 0, **kw)
+            if not fused:
+                L.check(lib.uvmi_sched_commit_dense(C.byref(s), bucket, *[d.data_ptr() for d in dense], tok.data_ptr(), lp.data_ptr(), retire_p,
+                                                    seed, None), "commit_dense")
+        torch.cuda.synchronize()
+        n_done = int(t["counters"][1])
+        ring = sorted(zip(t["done_req"][:n_done].tolist(), t["done_slot"][:n_done].tolist(), t["done_cnt"][:n_done].tolist()))
+        states.append(dict(slots=slots, init=init, t={k_: v.cpu().numpy() for k_, v in t.items() if not k_.startswith("done_")},
+                           dense=[d.cpu().numpy() for d in dense], ring=ring))
+    a, b = states
+    assert len(a["ring"]) > 5 and a["ring"] == b["ring"]
+    for k_ in a["t"]:
+        assert np.array_equal(a["t"][k_], b["t"][k_]), k_
+    for j in range(6):
+        assert np.array_equal(a["dense"][j], b["dense"][j]), j
+    assert (a["dense"][0] >= 0).sum() > 5      # some rows go on
+
+
 def _engine(dtype=torch.float32, window=16, max_tokens=1024):
     from ultraviolet_amd.engine import UVEngine, UVWeights, make_config, random_params
     cfg = make_config("uv-test", window=window)

@@ -80,7 +80,7 @@ class SampleArgs(C.Structure):
                 ("tok", C.c_void_p), ("logp", C.c_void_p), ("u_out", C.c_void_p),
                 ("B", C.c_int), ("V", C.c_int),
                 ("cap_a", C.c_float), ("cap_b", C.c_float), ("cap_c", C.c_float), ("temperature", C.c_float),
-                ("top_k", C.c_int), ("top_p", C.c_float), ("thr_out", C.c_void_p)]
+                ("top_k", C.c_int), ("top_p", C.c_float), ("thr_out", C.c_void_p), ("commit", C.c_void_p)]
 
 
 class QkvPostArgs(C.Structure):
@@ -102,6 +102,11 @@ class SchedState(C.Structure):
                 ("pos", C.c_void_p), ("starts", C.c_void_p), ("out_tok", C.c_void_p), ("out_lp", C.c_void_p),
                 ("done_req", C.c_void_p), ("done_slot", C.c_void_p), ("done_cnt", C.c_void_p), ("counters", C.c_void_p),
                 ("max_new", C.c_int64), ("eos_id", C.c_int64), ("B", C.c_int), ("done_cap", C.c_int)]
+
+
+class SampleCommit(C.Structure):
+    _fields_ = [("state", C.POINTER(SchedState)), ("act_slot", C.c_void_p), ("tok_c", C.c_void_p), ("pos_c", C.c_void_p),
+                ("starts_c", C.c_void_p), ("req_c", C.c_void_p), ("cnt_c", C.c_void_p), ("retire_p", C.c_float), ("seed", C.c_uint64)]
 
 
 _lib = None

@@ -14,6 +14,7 @@
 // drawn from Philox4x32-10 keyed by the seed with counter (token index, request id lo, request id hi, "SAMP"), so a
 // request's stream does not depend on the slot it occupies.
 #include "common.h"
+#include "sched_commit.h"
 
 namespace uvmi {
 
@@ -42,7 +43,16 @@ struct SampleParams {
   float neg_a_over_t;           // -(a/T)
   float cap_a, cap_b, cap_c, inv_c;
   int top_k; float top_p; float* thr_out;
+  // optional: commit the drawn token to the slot table in the same launch (row = dense row of a decode step)
+  int commit; float retire_p; uint64_t commit_seed; uvmi_sched_state S; DenseArrays D;
 };
+
+// The row's result; with P.commit also what uvmi_sched_commit_dense does for the row (one thread per row calls this).
+__device__ __forceinline__ void emit(const SampleParams P, int row, int tok, float logp) {
+  P.tok[row] = tok;
+  P.logp[row] = logp;
+  if (P.commit) commit_row<true>(P.S, P.D, row, tok, logp, P.retire_p, P.commit_seed);
+}
 
 template <int DT>
 __device__ __forceinline__ void load8(const void* row, int i, float (&o)[8]) {  // elements 8i .. 8i+7
@@ -152,11 +162,10 @@ __global__ __launch_bounds__(NT) void sample_kernel(const void* a_x, int64_t a_s
   }
   if (lane == 0) {
     const int tok = ck * CHUNK + ln * 8 + jsel;
-    P.tok[row] = tok;
     // logp = (z_tok - a)/T - log S, with (z - a)/T = -(a/T) / (1 + exp(t))
     const float E = __builtin_amdgcn_exp2f(fmaf(xsel, P.inv_c_l2, P.b_over_c_l2));
-    P.logp[row] = P.neg_a_over_t * __builtin_amdgcn_rcpf(1.0f + E) - __logf(S);
     if (P.u_out) P.u_out[row] = u;
+    emit(P, row, tok, P.neg_a_over_t * __builtin_amdgcn_rcpf(1.0f + E) - __logf(S));
   }
 }
 
@@ -374,11 +383,10 @@ __global__ __launch_bounds__(256) void sample_filtered_kernel(SampleParams P) {
     }
   }
   if (lane == 0) {
-    P.tok[row] = ck * CHUNK + sel;
     const float E = __builtin_amdgcn_exp2f(fmaf(xsel, P.inv_c_l2, P.b_over_c_l2));
-    P.logp[row] = P.neg_a_over_t * __builtin_amdgcn_rcpf(1.0f + E) - __logf(S);
     if (P.u_out) P.u_out[row] = u;
     if (P.thr_out) P.thr_out[row] = __uint_as_float(thr);
+    emit(P, row, ck * CHUNK + sel, P.neg_a_over_t * __builtin_amdgcn_rcpf(1.0f + E) - __logf(S));
   }
 }
 
@@ -419,10 +427,9 @@ __global__ __launch_bounds__(256) void argmax_kernel(SampleParams P) {
       tot += ssum[w];
       if (smax[w] > best || (smax[w] == best && sidx[w] < bi)) { best = smax[w]; bi = sidx[w]; }
     }
-    P.tok[row] = bi;
     const float E = __builtin_amdgcn_exp2f(fmaf(best, P.inv_c_l2, P.b_over_c_l2));
-    P.logp[row] = -P.cap_a * __builtin_amdgcn_rcpf(1.0f + E) - __logf(tot);
     if (P.u_out) P.u_out[row] = 0.f;
+    emit(P, row, bi, -P.cap_a * __builtin_amdgcn_rcpf(1.0f + E) - __logf(tot));
   }
 }
 
@@ -464,6 +471,19 @@ extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
   P.top_k = a->top_k > 0 && a->top_k < a->V ? a->top_k : 0;
   P.top_p = a->top_p > 0.f && a->top_p < 1.0f ? a->top_p : 1.0f;
   P.thr_out = a->thr_out;
+  P.commit = 0;
+  if (a->commit) {
+    const uvmi_sample_commit* c = a->commit;
+    UVMI_REQUIRE(c->state && c->act_slot && c->tok_c && c->pos_c && c->starts_c && c->req_c && c->cnt_c, UVMI_EINVAL,
+                 "uvmi_fused_sample: null pointer in commit");
+    const uvmi_sched_state* t = c->state;
+    UVMI_REQUIRE(t->slot_req && t->slot_cnt && t->slot_limit && t->slot_tok && t->pos && t->starts && t->out_tok && t->counters && t->done_req &&
+                     t->done_slot && t->done_cnt && t->B > 0 && t->max_new > 0 && t->done_cap > 0, UVMI_EINVAL,
+                 "uvmi_fused_sample: bad slot table in commit");
+    // the kernel reads req_id / tok_idx of a row before it rewrites the row's dense entries, so they may be the same arrays
+    P.commit = 1; P.retire_p = c->retire_p; P.commit_seed = c->seed; P.S = *t;
+    P.D = DenseArrays{c->act_slot, c->tok_c, c->pos_c, c->starts_c, c->req_c, c->cnt_c};
+  }
   const bool filtered = !greedy && (P.top_k > 0 || P.top_p < 1.0f);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(a->B), blk(256);

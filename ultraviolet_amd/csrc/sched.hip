@@ -14,21 +14,9 @@
 //
 // Both are integer bookkeeping on <= a few thousand slots: latency-bound, one workgroup / one thread per row.
 #include "common.h"
+#include "sched_commit.h"
 
 namespace uvmi {
-
-constexpr uint32_t DOMAIN_RETIRE = 0x52455452u;
-
-__device__ inline void philox_round10(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
-#pragma unroll
-  for (int r = 0; r < 10; r++) {
-    const uint64_t p0 = (uint64_t)0xD2511F53u * c[0], p1 = (uint64_t)0xCD9E8D57u * c[2];
-    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0, n1 = (uint32_t)p1, n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1, n3 = (uint32_t)p0;
-    c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
-    k0 += 0x9E3779B9u;
-    k1 += 0xBB67AE85u;
-  }
-}
 
 // One workgroup of 1024 threads; slots are handled in tiles of 1024 with a running base (ordered compaction).
 __global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, int64_t* tok_c,
@@ -77,47 +65,13 @@ __global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S,
   }
 }
 
-// DENSE: the step's dense arrays are carried to the next step in place of a new compaction - a row that goes on gets its
-// new token, position and token index, a row that retires becomes padding (slot -1, zeros) where it stands.
+// One thread per dense row (see commit_row).
 template <bool DENSE>
-__global__ __launch_bounds__(256) void sched_commit_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, const int64_t* new_tok,
-                                                           const float* new_lp, float retire_p, uint64_t seed, int64_t* tok_c,
-                                                           int64_t* pos_c, int64_t* starts_c, int64_t* req_c, int64_t* cnt_c) {
+__global__ __launch_bounds__(256) void sched_commit_kernel(uvmi_sched_state S, int n_bucket, DenseArrays D, const int64_t* new_tok,
+                                                           const float* new_lp, float retire_p, uint64_t seed) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= n_bucket) return;
-  const int64_t slot = act_slot[i];
-  if (slot < 0) return;
-  const int64_t tok = new_tok[i];
-  const int64_t c = S.slot_cnt[slot];
-  const int64_t col = c < S.max_new ? c : S.max_new - 1;   // clamp like the reference's buffers (rl_stream.py:122)
-  S.out_tok[slot * S.max_new + col] = (int32_t)tok;
-  if (S.out_lp) S.out_lp[slot * S.max_new + col] = new_lp ? new_lp[i] : 0.f;
-  S.slot_cnt[slot] = c + 1;
-  S.slot_tok[slot] = tok;
-  S.pos[slot] += 1;
-  bool fin = (c + 1 >= S.slot_limit[slot]) || (S.eos_id >= 0 && tok == S.eos_id);
-  const int64_t req = S.slot_req[slot];
-  if (!fin && retire_p > 0.f) {
-    uint32_t ctr[4] = {(uint32_t)c, (uint32_t)req, (uint32_t)((uint64_t)req >> 32), DOMAIN_RETIRE};
-    philox_round10(ctr, (uint32_t)seed, (uint32_t)(seed >> 32));
-    fin = (float)(ctr[0] >> 8) * 5.9604644775390625e-08f < retire_p;
-  }
-  if (fin) {
-    const int k = atomicAdd(&S.counters[1], 1) % S.done_cap;  // ring: the host must poll before done_cap more rows finish
-    S.done_req[k] = req;
-    S.done_slot[k] = slot;
-    S.done_cnt[k] = c + 1;
-    S.slot_req[slot] = -1;
-    S.pos[slot] = 0;      // parked: never overruns the cache (model.py:1345-1350)
-    S.starts[slot] = 0;
-  }
-  if (DENSE) {
-    act_slot[i] = fin ? -1 : slot;
-    tok_c[i] = fin ? 0 : tok;
-    pos_c[i] = fin ? 0 : pos_c[i] + 1;
-    cnt_c[i] = fin ? 0 : c + 1;
-    if (fin) { starts_c[i] = 0; req_c[i] = 0; }
-  }
+  commit_row<DENSE>(S, D, i, new_tok[i], new_lp ? new_lp[i] : 0.f, retire_p, seed);
 }
 
 // Admission after a prefill: bind request ids to slots and record the first sampled token (it counts as token 0 of
@@ -241,8 +195,9 @@ extern "C" int uvmi_sched_commit(const uvmi_sched_state* s, int n_bucket, const 
   int rc = check_state(s, "uvmi_sched_commit");
   if (rc) return rc;
   UVMI_REQUIRE(n_bucket > 0 && act_slot && new_tok, UVMI_EINVAL, "uvmi_sched_commit: bad arguments");
-  hipLaunchKernelGGL(sched_commit_kernel<false>, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket,
-                     const_cast<int64_t*>(act_slot), new_tok, new_lp, retire_p, seed, nullptr, nullptr, nullptr, nullptr, nullptr);
+  const DenseArrays D{const_cast<int64_t*>(act_slot), nullptr, nullptr, nullptr, nullptr, nullptr};
+  hipLaunchKernelGGL(sched_commit_kernel<false>, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket, D, new_tok,
+                     new_lp, retire_p, seed);
   UVMI_CHECK_LAUNCH("uvmi_sched_commit");
   return UVMI_OK;
 }
@@ -254,8 +209,9 @@ extern "C" int uvmi_sched_commit_dense(const uvmi_sched_state* s, int n_bucket, 
   if (rc) return rc;
   UVMI_REQUIRE(n_bucket > 0 && act_slot && tok_c && pos_c && starts_c && req_c && cnt_c && new_tok, UVMI_EINVAL,
                "uvmi_sched_commit_dense: bad arguments");
-  hipLaunchKernelGGL(sched_commit_kernel<true>, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket, act_slot,
-                     new_tok, new_lp, retire_p, seed, tok_c, pos_c, starts_c, req_c, cnt_c);
+  const DenseArrays D{act_slot, tok_c, pos_c, starts_c, req_c, cnt_c};
+  hipLaunchKernelGGL(sched_commit_kernel<true>, dim3((n_bucket + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_bucket, D, new_tok,
+                     new_lp, retire_p, seed);
   UVMI_CHECK_LAUNCH("uvmi_sched_commit_dense");
   return UVMI_OK;
 }

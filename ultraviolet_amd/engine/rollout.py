@@ -68,6 +68,9 @@ class Rollout:
         self.act, self.tok_c, self.pos_c = self.row_all[Np:], self.tok_all[Np:], self.pos_all[Np:]
         self.req_c, self.cnt_c = self.req_all[A:], self.cnt_all[A:]
         self.starts_c = z(slots)
+        self._commit_args = L.SampleCommit(C.pointer(self.sched), self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                           self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), self.retire_p,
+                                           self.seed & (2 ** 64 - 1))
         if mixed:
             # admission staging, one host -> device copy per mixed step: [tokens Np | cu A+1 | slot A | start A | limit A | req A]
             self.stage_n = Np + (A + 1) + 3 * A
@@ -166,10 +169,10 @@ class Rollout:
             self.n_active_host += len(batch)
             self._dense_n = None
 
-    def _sample(self, x, req, cnt):
+    def _sample(self, x, req, cnt, commit=None):
         if self.T > 0:
-            return fused_sample_seeded(x, self.seed, req, cnt, self.cfg.softcap, self.T, top_k=self.top_k, top_p=self.top_p)
-        return greedy_sample(x, self.cfg.softcap)
+            return fused_sample_seeded(x, self.seed, req, cnt, self.cfg.softcap, self.T, top_k=self.top_k, top_p=self.top_p, commit=commit)
+        return greedy_sample(x, self.cfg.softcap, commit=commit)
 
     @torch.no_grad()
     def _admit_mixed(self) -> bool:
@@ -269,13 +272,8 @@ class Rollout:
         fused = (lambda l: e.fused_cache_attention(l, self.tok_c[:n], st, pos, starts, n, rows=act)) if e.fuse_qkv else None
         h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st, fused_attn=fused)
         x = e.head(h)
-        if self.T > 0:
-            tok, lp = self._sample(x, self.req_c[:n], self.cnt_c[:n])
-        else:
-            tok, lp = greedy_sample(x, cfg.softcap)
-        L.check(lib.uvmi_sched_commit_dense(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
-                                            self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), tok.data_ptr(),
-                                            lp.data_ptr(), self.retire_p, self.seed & (2 ** 64 - 1), sp), "uvmi_sched_commit_dense")
+        # the sampler's launch also commits the rows' tokens (what uvmi_sched_commit_dense does in a launch of its own)
+        self._sample(x, self.req_c[:n], self.cnt_c[:n], commit=self._commit_args)
 
     def _attention(self, l, q, st, pos, starts, n, act):
         return self.e.cache_attention(l, q, st, pos, starts, n, rows=act)

@@ -23,7 +23,7 @@ def fused_sample_ok(x_or_dev, V: int, softcap, temperature: float, block: int = 
                 and a / temperature <= 80.0)
 
 
-def _run(x, u, softcap, temperature, seed, req_id, tok_idx, want_u, top_k=0, top_p=1.0, want_thr=False):
+def _run(x, u, softcap, temperature, seed, req_id, tok_idx, want_u, top_k=0, top_p=1.0, want_thr=False, commit=None):
     L.require_cuda(x, u, req_id, tok_idx)
     B, V = x.shape
     assert x.stride(1) == 1 and V % BLOCK == 0
@@ -35,7 +35,9 @@ def _run(x, u, softcap, temperature, seed, req_id, tok_idx, want_u, top_k=0, top
                      int(seed) & (2 ** 64 - 1), None if req_id is None else req_id.data_ptr(),
                      None if tok_idx is None else tok_idx.data_ptr(), tok.data_ptr(), lp.data_ptr(),
                      None if uo is None else uo.data_ptr(), B, V, a, b, c, float(temperature), int(top_k), float(top_p),
-                     None)
+                     None, None)
+    if commit is not None:   # an _lib.SampleCommit: the launch also commits the rows' tokens to the slot table
+        s.commit = C.addressof(commit)
     thr = None
     if want_thr:
         thr = torch.zeros(B, dtype=torch.float32, device=x.device)
@@ -54,20 +56,21 @@ def fused_sample(x: Tensor, u: Tensor, softcap, temperature: float = 1.0, block:
 
 
 def fused_sample_seeded(x: Tensor, seed: int, req_id: Tensor, tok_idx: Tensor, softcap, temperature: float = 1.0,
-                        return_u: bool = False, top_k: int = 0, top_p: float = 1.0):
+                        return_u: bool = False, top_k: int = 0, top_p: float = 1.0, commit=None):
     """Same draw with u = Philox4x32-10(key = seed, counter = (tok_idx, req_id, "SAMP")) generated in the kernel:
     replaces the torch.rand(B) feeding the reference's sampler (ultraviolet/perf.py:595) with a stream keyed by request
     and token index, so it does not depend on slot placement.  req_id, tok_idx: (B,) int64.  top_k / top_p truncate the
-    distribution as sample() does (model.py:1200-1209; see sample_filtered)."""
+    distribution as sample() does (model.py:1200-1209; see sample_filtered).  commit (an _lib.SampleCommit): the rows are the
+    dense rows of a decode step and the launch also commits their tokens to the slot table (uvmi_sched_commit_dense)."""
     assert req_id.dtype == torch.int64 and tok_idx.dtype == torch.int64
-    tok, lp, uo = _run(x, None, softcap, temperature, seed, req_id.contiguous(), tok_idx.contiguous(), return_u, top_k, top_p)
+    tok, lp, uo = _run(x, None, softcap, temperature, seed, req_id.contiguous(), tok_idx.contiguous(), return_u, top_k, top_p, commit=commit)
     return (tok, lp, uo) if return_u else (tok, lp)
 
 
-def greedy_sample(x: Tensor, softcap) -> tuple[Tensor, Tensor]:
+def greedy_sample(x: Tensor, softcap, commit=None) -> tuple[Tensor, Tensor]:
     """argmax (first maximal index) of the head output and log softmax(softcap(x))[argmax]: the T <= 0 branch of the
-    reference's sample() (ultraviolet/model.py:1198-1199) fused with the log-prob."""
-    tok, lp, _ = _run(x, None, softcap, 0.0, 0, None, None, False)
+    reference's sample() (ultraviolet/model.py:1198-1199) fused with the log-prob.  commit: as in fused_sample_seeded."""
+    tok, lp, _ = _run(x, None, softcap, 0.0, 0, None, None, False, commit=commit)
     return tok, lp
 
 
