@@ -22,7 +22,7 @@ from ..kernels.decode_attn import (build_attn_args, build_fused_args, decode_att
 from ..kernels.gemm import RESID, SWIGLU, gemm_tn
 from ..kernels.kv_quant import kv_write
 from ..kernels.varlen_attn import packed_attention
-from ..kernels.fused_sample import fused_sample, fused_sample_seeded, greedy_sample
+from ..kernels.fused_sample import fused_sample_seeded, greedy_sample
 from .config import UVConfig
 from .weights import UVWeights
 

@@ -261,9 +261,7 @@ class Rollout:
     def _step_body(self, n: int):
         """One decode step on the dense arrays of bucket n (compacted by the caller when they are stale: after an admission,
         or when the bucket changes); the commit carries them to the next step, so a step has no compaction launch."""
-        e, cfg, st = self.e, self.cfg, self.st
-        lib = L.lib()
-        sp = L.stream_ptr(self.act)
+        e, st = self.e, self.st
         act, pos, starts = self.act[:n], self.pos_c[:n], self.starts_c[:n]
 
         def attn(l, q):
