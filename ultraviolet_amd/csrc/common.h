@@ -39,6 +39,15 @@ __device__ __forceinline__ uint16_t float_to_bf16(float f) {
   __builtin_memcpy(&r, &b, 2);
   return r;
 }
+// two floats rounded to bf16 in one conversion (v_cvt_pk_bf16_f32): a in the low half of the word
+__device__ __forceinline__ uint32_t float2_to_bf16x2(float a, float b) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 r = __builtin_convertvector(f32x2{a, b}, bf16x2);
+  uint32_t w;
+  __builtin_memcpy(&w, &r, 4);
+  return w;
+}
 __device__ __forceinline__ float half_bits_to_float(uint16_t b) {
   half_t h;
   __builtin_memcpy(&h, &b, 2);
