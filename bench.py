@@ -78,7 +78,7 @@ def bench_c5(args):
 
     def make_rollout(use_graph):
         g = Rollout(eng, slots=n_seq, max_prompt=256, max_new=2048, temperature=1.0, seed=0, eos_id=None, check_every=16,
-                    bucket=64, use_graph=use_graph)
+                    bucket=32, use_graph=use_graph)
         for i, (p, l) in enumerate(zip(prompts, limits)):
             g.add(p, i, limit=l)
         return g
