@@ -2,5 +2,6 @@
 on-device continuous-batching loop.  Mirrors the inference half of ultraviolet/model.py and
 ultraviolet/kernels/fast_decode.py of the reference."""
 from .config import PRESETS, UVConfig, make_config  # noqa: F401
+from .evals import int8_check, teacher_forced_logits  # noqa: F401
 from .model import KVState, UVEngine  # noqa: F401
 from .weights import UVWeights, random_params  # noqa: F401
