@@ -498,7 +498,9 @@ extern "C" int uvmi_fused_sample(const uvmi_sample_args* a, void* stream) {
   else {
 #define UVMI_SK(DT, NT) \
   hipLaunchKernelGGL((sample_kernel<DT, NT>), grid, dim3(NT), 0, st, P.x, P.stride, P.V, P.inv_c_l2, P.b_over_c_l2, P.neg_a_over_t_l2, P)
-    const bool wide = a->B <= 256;  // (the chunk sums are formed per chunk whatever the width: the draw does not depend on it)
+    // 1024 threads per row are faster up to ~640 rows (measured: 12.0 against 14.5 us at 384 rows), slower from 1024 on; the
+    // chunk sums are formed per chunk whatever the width, so the draw does not depend on it
+    const bool wide = a->B <= 640;
     if (a->x_dtype == UVMI_F16) { if (wide) UVMI_SK(UVMI_F16, 1024); else UVMI_SK(UVMI_F16, 256); }
     else if (a->x_dtype == UVMI_BF16) { if (wide) UVMI_SK(UVMI_BF16, 1024); else UVMI_SK(UVMI_BF16, 256); }
     else { if (wide) UVMI_SK(UVMI_F32, 1024); else UVMI_SK(UVMI_F32, 256); }
