@@ -437,13 +437,15 @@ class UVEngine:
         cu[1:] = np.cumsum(lens)
         N = int(cu[-1])
         assert N <= self.max_tokens, f"{N} prefill tokens exceed the engine's max_tokens {self.max_tokens}"
-        x = np.fromiter((t for p in prompts for t in p), dtype=np.int64, count=N)
+        x = np.concatenate([np.asarray(p, dtype=np.int64) for p in prompts])   # (prompts may be lists or int arrays)
         seg = np.repeat(np.arange(len(prompts), dtype=np.int64), lens)
         pos = np.arange(N, dtype=np.int64) - cu[:-1][seg] + starts[seg]
         rows_np = np.asarray(rows, dtype=np.int64)
-        tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-        return dict(N=N, tok=tt(x), pos=tt(pos), row=tt(rows_np[seg]), last=tt((starts + lens - 1)[seg]), cu=tt(cu),
-                    last_idx=tt(cu[1:] - 1), rows=tt(rows_np), starts=tt(starts), ends=tt(starts + lens))
+        # one host -> device copy for all nine arrays
+        parts = [x, pos, rows_np[seg], (starts + lens - 1)[seg], cu, cu[1:] - 1, rows_np, starts, starts + lens]
+        flat = torch.from_numpy(np.concatenate(parts)).to(dev)
+        tok, pos_t, row, last, cu_t, last_idx, rows_t, starts_t, ends = flat.split([len(a) for a in parts])
+        return dict(N=N, tok=tok, pos=pos_t, row=row, last=last, cu=cu_t, last_idx=last_idx, rows=rows_t, starts=starts_t, ends=ends)
 
     @staticmethod
     def bind_prompts(pk: dict, st: KVState):

@@ -152,15 +152,11 @@ class Rollout:
             slots = [self.free.pop() for _ in batch]
             reqs = list(range(self.next_req, self.next_req + len(batch)))
             self.next_req += len(batch)
-            h = e.prefill([b[0] for b in batch], slots, self.st, left_pad=self.left_pad)
+            h = e.prefill([b[3] for b in batch], slots, self.st, left_pad=self.left_pad)
             x = e.head(h)
-            tt = lambda a: torch.as_tensor(a, dtype=torch.long, device=self.dev)
-            req_t = tt(reqs)
-            if self.T > 0:
-                tok, lp = self._sample(x, req_t, torch.zeros_like(req_t))
-            else:
-                tok, lp = greedy_sample(x, self.cfg.softcap)
-            slot_t, lim_t = tt(slots), tt([b[2] for b in batch])   # named: they must outlive the launch call
+            # request ids, slots and limits in one host -> device copy (named: they must outlive the launch call)
+            req_t, slot_t, lim_t = torch.as_tensor([reqs, slots, [b[2] for b in batch]], dtype=torch.long).to(self.dev).unbind(0)
+            tok, lp = self._sample(x, req_t, torch.zeros_like(req_t))
             rc = L.lib().uvmi_sched_admit(C.byref(self.sched), len(batch), slot_t.data_ptr(), req_t.data_ptr(), lim_t.data_ptr(),
                                           tok.data_ptr(), lp.data_ptr(), L.stream_ptr(tok))
             L.check(rc, "uvmi_sched_admit")
