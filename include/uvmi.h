@@ -301,6 +301,9 @@ typedef struct uvmi_qkv_post_args {
   const float* gate_w; int gate_ch;    /* (H, gate_ch) fp32 output-gate weights */
   float* gate_out;                     /* (n, H) fp32: 2 sigmoid(gate_w[h] . xn[:gate_ch]), rounded as in dtype; or NULL */
   float* vhat_out; float xsa_eps;      /* (n, KH, hd) fp32: v / max(|v|, xsa_eps); or NULL */
+  /* optional: uvmi_rope_table's output in dtype's rounding for positions 0 .. rope_positions - 1; tokens at those positions
+   * read their cos / sin from it (the same values the kernel would compute), others compute them */
+  const float* rope_table; int rope_positions;
 } uvmi_qkv_post_args;
 int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream);
 

@@ -143,6 +143,7 @@ struct QkvArgs {
   int64_t n, vocab;
   int H, KH, d, ve_ch, n_pairs, S, ring, has_ve, rope, q_dt, gate_ch;
   float eps, xsa_eps;
+  const float* rope_tab; int rope_n;   // optional table of the rounded cos / sin per position (row: cos[n_pairs], sin[n_pairs])
 };
 
 template <int DT>
@@ -154,6 +155,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
   const int64_t base = r * W;
   const int64_t p = A.pos[r];
   const int np_ = A.n_pairs;
+  const float* tab = A.rope_tab && p >= 0 && p < A.rope_n ? A.rope_tab + p * 2 * np_ : nullptr;   // (wave-uniform)
   // ---- queries: lane (hh = lane / 8, c = lane % 8) owns dims 8c..8c+7 of head 8*pass + hh
   {
     const int hh = lane >> 3, c = lane & 7;
@@ -163,9 +165,14 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
     {
       float cl = 1.f, sl = 0.f;
       if (A.rope && lane < np_) {
-        const float th = (float)p * A.inv_freq[lane];
-        cl = round_t<DT>(cosf(th));
-        sl = round_t<DT>(sinf(th));
+        if (tab) {
+          cl = tab[lane];
+          sl = tab[np_ + lane];
+        } else {
+          const float th = (float)p * A.inv_freq[lane];
+          cl = round_t<DT>(cosf(th));
+          sl = round_t<DT>(sinf(th));
+        }
       }
 #pragma unroll
       for (int j = 0; j < 8; j++) {
@@ -236,9 +243,14 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
   float cs1 = 1.f, sn1 = 0.f;
   const bool rot1 = A.rope && lane < 2 * np_;
   if (rot1) {
-    const float th = (float)p * A.inv_freq[lane % np_];
-    cs1 = round_t<DT>(cosf(th));
-    sn1 = round_t<DT>(sinf(th));
+    if (tab) {
+      cs1 = tab[lane % np_];
+      sn1 = tab[np_ + lane % np_];
+    } else {
+      const float th = (float)p * A.inv_freq[lane % np_];
+      cs1 = round_t<DT>(cosf(th));
+      sn1 = round_t<DT>(sinf(th));
+    }
   }
   const int64_t row = A.rows ? A.rows[r] : r;
   const int64_t slot = A.ring ? (p % A.S) : p;
@@ -450,6 +462,8 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   A.H = a->H; A.KH = a->KH; A.d = a->d; A.ve_ch = a->ve_ch; A.n_pairs = a->n_pairs; A.S = a->S; A.ring = a->ring; A.has_ve = a->has_ve;
   A.rope = a->rope; A.q_dt = a->q_dtype; A.eps = a->eps;
   A.gate_w = a->gate_w; A.gate_out = a->gate_out; A.vhat_out = a->vhat_out; A.gate_ch = a->gate_ch; A.xsa_eps = a->xsa_eps;
+  A.rope_tab = a->rope && a->rope_positions > 0 ? a->rope_table : nullptr;
+  A.rope_n = a->rope_positions;
   const dim3 grid((unsigned)((a->n + 3) / 4)), blk(256);
   dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
   UVMI_CHECK_LAUNCH("uvmi_qkv_post");

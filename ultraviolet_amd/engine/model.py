@@ -143,6 +143,9 @@ class UVEngine:
         a.H, a.KH, a.hd, a.d, a.ve_ch, a.n_pairs = cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_model, cfg.ve_gate_channels, cfg.n_pairs
         a.ring, a.has_ve = int(not glob), int(has_ve)
         a.rope = int(((not glob) or cfg.global_rope) and cfg.n_pairs > 0)
+        if a.rope and st is not None:   # cos / sin from the table of the state's positions instead of per-token cosf / sinf
+            tab = self.rope_table(st.max_len)
+            a.rope_table, a.rope_positions = tab.data_ptr(), tab.size(0)
         a.eps = self.eps
         if cfg.xsa:
             a.vhat_out, a.xsa_eps = b["vhat"].data_ptr(), float(cfg.xsa_eps)
