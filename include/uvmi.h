@@ -226,6 +226,23 @@ size_t uvmi_prefill_attn_workspace_bytes(int N);
 /* 1 = MFMA kernel, 0 = generic kernel, negative = unsupported */
 int uvmi_prefill_attn_path(const uvmi_prefill_attn_args* a);
 
+/* Backward of uvmi_prefill_attn: replaces mathk::varlen_attn_bwd (ultraviolet/kernels/varlen_attn.py:56-66, the
+ * aten._efficient_attention_backward call with K / V expanded to the query heads and their gradients summed back over the
+ * group).  All tensors contiguous: q, o, go, dq (N, H, hd); k, v, dk, dv (N, KH, hd), one 16-bit dtype, head_dim 64;
+ * cu_seqlens (n_seg + 1,) as in the forward.  The row log-sum-exp is recomputed (the forward does not return it).  fp32
+ * arithmetic on the vector units (a first, plain form: no matrix cores).  workspace: (2 N H) fp32 (lse and go . o). */
+typedef struct uvmi_prefill_attn_bwd_args {
+  const void* q; const void* k; const void* v; const void* o; const void* go; int dtype;
+  void* dq; void* dk; void* dv;
+  const void* cu_seqlens; int idx_dtype; int n_seg;
+  int N, H, KH, hd;
+  float scale;
+  int window;                              /* 0 = none */
+  void* workspace; size_t workspace_bytes; /* >= uvmi_prefill_attn_bwd_workspace_bytes(N, H) */
+} uvmi_prefill_attn_bwd_args;
+int uvmi_prefill_attn_bwd(const uvmi_prefill_attn_bwd_args* a, void* stream);
+size_t uvmi_prefill_attn_bwd_workspace_bytes(int N, int H);
+
 /* ------------------------------------------------------------------------------------------------------------
  * Fused softcap + categorical draw + behaviour log-prob.  Replaces fused_sample
  * (ultraviolet/kernels/fused_sample.py:68-77) and the torch.rand call feeding it (ultraviolet/perf.py:595).

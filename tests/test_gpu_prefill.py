@@ -177,3 +177,53 @@ def test_packed_attention_fused_post_epilogue(dtype, window):
     assert float((err / (want.abs() + 1.0)).max()) <= 3 * ulp, float((err / (want.abs() + 1.0)).max())
     no_gate = packed_attention(q, k, v, cu, 0.125, window, workspace=ws, post=(vhat, None, None))
     assert float((no_gate.double() - z).abs().max()) <= 2 * ulp * float(z.abs().max())
+
+
+def _grad_case(lens, H, K, dtype, window, seed=0):
+    from oracle.varlen_attn import varlen_attention_grad_ref
+    from ultraviolet_amd.kernels import varlen_attention
+    q, k, v, cu = _case(lens, H, K, 64, dtype, seed=seed)
+    go = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 100)).to(dtype)
+    qd, kd, vd = (t[None].to(DEV).requires_grad_() for t in (q, k, v))
+    o = varlen_attention(qd, kd, vd, cu.to(DEV), max(max(lens), 1), SC, window)
+    o.backward(go[None].to(DEV))
+    torch.cuda.synchronize()
+    ref = varlen_attention_grad_ref(to_np(q), to_np(k), to_np(v), to_np(go), to_np(cu), SC, window)
+    got = [to_np(t.grad[0]).astype(np.float64) for t in (qd, kd, vd)]
+    return got, ref
+
+
+@pytest.mark.parametrize("window", [None, 256])
+def test_backward_reference_case_fp16(window):
+    """The reference's own test of the varlen backward (tests/test_perf_opt.py:40-61): lens [300, 1000, 57, 700, 1], 8 query
+    heads on 1 kv head, fp16, window None / 256, gradients through autograd; its bar: |g - g_ref| / |g_ref| < 5e-3 for each
+    of dq, dk, dv (norms over the whole tensor)."""
+    got, ref = _grad_case([300, 1000, 57, 700, 1], 8, 1, torch.float16, window)
+    for a, b in zip(got, ref):
+        assert np.isfinite(a).all()
+        assert np.linalg.norm(a - b) / np.linalg.norm(b) < 5e-3, np.linalg.norm(a - b) / np.linalg.norm(b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("lens,H,K,window", [([1], 8, 1, None), ([0, 5, 0, 0, 40, 0], 8, 1, 16), ([31, 33, 64, 1, 2, 95, 7], 8, 2, 33),
+                                             ([70, 3], 4, 4, 1), ([130], 2, 1, None), ([65, 64, 63], 8, 8, 64)])
+def test_backward_ragged_and_edges(dtype, lens, H, K, window):
+    """Empty and single-token segments, segment boundaries inside a wave's 64 queries / 32 keys, window 1 (every query sees
+    only itself: dq = dk = 0 up to rounding, dv = go summed over the group), grouped and per-head K / V."""
+    got, ref = _grad_case(lens, H, K, dtype, window, seed=3)
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for a, b in zip(got, ref):
+        assert np.isfinite(a).all()
+        assert np.abs(a - b).max() <= 2 * ulp * max(np.abs(b).max(), 1e-3) + 1e-6, (np.abs(a - b).max(), np.abs(b).max())
+
+
+def test_backward_rejects_what_it_cannot_do():
+    from ultraviolet_amd import _lib as L
+    from ultraviolet_amd.kernels.varlen_attn import packed_attention_backward
+    cu = torch.tensor([0, 4], dtype=torch.int32, device=DEV)
+    z = lambda *s_, dt=torch.float16: torch.zeros(*s_, dtype=dt, device=DEV)
+    with pytest.raises(L.UvmiError):   # head_dim 32
+        packed_attention_backward(z(4, 2, 32), z(4, 2, 32), z(4, 1, 32), z(4, 1, 32), z(4, 2, 32), cu, 1.0)
+    with pytest.raises(L.UvmiError):   # fp32 tensors
+        packed_attention_backward(*(z(4, 2, 64, dt=torch.float32) for _ in range(2)), *(z(4, 1, 64, dt=torch.float32) for _ in range(2)),
+                                  z(4, 2, 64, dt=torch.float32), cu, 1.0)

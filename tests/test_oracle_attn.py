@@ -109,3 +109,57 @@ def test_varlen_matches_sdpa_per_segment(window):
         z = torch.nn.functional.scaled_dot_product_attention(q[a:b].double().transpose(0, 1), k[a:b].double().transpose(0, 1).expand(8, Lq, 64),
                                                              v[a:b].double().transpose(0, 1).expand(8, Lq, 64), attn_mask=m, scale=0.14125)
         np.testing.assert_allclose(out[a:b], z.transpose(0, 1).numpy(), atol=3e-5, rtol=3e-5)
+
+
+@pytest.mark.parametrize("window", [None, 3])
+def test_varlen_grad_matches_finite_differences_and_autograd(window):
+    """Pins oracle.varlen_attn.varlen_attention_grad_ref twice: by central differences of the forward restatement (float64,
+    every input element of a tiny ragged case with an empty segment and grouped kv heads), and by torch autograd through a
+    masked softmax written with torch ops (the formulation of the reference's test, tests/test_perf_opt.py:40-61)."""
+    rng = np.random.default_rng(7)
+    lens = [4, 0, 6, 1]
+    N, H, K, hd, sc = sum(lens), 4, 2, 8, 0.37
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    q, k, v, go = (rng.standard_normal(s_) for s_ in ((N, H, hd), (N, K, hd), (N, K, hd), (N, H, hd)))
+
+    def fwd64(q_, k_, v_):   # the forward restatement, in float64
+        out = np.zeros((N, H, hd))
+        for a, b in zip(cu[:-1], cu[1:]):
+            if b == a:
+                continue
+            i = np.arange(b - a)
+            d = i[:, None] - i[None, :]
+            m = (d >= 0) & ((d < window) if window else True)
+            for h in range(H):
+                s_ = np.where(m, q_[a:b, h] @ k_[a:b, h // (H // K)].T * sc, -np.inf)
+                w = np.exp(s_ - s_.max(-1, keepdims=True))
+                out[a:b, h] = (w / w.sum(-1, keepdims=True)) @ v_[a:b, h // (H // K)]
+        return out
+    np.testing.assert_allclose(fwd64(q, k, v), varlen_attn.varlen_attention_ref(q, k, v, cu, sc, window), atol=2e-6)
+    dq, dk, dv = varlen_attn.varlen_attention_grad_ref(q, k, v, go, cu, sc, window)
+    eps = 1e-6
+    for x, gx, idx in ((q, dq, 0), (k, dk, 1), (v, dv, 2)):
+        num = np.zeros_like(x)
+        for pos in np.ndindex(x.shape):
+            args = [q.copy(), k.copy(), v.copy()]
+            args[idx][pos] += eps
+            up = (fwd64(*args) * go).sum()
+            args[idx][pos] -= 2 * eps
+            num[pos] = (up - (fwd64(*args) * go).sum()) / (2 * eps)
+        np.testing.assert_allclose(gx, num, atol=2e-8 + 1e-6 * np.abs(num).max())
+    # torch autograd
+    tq, tk, tv = (torch.tensor(x, dtype=torch.float64, requires_grad=True) for x in (q, k, v))
+    outs = []
+    for a, b in zip(cu[:-1], cu[1:]):
+        if b == a:
+            continue
+        i = torch.arange(b - a)
+        d = i[:, None] - i[None, :]
+        m = (d >= 0) & ((d < window) if window else torch.ones_like(d, dtype=torch.bool))
+        kk = tk[a:b].repeat_interleave(H // K, dim=1).transpose(0, 1)
+        vv = tv[a:b].repeat_interleave(H // K, dim=1).transpose(0, 1)
+        s_ = (tq[a:b].transpose(0, 1) @ kk.transpose(1, 2) * sc).masked_fill(~m, float("-inf"))
+        outs.append((s_.softmax(-1) @ vv).transpose(0, 1))
+    (torch.cat(outs) * torch.tensor(go)).sum().backward()
+    for gx, t in ((dq, tq), (dk, tk), (dv, tv)):
+        np.testing.assert_allclose(gx, t.grad.numpy(), atol=1e-12, rtol=1e-10)

@@ -65,6 +65,14 @@ class PrefillAttnArgs(C.Structure):
                 ("segments_ready", C.c_int), ("post_vhat", C.c_void_p), ("post_gate", C.c_void_p), ("post_xsa", C.c_void_p)]
 
 
+class PrefillAttnBwdArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("go", C.c_void_p), ("dtype", C.c_int),
+                ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+                ("cu_seqlens", C.c_void_p), ("idx_dtype", C.c_int), ("n_seg", C.c_int),
+                ("N", C.c_int), ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int), ("scale", C.c_float), ("window", C.c_int),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 class KvAppendArgs(C.Structure):
     _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("x_dtype", C.c_int), ("sxb", C.c_int64), ("sxh", C.c_int64),
                 ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
@@ -130,6 +138,9 @@ def lib() -> C.CDLL:
         L.uvmi_prefill_attn_path.argtypes = [C.POINTER(PrefillAttnArgs)]
         L.uvmi_prefill_attn_workspace_bytes.restype = C.c_size_t
         L.uvmi_prefill_attn_workspace_bytes.argtypes = [C.c_int]
+        L.uvmi_prefill_attn_bwd.argtypes = [C.POINTER(PrefillAttnBwdArgs), C.c_void_p]
+        L.uvmi_prefill_attn_bwd_workspace_bytes.restype = C.c_size_t
+        L.uvmi_prefill_attn_bwd_workspace_bytes.argtypes = [C.c_int, C.c_int]
         L.uvmi_quantize_rows.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int64, C.c_void_p, C.c_void_p,
                                          C.c_void_p]
         L.uvmi_dequantize_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
@@ -187,4 +198,4 @@ EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu", "uvmi_swiglu_norm",
-           "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_commit_dense", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]
+           "uvmi_prefill_attn_bwd", "uvmi_prefill_attn_bwd_workspace_bytes", "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_commit_dense", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]

@@ -1,7 +1,8 @@
 """Packed (cu_seqlens) causal attention with an optional sliding window: host side of uvmi_prefill_attn.
 
-Mirrors ultraviolet/kernels/varlen_attn.py:87-93 of the reference (forward only; the reference's backward belongs to
-the trainer).  q / k / v must be device tensors; there is no CPU path."""
+Mirrors ultraviolet/kernels/varlen_attn.py of the reference: the forward (:87-93) on the MFMA kernel, and the backward
+(:56-84) in a first, plain form (uvmi_prefill_attn_bwd), wired into autograd as the reference wires its custom ops.
+q / k / v must be device tensors; there is no CPU path."""
 from __future__ import annotations
 
 import ctypes as C
@@ -79,9 +80,49 @@ def packed_attention_path(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, s
     return int(L.lib().uvmi_prefill_attn_path(C.byref(a)))
 
 
+def packed_attention_backward(go: Tensor, q: Tensor, k: Tensor, v: Tensor, o: Tensor, cu_seqlens: Tensor, scale: float,
+                              window: int | None = None) -> tuple[Tensor, Tensor, Tensor]:
+    """(dq, dk, dv) of packed_attention for the output gradient go: q, o, go (N, H, 64), k, v (N, K, 64), one 16-bit dtype
+    (reference: mathk::varlen_attn_bwd, varlen_attn.py:56-66; gradients of K / V are summed over the heads of a group)."""
+    L.require_cuda(go, q, k, v, o, cu_seqlens)
+    assert q.dim() == 3 and k.dim() == 3 and k.shape == v.shape and q.shape == o.shape == go.shape
+    assert q.dtype == k.dtype == v.dtype == o.dtype == go.dtype
+    assert cu_seqlens.dim() == 1 and cu_seqlens.numel() >= 1 and cu_seqlens.is_contiguous()
+    go, q, k, v, o = (t.contiguous() for t in (go, q, k, v, o))
+    N, H, hd = q.shape
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ws = torch.empty(L.lib().uvmi_prefill_attn_bwd_workspace_bytes(N, H), dtype=torch.uint8, device=q.device)
+    a = L.PrefillAttnBwdArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), go.data_ptr(), L.dtype_code(q.dtype),
+                             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), cu_seqlens.data_ptr(), L.dtype_code(cu_seqlens.dtype),
+                             cu_seqlens.numel() - 1, N, H, k.size(1), hd, float(scale), int(window or 0), ws.data_ptr(), ws.numel())
+    L.check(L.lib().uvmi_prefill_attn_bwd(C.byref(a), L.stream_ptr(q)), "uvmi_prefill_attn_bwd")
+    return dq, dk, dv
+
+
+class _PackedAttention(torch.autograd.Function):
+    """packed_attention with the backward above (the reference registers its pair of custom ops with autograd the same
+    way, varlen_attn.py:69-84)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens, scale, window):
+        o = packed_attention(q, k, v, cu_seqlens, scale, window)
+        ctx.save_for_backward(q, k, v, o, cu_seqlens)
+        ctx.scale, ctx.window = scale, window
+        return o
+
+    @staticmethod
+    def backward(ctx, go):
+        q, k, v, o, cu = ctx.saved_tensors
+        dq, dk, dv = packed_attention_backward(go, q, k, v, o, cu, ctx.scale, ctx.window)
+        return dq, dk, dv, None, None, None
+
+
 def varlen_attention(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, max_seqlen: int, scale: float,
                      window: int | None = None) -> Tensor:
     """The reference's signature: q (1, N, H, hd), k / v (1, N, K, hd) packed along N, cu_seqlens (S+1,) with cu[0] = 0
-    and cu[-1] = N; returns (1, N, H, hd).  max_seqlen is accepted for compatibility (the kernel does not need it)."""
+    and cu[-1] = N; returns (1, N, H, hd).  max_seqlen is accepted for compatibility (the kernel does not need it).
+    Differentiable in q, k, v (16-bit inputs, head_dim 64)."""
     assert q.dim() == 4 and q.size(0) == 1 and k.size(0) == 1 and v.size(0) == 1
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _PackedAttention.apply(q[0], k[0], v[0], cu_seqlens, float(scale), int(window or 0))[None]
     return packed_attention(q[0], k[0], v[0], cu_seqlens, scale, window)[None]
