@@ -435,3 +435,37 @@ def test_rollout_with_truncated_sampling_draws_inside_the_nucleus():
         assert int(rank.max()) < K, rank
         ref_lp = torch.log_softmax(lg, -1).gather(1, torch.as_tensor(toks)[:, None])[:, 0]
         assert float((ref_lp - torch.as_tensor(lps)).abs().max()) < 5e-2            # bf16 logits: the replay is not bit-identical
+
+
+@pytest.mark.parametrize("dtype,left_pad", [(torch.float32, False), (torch.bfloat16, True)])
+def test_shared_prompts_are_prefilled_once_and_copied(dtype, left_pad):
+    """A sampling group (the same prompt under several requests, as in the GRPO rollout) is prefilled once and its cache rows
+    are copied: after admission every member's cache, position and start equal the first member's bit for bit, greedy
+    continuations of a group are identical, and the rollout returns what the one that prefills every request returns."""
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg, eng = _engine(dtype, window=16)
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(2, cfg.vocab_size, size=int(n)).tolist() for n in (5, 23, 9, 31)]
+    outs = []
+    for share in (True, False):
+        g = Rollout(eng, slots=12, max_prompt=32, max_new=20, temperature=0.0, check_every=4, bucket=4, left_pad=left_pad, share_prompts=share)
+        for i in range(12):
+            g.add(prompts[i // 3], i)      # groups of 3
+        g._admit()
+        torch.cuda.synchronize()
+        if share:
+            slot_of = {int(r): s_ for s_, r in enumerate(g.slot_req.tolist()) if r >= 0}
+            for grp in range(4):
+                a = slot_of[3 * grp]
+                for m in (1, 2):
+                    b_ = slot_of[3 * grp + m]
+                    assert int(g.st.pos[a]) == int(g.st.pos[b_]) and int(g.st.starts[a]) == int(g.st.starts[b_])
+                    for l in range(cfg.n_layers):
+                        assert torch.equal(g.st.k[l][a], g.st.k[l][b_]) and torch.equal(g.st.v[l][a], g.st.v[l][b_])
+                        assert torch.equal(g.st.k_scale[l][a], g.st.k_scale[l][b_]) and torch.equal(g.st.v_scale[l][a], g.st.v_scale[l][b_])
+        outs.append({m: row for m, row, _, _ in g.run(max_chunks=200)})
+        assert sorted(outs[-1]) == list(range(12))
+    for grp in range(4):
+        assert outs[0][3 * grp] == outs[0][3 * grp + 1] == outs[0][3 * grp + 2]
+    same = sum(outs[0][i] == outs[1][i] for i in range(12))
+    assert same >= (12 if dtype == torch.float32 else 9), same

@@ -57,6 +57,19 @@ class KVState:
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.k + self.v + self.k_scale + self.v_scale if t is not None)
 
+    @torch.no_grad()
+    def copy_rows(self, src: Tensor, dst: Tensor, upto: int):
+        """Cache rows dst <- cache rows src for the first `upto` slots of every layer, with pos and starts (src, dst: (n,)
+        int64 on the device).  A sequence's cache depends only on its own tokens and quantisation is per row, so a prompt
+        shared by several sequences is prefilled once and copied: the copies hold the bytes their own prefill would write."""
+        for l in range(self.cfg.n_layers):
+            for t in (self.k[l], self.v[l], self.k_scale[l], self.v_scale[l]):
+                if t is not None:
+                    n = min(upto, t.size(2))
+                    t[dst, :, :n] = t[src, :, :n]
+        self.pos[dst] = self.pos[src]
+        self.starts[dst] = self.starts[src]
+
 
 def kv_bytes_per_seq(cfg: UVConfig, ctx: int) -> int:
     """int8 cache bytes of one sequence at context ctx (reference: fast_decode.py:64-67)."""

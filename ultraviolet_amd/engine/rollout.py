@@ -29,7 +29,8 @@ class Rollout:
     def __init__(self, engine: UVEngine, slots: int, max_prompt: int, max_new: int, temperature: float = 1.0,
                  seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
                  use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False,
-                 admit_cap: int = 16, top_k: int = 0, top_p: float = 1.0, kv_dtype: str = "int8", overlap_harvest: bool = False):
+                 admit_cap: int = 16, top_k: int = 0, top_p: float = 1.0, kv_dtype: str = "int8", overlap_harvest: bool = False,
+                 share_prompts: bool = False):
         self.e, self.cfg = engine, engine.cfg
         self.top_k, self.top_p = int(top_k), float(top_p)   # truncated sampling (sample(), model.py:1200-1209); off by default
         self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
@@ -93,6 +94,7 @@ class Rollout:
         self._hv_stream = torch.cuda.Stream(device=dev)   # default priority; carries only the harvest's device -> host copies
         self.harvest_pending = False
         self.overlap_harvest = bool(overlap_harvest)
+        self.share_prompts = bool(share_prompts)   # admission prefills identical prompts of a call once and copies their cache rows
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.mixed_graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.queue = collections.deque()
@@ -105,6 +107,7 @@ class Rollout:
         self.version = 0
         self.n_decode_steps = 0
         self.n_tokens = 0
+        self.n_prefill_tokens = 0                 # prompt tokens that went through a prefill pass of _admit (shared prompts once)
 
     # ------------------------------------------------------------------------------------------------ requests
     def add(self, prompt_ids, meta, limit: int | None = None):
@@ -142,17 +145,38 @@ class Rollout:
         """Prefill queued requests into free slots (FIFO), in calls of at most engine.max_tokens packed tokens."""
         e = self.e
         while self.queue and self.free:
-            batch, ntok = [], 0
-            while self.queue and len(batch) < len(self.free) and ntok + len(self.queue[0][0]) <= e.max_tokens:
-                it = self.queue.popleft()
+            # prompts that occur several times in the call (a sampling group) are prefilled once: only their first occurrence
+            # counts against the pass's token budget
+            batch, ntok, first, src = [], 0, {}, []
+            while self.queue and len(batch) < len(self.free):
+                it = self.queue[0]
+                key = it[3].tobytes() if self.share_prompts else None
+                new = key is None or key not in first
+                if new and ntok + len(it[0]) > e.max_tokens:
+                    break
+                self.queue.popleft()
+                if key is not None:
+                    src.append(first.setdefault(key, len(batch)))
+                if new:
+                    ntok += len(it[0])
                 batch.append(it)
-                ntok += len(it[0])
             if not batch:
                 raise RuntimeError("a queued prompt exceeds the engine's max_tokens")
             slots = [self.free.pop() for _ in batch]
             reqs = list(range(self.next_req, self.next_req + len(batch)))
             self.next_req += len(batch)
-            h = e.prefill([b[3] for b in batch], slots, self.st, left_pad=self.left_pad)
+            self.n_prefill_tokens += ntok
+            if len(first) < len(batch) and self.share_prompts:
+                uniq = sorted(first.values())
+                at = {j: u for u, j in enumerate(uniq)}
+                h = e.prefill([batch[j][3] for j in uniq], [slots[j] for j in uniq], self.st, left_pad=self.left_pad)
+                dup = [j for j in range(len(batch)) if src[j] != j]
+                ix = torch.as_tensor([[at[s_] for s_ in src], [slots[s_] for s_ in src], slots], dtype=torch.long).to(self.dev)
+                d_ix = torch.as_tensor(dup, dtype=torch.long).to(self.dev)
+                self.st.copy_rows(ix[1][d_ix], ix[2][d_ix], max(len(batch[j][3]) for j in uniq))
+                h = h.index_select(0, ix[0])
+            else:
+                h = e.prefill([b[3] for b in batch], slots, self.st, left_pad=self.left_pad)
             x = e.head(h)
             # request ids, slots and limits in one host -> device copy (named: they must outlive the launch call)
             req_t, slot_t, lim_t = torch.as_tensor([reqs, slots, [b[2] for b in batch]], dtype=torch.long).to(self.dev).unbind(0)
