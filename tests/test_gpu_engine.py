@@ -359,11 +359,13 @@ def test_large_pass_plans_match_unfused(dtype, plan):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("lens,window,max_len", [((100, 130, 90, 150, 129, 64), 128, 192), ((300, 420, 260, 500, 257, 300), 256, 576)])
+@pytest.mark.parametrize("lens,window,max_len", [((100, 130, 90, 150, 129, 64), 128, 192), ((300, 420, 260, 500, 257, 300), 256, 576),
+                                                 ((300, 20, 260, 330, 1, 300), 1024, 1056)])
 def test_fused_qkv_single_layer_is_exact_with_several_waves_per_row(dtype, lens, window, max_len):
     """Caches of 128..255 slots run the attention kernel with 2 waves per row and longer ones with 4 (own key formed by the
     first wave, own value by the second, q handed over through LDS): the appended bytes must still equal the separate
-    post-processing kernel's, on a ring layer (wraps during the run) and on a global layer."""
+    post-processing kernel's, on a ring layer (wraps during the run where it is shorter than the rows) and on a global
+    layer, also on caches of more than 1024 slots."""
     for over in (dict(window=window, global_every=0, ve_every=1), dict(window=0, global_every=1, ve_every=0)):
         cfg, params, eng, _ = _setup("uv-test", dtype=dtype, perturb=0.05, n_layers=1, attn_gate_channels=128, **over)
         assert eng.fuse_qkv

@@ -60,6 +60,20 @@ def test_global_ragged(dtype, int8, B, KH, G, hd, splits):
     _attn_check(q, k, v, ks, vs, pos, starts, 1.13 / hd ** 0.5, splits=splits)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,S,ring", [(3, 1056, False), (200, 1056, False), (300, 2080, False), (500, 1024, False), (40, 1024, True)])
+def test_few_and_many_rows_on_long_caches(dtype, B, S, ring):
+    """Caches of >= 1024 slots with 3 .. 500 rows: rows from one key to the whole cache, left-padded starts, a ring of 1024
+    slots several times around - rows that leave most of a workgroup's waves without a tile next to rows that fill it."""
+    q, k, v, ks, vs = attn_case(B, 1, 8, 64, S, True, dtype=dtype)
+    g = torch.Generator().manual_seed(B + S)
+    pos = torch.randint(0, S if not ring else 5 * S, (B,), generator=g)
+    pos[0], pos[1 % B] = (S - 1 if not ring else 3 * S + 17), 0
+    starts = (torch.rand(B, generator=g) * (pos + 1).float()).long()
+    starts[0] = 0
+    _attn_check(q, k, v, ks, vs, pos, starts, 1.13 / 8, window=S if ring else 0, ring=ring)
+
+
 @pytest.mark.parametrize("int8", [False, True])
 @pytest.mark.parametrize("W,hd,G", [(128, 128, 5), (256, 64, 8), (1024, 128, 4), (100, 128, 4), (64, 64, 8),
                                     (100, 64, 8)])
