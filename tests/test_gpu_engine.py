@@ -123,20 +123,25 @@ def _force_plan(eng, plan):
         eng.skinny_rows, eng.fold_qkv_rows, eng.fold_o_rows = _TRUNK_PLANS[plan]
 
 
+@pytest.mark.parametrize("dtype,max_bar,mean_bar", [(torch.bfloat16, 0.15, 0.02), (torch.float16, 0.04, 0.005)])
 @pytest.mark.parametrize("plan", list(_TRUNK_PLANS))
-def test_bf16_engine_close_to_oracle(plan):
-    """reference bar for the int8 kernel path vs its SDPA path: max |logit diff| < 0.25, argmax agreement > 0.9
-    (tests/test_math_kernels.py:170-172) - for each of the decode pass's launch plans (the one for few rows, and the two
-    for many rows: residual updates inside the projections, the MLP's pre-norm inside the SwiGLU launch)."""
-    cfg, params, eng, OracleModel = _setup(dtype=torch.bfloat16, window=16)
+def test_16bit_engine_close_to_oracle(plan, dtype, max_bar, mean_bar):
+    """The 16-bit engine against the oracle run in the same 16-bit arithmetic (both sides use the int8 cache and round at
+    the same points), for each of the decode pass's launch plans (the one for few rows, and the two for many rows:
+    residual updates inside the projections, the MLP's pre-norm inside the SwiGLU launch).  Bars: twice the measured gap -
+    bf16 max 0.062-0.077 / mean 0.0099, fp16 max 0.016-0.020 / mean 0.0026 on logits in (0, 23), i.e. one or two units in
+    the last place of the tied head's 16-bit output; every argmax agrees.  (The reference's bar for its int8 kernel path
+    against its unquantized SDPA path is 0.25 / 0.9, tests/test_math_kernels.py:170-172.)"""
+    cfg, params, eng, OracleModel = _setup(dtype=dtype, window=16)
     _force_plan(eng, plan)
     prompts = _prompts(cfg, (5, 12, 9, 20, 3, 17))
     cont = np.random.default_rng(1).integers(1, cfg.vocab_size, size=(6, 30))
     lg, _ = _teacher_forced(eng, prompts, cont, 64)
-    ref, _ = _oracle_teacher_forced(OracleModel(cfg, params, torch.bfloat16), prompts, cont, 64)
+    ref, _ = _oracle_teacher_forced(OracleModel(cfg, params, dtype), prompts, cont, 64)
     assert np.isfinite(lg).all()
-    assert np.abs(lg - ref).max() < 0.25
-    assert (lg.argmax(-1) == ref.argmax(-1)).mean() > 0.9
+    d = np.abs(lg - ref)
+    assert d.max() < max_bar and d.mean() < mean_bar, (d.max(), d.mean())
+    assert (lg.argmax(-1) == ref.argmax(-1)).mean() > 0.98
 
 
 def test_graph_replay_matches_eager_and_seeded_sampling_is_reproducible():

@@ -93,12 +93,32 @@ inline int dtype_bytes(int dt) {
 }
 
 // wave64 butterfly reductions (ds_bpermute based; used off the hot loops)
-// One element of the partial rotation: x cos - y sin for the first half of a pair, x cos + y sin for the second, as one
-// fma on the rounded product y sin.  Every kernel that rotates q or k goes through here, so they round alike.
-__device__ __forceinline__ float rope_rot(float x, float y, float c, float s, bool first) {
-  const float t = __fmul_rn(y, s);
-  return __builtin_fmaf(x, c, first ? -t : t);
+// a * b and a + b as operations of their own.  The compiler narrows float arithmetic on values that came from fp16 to
+// native fp16 instructions and, with floating-point contraction on (the HIP default), would then fuse such a product and
+// sum into one v_fma_f16 - one rounding where the reference's tensor expressions on 16-bit tensors round twice.  The
+// pragma takes the contraction permission off these two operations wherever they are inlined.
+__device__ __forceinline__ float mul_sep(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
 }
+__device__ __forceinline__ float add_sep(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+
+// One element of the partial rotation: x cos - y sin for the first half of a pair, x cos + y sin for the second, with the
+// roundings of the reference's expression x1 * cos - x2 * sin on tensors of the activation type (ultraviolet/model.py:219-226):
+// each product is rounded to that type (rnd), then their sum.  Every kernel that rotates q or k goes through here, so
+// they round alike.
+template <class R>
+__device__ __forceinline__ float rope_rot(float x, float y, float c, float s, bool first, R rnd) {
+  const float a = rnd(mul_sep(x, c)), t = rnd(mul_sep(y, s));
+  return rnd(add_sep(a, first ? -t : t));
+}
+
+// v + g * e with the roundings of the reference's v + g * ve on tensors of the activation type (ultraviolet/model.py:312-315)
+template <class R>
+__device__ __forceinline__ float ve_add(float v, float g, float e, R rnd) { return rnd(add_sep(v, rnd(mul_sep(g, e)))); }
 
 __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

@@ -321,7 +321,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       const bool first = cc < 2, rot = cc < 4;
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        const float v = rq(rope_rot(x[j], dpp_mov<0x4e>(x[j]), cs[j], sn[j], first));
+        const float v = rope_rot(x[j], dpp_mov<0x4e>(x[j]), cs[j], sn[j], first, rq);
         x[j] = rot ? v : x[j];
       }
     }
@@ -363,7 +363,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     const float rs = rsqrtf(bfly_sum(k * k) * (1.0f / 64.0f) + P.f_eps);
     k = rq(k * rs);
     if (P.f_rope) {
-      const float kr = rq(rope_rot(k, lane_xor16(k), kcs, ksn, lane < 16));
+      const float kr = rope_rot(k, lane_xor16(k), kcs, ksn, lane < 16, rq);
       k = lane < 32 ? kr : k;
     }
     uint16_t sbk;
@@ -395,7 +395,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     float v = cvt_in(raw);
     if (P.f_has_ve) {
       const float gv = rq(2.0f * rq(1.0f / (1.0f + __expf(-cvt_in(vlog)))));
-      v = rq(v + rq(gv * cvt_in(raw_ve)));
+      v = ve_add(v, gv, cvt_in(raw_ve), rq);
     }
     const float nv = fmaxf(sqrtf(bfly_sum(v * v)), P.f_xsa_eps);
     uint16_t sbv;

@@ -207,7 +207,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
         for (int j = 0; j < 8; j++) y[j] = __shfl_xor(x[j], pl, 64);  // partner chunk: c <-> c ^ pl inside the head
         if (rot) {
 #pragma unroll
-          for (int j = 0; j < 8; j++) x[j] = round_t<DT>(rope_rot(x[j], y[j], cs[j], sn[j], first));
+          for (int j = 0; j < 8; j++) x[j] = rope_rot(x[j], y[j], cs[j], sn[j], first, [](float f) { return round_t<DT>(f); });
         }
       }
       if (h < A.H) {
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       k = round_t<DT>(k * rs);
       if (A.rope) {
         const float other = __shfl_xor(k, np_, 64);
-        if (rot1) k = round_t<DT>(rope_rot(k, other, cs1, sn1, lane < np_));
+        if (rot1) k = rope_rot(k, other, cs1, sn1, lane < np_, [](float f) { return round_t<DT>(f); });
       }
     }
     float v = elem<DT>::ld(A.qkv, base + (A.H + A.KH + kh) * 64 + lane);
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       if (t < 0) t = 0;
       if (t >= A.vocab) t = A.vocab - 1;
       const float ve = elem<DT>::ld(A.ve_table, (t * A.KH + kh) * 64 + lane);
-      v = round_t<DT>(v + round_t<DT>(g * ve));
+      v = ve_add(v, g, ve, [](float f) { return round_t<DT>(f); });
     }
     if (A.k_out) elem<DT>::st(A.k_out, (r * A.KH + kh) * 64 + lane, k);
     if (A.v_out) elem<DT>::st(A.v_out, (r * A.KH + kh) * 64 + lane, v);
