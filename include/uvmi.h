@@ -155,6 +155,19 @@ int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus);
  * G <= 16), negative if unsupported.  Mirrors decode_attn_cuda.supported (decode_attn_cuda.py:265-270). */
 int uvmi_decode_attn_path(const uvmi_attn_args* a);
 
+/* uvmi_decode_attn for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference (its op allocates its split partials per call,
+ * ultraviolet/kernels/decode_attn.py:157-159).  Same arguments, kernels and results as uvmi_decode_attn, except that
+ * workspace / workspace_bytes are ignored: when num_splits > 1 the split partials go to an array of
+ * UVMI_NOALLOC_SCRATCH_BYTES that is part of the library's device code (each GPU the library runs on holds it until the
+ * process ends).  A call whose partials (uvmi_decode_attn_workspace_bytes) exceed it returns UVMI_EWORKSPACE.  The call
+ * makes no hipMalloc / hipFree and no allocating library call; its first use on a device looks the array's address up
+ * once (make that first call outside a graph capture).  Nothing in the array has to start at zero - every partial a
+ * call reads it has written itself - but all calls on one GPU share it: calls that overlap on one GPU (two streams,
+ * two threads) race; serialise them or use uvmi_decode_attn with separate workspaces. */
+#define UVMI_NOALLOC_SCRATCH_BYTES (8u << 20)
+int uvmi_decode_attn_noalloc(const uvmi_attn_args* a, void* stream);
+
 /* ------------------------------------------------------------------------------------------------------------
  * Skinny 16-bit GEMM of a small decode step's projections: C (M, N) = A (M, K) . W (N, K)^T, fp32 accumulation, A, W, C
  * in `dtype` (F16 / BF16), rows contiguous with pitches lda, ldw, ldc (elements).  Replaces the F.linear calls of the

@@ -30,6 +30,7 @@
 #include "common.h"
 
 #include <cstdlib>
+#include <mutex>
 
 namespace uvmi {
 
@@ -999,7 +1000,9 @@ extern "C" int uvmi_decode_attn_path(const uvmi_attn_args* a) {
   return mfma_ok(a) ? 1 : 0;
 }
 
-extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
+// The launch sequence of uvmi_decode_attn with the split partials in `ws` (ws_bytes of device memory; unused when
+// num_splits == 1): the caller's workspace, or this library's own scratch array.
+static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes, const char* who, void* stream) {
   int rc = check_common(a);
   if (rc) return rc;
   if (a->B == 0) return UVMI_OK;
@@ -1040,11 +1043,10 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   }
   if (a->num_splits > 1) {
     const size_t need = uvmi_decode_attn_workspace_bytes(a->B, a->H, a->KH, a->hd, a->num_splits);
-    UVMI_REQUIRE(a->workspace && a->workspace_bytes >= need, UVMI_EWORKSPACE,
-                 "uvmi_decode_attn: workspace of %zu bytes needed, %zu given", need, a->workspace_bytes);
-    UVMI_REQUIRE(((uintptr_t)a->workspace % 16) == 0, UVMI_EWORKSPACE, "uvmi_decode_attn: workspace must be 16-byte aligned");
+    UVMI_REQUIRE(ws && ws_bytes >= need, UVMI_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, ws_bytes);
+    UVMI_REQUIRE(((uintptr_t)ws % 16) == 0, UVMI_EWORKSPACE, "%s: workspace must be 16-byte aligned", who);
     const size_t rows = (size_t)a->B * a->H * a->num_splits;
-    P.ws_o = (float*)a->workspace;
+    P.ws_o = (float*)ws;
     P.ws_m = P.ws_o + rows * a->hd;
     P.ws_l = P.ws_m + rows;
   }
@@ -1111,4 +1113,47 @@ extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
     UVMI_CHECK_LAUNCH("uvmi_decode_attn(combine)");
   }
   return UVMI_OK;
+}
+
+extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
+  UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_decode_attn: null args");
+  return decode_attn_launch(a, a->workspace, a->workspace_bytes, "uvmi_decode_attn", stream);
+}
+
+// ------------------------------------------------------------------------------------ the entry point that allocates nothing
+// Split partials of uvmi_decode_attn_noalloc live in this array instead of a caller's workspace.  It is part of the
+// library's code object: every GPU the library runs on holds its own copy, at its own address, until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress - never a device address.
+static __device__ __align__(256) unsigned char scratch[UVMI_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device ordinal, resolved on the first call there
+}  // namespace
+
+extern "C" int uvmi_decode_attn_noalloc(const uvmi_attn_args* a, void* stream) {
+  UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_decode_attn_noalloc: null args");
+  void* ws = nullptr;
+  if (a->num_splits > 1) {
+    const size_t need = uvmi_decode_attn_workspace_bytes(a->B, a->H, a->KH, a->hd, a->num_splits);
+    UVMI_REQUIRE(need <= (size_t)UVMI_NOALLOC_SCRATCH_BYTES, UVMI_EWORKSPACE,
+                 "uvmi_decode_attn_noalloc: B=%d H=%d num_splits=%d needs %zu bytes of split partials, the built-in scratch holds %zu; "
+                 "use fewer splits or uvmi_decode_attn with a workspace", a->B, a->H, a->num_splits, need, (size_t)UVMI_NOALLOC_SCRATCH_BYTES);
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    UVMI_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, UVMI_EHIP, "uvmi_decode_attn_noalloc: hipGetDevice: %s (device %d)",
+                 hipGetErrorString(e), dev);
+    {
+      std::lock_guard<std::mutex> lock(g_scratch_mu);
+      if (!g_scratch_ptr[dev]) {  // once per device, with that device current
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        UVMI_REQUIRE(e == hipSuccess && p, UVMI_EHIP, "uvmi_decode_attn_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+      }
+      ws = g_scratch_ptr[dev];
+    }
+  }
+  return decode_attn_launch(a, ws, ws ? (size_t)UVMI_NOALLOC_SCRATCH_BYTES : 0, "uvmi_decode_attn_noalloc", stream);
 }
