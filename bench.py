@@ -203,11 +203,6 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
             del built
         if (s + 1) % g.ce == 0:
             g.poll()
-    if os.environ.get("UVMI_BENCH_VERBOSE"):
-        for i, ((a0, a1), (b0, b1), gbts, rbts) in enumerate(samples):
-            ta, tb = a0.elapsed_time(a1) * 1e3 / reps, b0.elapsed_time(b1) * 1e3 / reps
-            print(f"# sample {i}: global {gbts / 1e6:.1f} MB {(ta - tb) / n_glob:.2f} us, ring {rbts / 1e6:.1f} MB {tb / len(ring_layers):.2f} us",
-                  file=sys.stderr)
     eng.qkvx_keep = None
     tA = sum(a.elapsed_time(b) for (a, b), _, _, _ in samples) * 1e3 / reps      # us, all layers, summed over samples
     tB = sum(a.elapsed_time(b) for _, (a, b), _, _ in samples) * 1e3 / reps      # us, ring layers only

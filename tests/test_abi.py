@@ -76,3 +76,118 @@ def test_product_code_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 txt = open(os.path.join(dp, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", txt, flags=re.M), f
+
+
+# ---------------------------------------------------------------------------------------------- header <-> ctypes layout
+_STRUCTS = {"uvmi_attn_args": "AttnArgs", "uvmi_attn_qkv_fuse": "AttnQkvFuse", "uvmi_gemm_args": "GemmArgs",
+            "uvmi_prefill_attn_args": "PrefillAttnArgs", "uvmi_prefill_attn_bwd_args": "PrefillAttnBwdArgs",
+            "uvmi_kv_append_args": "KvAppendArgs", "uvmi_sample_args": "SampleArgs", "uvmi_qkv_post_args": "QkvPostArgs",
+            "uvmi_sched_state": "SchedState", "uvmi_sample_commit": "SampleCommit"}
+_CTYPE = {"int": C.c_int, "int64_t": C.c_int64, "uint64_t": C.c_uint64, "float": C.c_float, "size_t": C.c_size_t}
+
+
+def _header_structs():
+    """{struct name: [(field, C type or 'ptr')]} parsed from include/uvmi.h, in declaration order."""
+    src = open(os.path.join(ROOT, "include", "uvmi.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    out = {}
+    for name, body in re.findall(r"typedef\s+struct\s+(\w+)\s*\{(.*?)\}\s*\w+\s*;", src, flags=re.S):
+        fields = []
+        for decl in body.split(";"):
+            decl = " ".join(decl.split())
+            if not decl:
+                continue
+            m = re.match(r"^(?:const\s+)?(?:struct\s+)?(\w+)\s*(.*)$", decl)
+            base, rest = m.group(1), m.group(2)
+            for d in rest.split(","):
+                d = d.strip()
+                fields.append((d.lstrip("* ").strip(), "ptr" if "*" in d else base))
+        out[name] = fields
+    return out
+
+
+def test_ctypes_structures_follow_the_header_field_for_field():
+    """Order, names and types of every argument structure in ultraviolet_amd/_lib.py against include/uvmi.h, and the dtype
+    codes: a binding that drifts from the header reads garbage without any error."""
+    from ultraviolet_amd import _lib
+    hs = _header_structs()
+    assert set(hs) == set(_STRUCTS), set(hs) ^ set(_STRUCTS)
+    for cname, pyname in _STRUCTS.items():
+        cls = getattr(_lib, pyname)
+        assert [f for f, _ in hs[cname]] == [f[0] for f in cls._fields_], cname
+        for (fname, ctype), (_, pytype) in zip(hs[cname], cls._fields_):
+            if ctype == "ptr":
+                assert pytype is C.c_void_p or issubclass(pytype, C._Pointer), (cname, fname)
+            else:
+                assert pytype is _CTYPE[ctype], (cname, fname, ctype, pytype)
+    hdr = open(os.path.join(ROOT, "include", "uvmi.h")).read()
+    codes = dict(re.findall(r"#define UVMI_(F16|BF16|F32|I8|I32|I64) (\d+)", hdr))
+    assert {k: int(v) for k, v in codes.items()} == dict(F16=_lib.F16, BF16=_lib.BF16, F32=_lib.F32, I8=_lib.I8, I32=_lib.I32, I64=_lib.I64)
+
+
+def test_ctypes_offsets_equal_the_c_compilers(tmp_path):
+    """sizeof and every offsetof as gcc lays the header's structures out, against ctypes' layout of the bindings."""
+    import subprocess
+    from ultraviolet_amd import _lib
+    hs = _header_structs()
+    lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "uvmi.h"', "int main(void) {"]
+    for cname in _STRUCTS:
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for f, _ in hs[cname]:
+            lines.append(f'  printf("{cname}.{f} %zu\\n", offsetof({cname}, {f}));')
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, pyname in _STRUCTS.items():
+        cls = getattr(_lib, pyname)
+        assert int(got[cname]) == C.sizeof(cls), cname
+        for f, _ in hs[cname]:
+            assert int(got[f"{cname}.{f}"]) == getattr(cls, f).offset, (cname, f)
+
+
+def test_reference_names_are_mirrored():
+    """The names the reference's callers import (ultraviolet/kernels/__init__.py:9-10, model.py:867, 886, 942, perf.py:579-625,
+    scripts/rl_grpo.py:1091-1094) exist here; decode_attention_ref / fused_sample_ref are deliberately absent from the
+    product (they are the oracle)."""
+    import torch
+    import ultraviolet_amd.kernels as K
+    from ultraviolet_amd import perf
+    from ultraviolet_amd.kernels import fast_decode, fused_sample, varlen_attn
+    for n in ("decode_attention", "default_splits", "dequantize_kv", "kv_write", "kv_write_rows", "quantize_kv"):
+        assert callable(getattr(K, n))
+    assert not hasattr(K, "decode_attention_ref") and not hasattr(fused_sample, "fused_sample_ref")
+    for n in ("KernelDecodeState", "prefill_fast", "decode_step_fast", "prefill_packed_host", "patch_model", "unpatch_model"):
+        assert hasattr(fast_decode, n)
+    for n in ("fused_sample", "fused_sample_ok"):
+        assert callable(getattr(fused_sample, n))
+    assert callable(varlen_attn.varlen_attention)
+    for n in ("make_streamgen", "install_fz", "StreamGen", "sync_weights_inplace"):
+        assert hasattr(perf, n)
+    assert perf.make_streamgen(perf.StreamGen, ["lp", "hv", "rfh", "fz"]) is perf.StreamGen
+    from ultraviolet_amd import _lib
+    with pytest.raises(_lib.UvmiError):
+        perf.make_streamgen(perf.StreamGen, ["lpp"])
+    s = str(torch.ops.mathk.decode_attn.default._schema)   # the reference's op name and argument list (decode_attn.py:174-178)
+    assert s.startswith("mathk::decode_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor pos, Tensor starts, float scale")
+    assert "num_splits" in s and "block_n" in s and "num_warps" in s and "str backend" in s
+    assert "mathk::varlen_attn_fwd(Tensor q, Tensor k, Tensor v, Tensor cu" in str(torch.ops.mathk.varlen_attn_fwd.default._schema)
+    assert "mathk::varlen_attn_bwd(Tensor go" in str(torch.ops.mathk.varlen_attn_bwd.default._schema)
+    import inspect
+    assert inspect.signature(fast_decode.patch_model).parameters["kv_dtype"].default == "fp16"   # fast_decode.py:341
+
+
+def test_checkpoint_with_unsupported_layers_is_refused():
+    """A reference checkpoint whose cfg switches on MUDD / the bigram table / conv layers / a non-attention local mixer must
+    not load into the attention-only engine with those fields dropped."""
+    from ultraviolet_amd.engine import UVWeights, as_uvconfig, make_config
+    base = make_config("uv-test").to_dict()
+    for extra in (dict(mudd=True), dict(bigram_rows=1024), dict(conv_layers=[1]), dict(local_mixer="gdn")):
+        with pytest.raises(ValueError):
+            UVWeights.from_checkpoint({"model": {}, "cfg": dict(base, **extra)}, device="cpu")
+    import types
+    with pytest.raises(ValueError):
+        as_uvconfig(types.SimpleNamespace(**base, mudd=True))
+    assert as_uvconfig(dict(base, mudd=False, local_mixer="attn")).d_model == base["d_model"]

@@ -451,3 +451,89 @@ def test_int8_check_gate_on_lively_weights():
     assert r["tokens"] == 6 * 47 and np.isfinite(r["nll_unquantized"]) and np.isfinite(r["nll_kernel_int8"])
     assert abs(r["rel_change"]) < 2e-3, r
     assert r["top1_agree"] > 0.9 and 0 <= r["kl"] < 1e-2, r
+
+
+def test_prefill_packed_host_equals_prefill_fast():
+    """prefill_packed_host(model, prompts, rows, st, dev) (fast_decode.py:210-269) against prefill(idx, starts, st, rows) on the
+    left-padded batch: identical logits, cache bytes, scales, pos, starts and host_pos (the reference's own claim for the
+    pair, tests/test_perf_fz.py:198-236)."""
+    from ultraviolet_amd.kernels import fast_decode as fd
+    cfg, params, eng, _ = _setup(window=32)
+    m = fd.patch_model(_StubModel(cfg, params), kv_dtype="int8", dtype=torch.bfloat16, max_tokens=512)
+    prompts = _prompts(cfg, (7, 19, 12, 1), seed=8)
+    rows = [3, 0, 2, 5]
+    T = max(len(p) for p in prompts)
+    idx = torch.zeros(len(prompts), T, dtype=torch.long)
+    starts = torch.tensor([T - len(p) for p in prompts])
+    for b, p in enumerate(prompts):
+        idx[b, T - len(p):] = torch.as_tensor(p)
+    s1, s2 = m.new_state(6, 48), m.new_state(6, 48)
+    l1 = m.prefill(idx.to(DEV), starts.to(DEV), s1, rows=torch.tensor(rows, device=DEV))
+    l2 = fd.prefill_packed_host(m, prompts, rows, s2, DEV)
+    assert torch.equal(l1, l2)
+    assert torch.equal(s1.pos, s2.pos) and torch.equal(s1.starts, s2.starts) and np.array_equal(s1.host_pos, s2.host_pos)
+    for l in range(cfg.n_layers):
+        for a, b_ in ((s1.k[l], s2.k[l]), (s1.v[l], s2.v[l]), (s1.k_scale[l], s2.k_scale[l]), (s1.v_scale[l], s2.v_scale[l])):
+            assert torch.equal(a, b_)
+
+
+def test_patched_model_follows_in_place_parameter_updates():
+    """The reference's patched methods read the model's live weights; here the engine keeps fused device copies, refreshed
+    by the patched methods themselves when a parameter was written in place (same device addresses afterwards)."""
+    from ultraviolet_amd.kernels import fast_decode as fd
+    cfg, params, eng, _ = _setup(window=32)
+    m = fd.patch_model(_StubModel(cfg, params), kv_dtype="int8", dtype=torch.float32, max_tokens=256)
+    st = m.new_state(2, 48)
+    idx = torch.tensor([[5, 6, 7, 8], [9, 10, 11, 12]], device=DEV)
+    l0 = m.prefill(idx, torch.zeros(2, dtype=torch.long, device=DEV), st)
+    ptr = m._uvmi_engine.w.layers[0]["wqkv"].data_ptr()
+    m._sd["blocks.0.attn.wq"].mul_(1.05)                       # an optimizer step / sync_weights_inplace writes like this
+    st2 = m.new_state(2, 48)
+    l1 = m.prefill(idx, torch.zeros(2, dtype=torch.long, device=DEV), st2)
+    assert m._uvmi_engine.w.layers[0]["wqkv"].data_ptr() == ptr and not torch.allclose(l0, l1)
+    cfg2, params2, eng2, _ = _setup(window=32)
+    params2["blocks.0.attn.wq"] = params2["blocks.0.attn.wq"] * np.float32(1.05)
+    from ultraviolet_amd.engine import KVState, UVEngine, UVWeights
+    e3 = UVEngine(UVWeights(cfg2, params2, torch.float32, DEV), max_tokens=256)
+    ref = e3.logits(e3.prefill([[5, 6, 7, 8], [9, 10, 11, 12]], [0, 1], KVState(cfg2, 2, 48, DEV)))
+    torch.testing.assert_close(l1, ref, atol=1e-5, rtol=1e-5)
+
+
+def test_streamgen_adapter_runs_the_reference_loop():
+    """perf.make_streamgen(StreamGen, flags)(model, slots, max_prompt, max_new, T, eos) as rl_grpo.stream_loop builds it
+    (scripts/rl_grpo.py:1091-1105): every request comes back once as (meta, tokens, logp, start_version), rows are
+    EOS-terminated or max_new long (tests/test_rl_stream.py:82-94), in-place weight updates between chunks are picked up."""
+    from ultraviolet_amd import perf
+    cfg, params, eng, _ = _setup(dtype=torch.bfloat16, window=32)
+    model = _StubModel(cfg, params)
+    Gen = perf.make_streamgen(perf.StreamGen, ["lp", "hv", "rfh", "fz"])
+    g = Gen(model, 4, 24, 12, 1.0, 0, check_every=4, dtype=torch.bfloat16, row_bucket=4)
+    assert perf.install_fz(g) is True
+    prompts = _prompts(cfg, (9, 20, 4, 17, 12, 6, 3), seed=2)
+    for i, p in enumerate(prompts):
+        g.add(p, i)
+    res = []
+    for it in range(200):
+        if g.n_outstanding() == 0:
+            break
+        res += g.chunk()
+        if it == 1:
+            model._sd["blocks.0.attn.wq"].mul_(1.01)
+    res += g.harvest_end() if g.harvest_pending else []
+    assert sorted(m for m, *_ in res) == list(range(len(prompts)))
+    for meta, row, lp, v0 in res:
+        assert len(row) == len(lp) and (row[-1] == 0 or len(row) == 12) and 0 not in row[:-1]
+        assert np.isfinite(lp).all() and (lp <= 1e-6).all() and v0 in (0, 1)
+    assert g.version == 1
+
+
+def test_reference_op_name_runs_the_hip_kernels():
+    """torch.ops.mathk.decode_attn (the reference's registered op, decode_attn.py:174-190) with its argument list."""
+    from util import attn_case
+    from ultraviolet_amd.kernels import decode_attention
+    q, k, v, ks, vs = (t.to(DEV) for t in attn_case(9, 1, 8, 64, 256, True, seed=3, dtype=torch.bfloat16))
+    pos = torch.randint(0, 256, (9,), device=DEV)
+    starts = torch.zeros(9, dtype=torch.long, device=DEV)
+    a = torch.ops.mathk.decode_attn(q, k, v, pos, starts, 0.14125, 0, False, ks, vs, 2, 16, 1, "auto")
+    b_ = decode_attention(q, k, v, pos, starts, 0.14125, k_scale=ks, v_scale=vs, num_splits=2)
+    assert torch.equal(a, b_)

@@ -170,16 +170,6 @@ struct AttnState {
 // WPR waves of a workgroup share one work item (row, kv head, split): wave w takes super-tiles w, w + WPR, ... of the
 // chunk, so the workgroup streams 32 * WPR consecutive keys (2 KB * WPR of K and of V) per step, which keeps many more
 // DRAM pages open-and-hit than one wave per row does; the WPR online-softmax states are merged through LDS at the end.
-#ifdef UVMI_ATTN_TIMING
-__device__ unsigned long long g_attn_tim[1 << 15][8];
-#define UVMI_TS(k, force)                                          \
-  do {                                                             \
-    if (force) __builtin_amdgcn_s_waitcnt(0);                      \
-    tim_[k] = wall_clock64();                                      \
-  } while (0)
-#else
-#define UVMI_TS(k, force) do { } while (0)
-#endif
 
 // FUSE: the row's own token is taken from the projection output (q, k, v, gate logits) instead of from q and the cache:
 // the kernel normalises and rotates q and k, adds the value embedding to v, quantises k and v into the cache, and attends
@@ -193,10 +183,6 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
                        int a_splits, int a_kh, AttnParams P) {
   P.pos = a_pos; P.starts = a_starts; P.rows = a_rows; P.n_items = a_items; P.idx64 = a_idx64; P.splits = a_splits; P.KH = a_kh;
   if (FUSE) P.f_qkv = a_q; else P.q = a_q;
-#ifdef UVMI_ATTN_TIMING
-  unsigned long long tim_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  UVMI_TS(0, 0);
-#endif
   constexpr int IPB = 4 / WPR;  // items per block
   __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
   __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
@@ -266,7 +252,6 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   const int s0 = rp.a0 + sid * rp.chunk;
   const int s1 = live ? min(s0 + rp.chunk, rp.p + 1) : s0;
   const int lo_eff = max(rp.lo, s0);
-  UVMI_TS(1, 0);
 
   // ---- Q^T operands: lane (n, g) holds q[head][16g + 8s + j] as fp16 (bf16 inputs are converted; exact for
   // 2^-14 <= |q| <= 65504).  The K operand carries a +1152 bias, cancelled by starting the accumulator at
@@ -612,8 +597,6 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       step(TT, tb, true);
     }
   }
-
-  UVMI_TS(2, 0);
   // ---- reduce l and sum P' over the 4 lane groups, merge stream B into stream A (lanes n and n^8), undo the bias
   float lsum = xsum32(xsum16(st.lrun)), ps = xsum32(xsum16(st.psum));
   const float m2 = st.mrun == -INFINITY ? -INFINITY : st.mrun * c;  // exp2 domain
@@ -641,7 +624,6 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       if (g == 0) { sh_ml[wave][head][0] = mm; sh_ml[wave][head][1] = lm; }
     }
     __syncthreads();
-    UVMI_TS(3, 0);
     if (wsub != 0 || !live) return;
     if (strm == 0) {
       float mw[WPR];
@@ -694,7 +676,6 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
           vv[4 * i] = dead ? 0.f : x.x; vv[4 * i + 1] = dead ? 0.f : x.y; vv[4 * i + 2] = dead ? 0.f : x.z; vv[4 * i + 3] = dead ? 0.f : x.w;
         }
         const float gate = dead ? 0.f : (FUSE || P.post_gate ? sh_post[wave][64 + head] : 1.0f);
-        UVMI_TS(4, 1);
         float proj = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -753,13 +734,6 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       }
     }
   }
-#ifdef UVMI_ATTN_TIMING
-  UVMI_TS(5, 0);
-  if (lane == 0 && item < (1 << 15)) {
-    for (int k = 0; k < 6; k++) g_attn_tim[item][k] = tim_[k];
-    g_attn_tim[item][6] = (unsigned long long)(s1 - s0);
-  }
-#endif
 }
 
 // ------------------------------------------------------------------------------------------------- generic kernel
@@ -987,12 +961,6 @@ extern "C" int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus) {
   if (s < 1) s = 1;
   return (int)s;
 }
-
-#ifdef UVMI_ATTN_TIMING
-extern "C" int uvmi_debug_attn_timing(void* host_dst, size_t bytes) {
-  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(g_attn_tim), bytes, 0, hipMemcpyDeviceToHost);
-}
-#endif
 
 extern "C" int uvmi_decode_attn_path(const uvmi_attn_args* a) {
   int rc = check_common(a);

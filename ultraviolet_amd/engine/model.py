@@ -10,7 +10,6 @@ model.py:1099-1100)."""
 from __future__ import annotations
 
 import ctypes as C
-import os
 
 import numpy as np
 import torch
@@ -89,8 +88,12 @@ def rms_norm_eps(dtype: torch.dtype) -> float:
 
 
 class UVEngine:
-    def __init__(self, weights: UVWeights, max_tokens: int):
-        """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens)."""
+    def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 2048, fold_o_rows: int = 1024,
+                 lean: bool = True, fold: bool = True):
+        """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens).
+        skinny_rows, fold_qkv_rows, fold_o_rows: row counts up to which a decode pass runs its projections on the skinny
+        GEMM (see below); lean / fold: the launch plans that drop the residual-add and norm launches (off: the general
+        path).  The defaults are the measured optimum on UV-50M; tests force the other plans through them."""
         self.w, self.cfg = weights, weights.cfg
         cfg, dt, dev = self.cfg, weights.dtype, weights.device
         assert cfg.head_dim == 64, "the fused kernels are written for head_dim 64"
@@ -110,11 +113,12 @@ class UVEngine:
         # Passes of at most this many rows run their K = d_model projections on the skinny GEMM (the MLP's SwiGLU in its
         # epilogue); above it, and for the down projection, the library GEMM is faster.  Measured on UV-50M decode steps:
         # 0.544 -> 0.476 ms at 128 rows, 0.551 -> 0.523 at 256, 0.606 -> 0.589 at 384, slower from 512 on.
-        self.skinny_rows = int(os.environ.get("UVMI_SKINNY_ROWS", "384")) if dt in (torch.bfloat16, torch.float16) else 0
+        self.skinny_rows = int(skinny_rows) if dt in (torch.bfloat16, torch.float16) else 0
         # above skinny_rows the skinny kernel still carries the QKV projection (with the pre-norm) and the output projection
         # (with the residual update) up to these many rows
-        self.fold_qkv_rows = int(os.environ.get("UVMI_FOLD_QKV_ROWS", "2048"))
-        self.fold_o_rows = int(os.environ.get("UVMI_FOLD_O_ROWS", "1024"))
+        self.fold_qkv_rows = int(fold_qkv_rows)
+        self.fold_o_rows = int(fold_o_rows)
+        self.lean, self.fold = bool(lean), bool(fold)
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -310,18 +314,18 @@ class UVEngine:
         # Small passes whose every layer takes the fused attention never need the normalised hidden in memory: the block's
         # second residual update then rides on the down projection and the next block's pre-norm on its QKV projection (a row
         # scale of the product), and only the final norm is a launch of its own.
-        lean = (skinny and fused_attn is not None and os.environ.get("UVMI_LEAN", "1") != "0"
+        lean = (skinny and fused_attn is not None and self.lean
                 and all("gu_il" in W and self.fused_layer_ok(l, st) for l, W in enumerate(self.w.layers))
                 and cfg.d_ff % 64 == 0 and cfg.d_ff <= 1984)
         # Larger passes under the same condition keep the library GEMMs but still never add a launch for a residual update or
         # for the MLP's pre-norm: both residual updates are the library's own C = alpha A B + beta C on the hidden in place,
         # and the pre-norm is a row scale inside the SwiGLU launch (7 launches per layer where the general path has 8; 6 while
         # the QKV projection with the pre-norm in it is still faster on the skinny kernel).
-        folded = (not skinny and fused_attn is not None and os.environ.get("UVMI_FOLD", "1") != "0" and self.dtype != torch.float32
+        folded = (not skinny and fused_attn is not None and self.fold and self.dtype != torch.float32
                   and all(self.fused_layer_ok(l, st) for l in range(cfg.n_layers)) and cfg.d_ff % 8 == 0)
         if folded:
             return self._trunk_folded(n, fused_attn)
-        fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and os.environ.get("UVMI_FOLD", "1") != "0"
+        fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and self.fold
         x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):

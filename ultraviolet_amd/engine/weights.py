@@ -7,7 +7,7 @@ import math
 import numpy as np
 import torch
 
-from .config import UVConfig
+from .config import UVConfig, as_uvconfig
 
 
 def random_params(cfg: UVConfig, seed: int = 0, perturb: float = 0.02, lively: bool = True) -> dict[str, np.ndarray]:
@@ -152,10 +152,9 @@ class UVWeights:
 
     @classmethod
     def from_checkpoint(cls, ckpt: dict, dtype=torch.bfloat16, device="cuda") -> "UVWeights":
-        """ckpt = {"model": state_dict, "cfg": dict} as the reference saves it (README.md:26-28)."""
-        fields = UVConfig.__dataclass_fields__
-        cfg = UVConfig(**{k: v for k, v in ckpt["cfg"].items() if k in fields})
-        return cls(cfg, ckpt["model"], dtype, device)
+        """ckpt = {"model": state_dict, "cfg": dict} as the reference saves it (README.md:26-28).  Raises ValueError for a
+        configuration with layers this engine does not implement (as_uvconfig)."""
+        return cls(as_uvconfig(ckpt["cfg"]), ckpt["model"], dtype, device)
 
     def nbytes(self) -> int:
         n = self.embed.numel() * self.embed.element_size()

@@ -122,6 +122,28 @@ def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, n
     return torch.empty(q.shape, device=q.device, dtype=torch.float32 if out_fp32 else q.dtype)
 
 
+def _register_reference_op():
+    """The reference registers its op as mathk::decode_attn (ultraviolet/kernels/decode_attn.py:174-190); code that calls
+    torch.ops.mathk.decode_attn directly finds the HIP path under the same name and signature (block_n, num_warps and
+    backend are accepted and ignored).  Skipped when the name is already taken (the reference imported in the same process)."""
+    try:
+        @torch.library.custom_op("mathk::decode_attn", mutates_args=())
+        def op(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float, window: int, ring: bool,
+               k_scale: Tensor | None, v_scale: Tensor | None, num_splits: int, block_n: int, num_warps: int, backend: str) -> Tensor:
+            out = torch.empty(q.shape, device=q.device, dtype=q.dtype)
+            return _launch(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, out)
+
+        @op.register_fake
+        def _(q, k_cache, v_cache, pos, starts, scale, window, ring, k_scale, v_scale, num_splits, block_n, num_warps, backend):
+            return torch.empty_like(q)
+        return op
+    except RuntimeError:
+        return None
+
+
+_reference_op = _register_reference_op()
+
+
 def decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tensor, starts: Tensor, scale: float, *,
                      window: int = 0, ring: bool | None = None, k_scale: Tensor | None = None,
                      v_scale: Tensor | None = None, ctx_hint: int | None = None, num_splits: int | None = None,

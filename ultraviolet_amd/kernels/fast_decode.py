@@ -7,7 +7,6 @@ instance exactly as the reference's patch_model does (fast_decode.py:341-364); t
 kv_dtype "int8" (the fast path) or "fp16" (unquantized, in the engine's 16-bit dtype); attention-only presets (uv-50m-alpha) only."""
 from __future__ import annotations
 
-import dataclasses
 import types
 
 import numpy as np
@@ -16,27 +15,18 @@ from torch import Tensor
 
 from .. import _lib as L
 from ..engine.config import UVConfig
+from ..engine.config import as_uvconfig as _as_uvconfig
 from ..engine.model import KVState, UVEngine
 from ..engine.model import kv_bytes_per_seq as _kv_bytes
 from ..engine.weights import UVWeights
 
 
 def as_uvconfig(cfg) -> UVConfig:
-    """UVConfig from a UVConfig, a dict, a dataclass or any object carrying the reference's MathConfig field names."""
-    if isinstance(cfg, UVConfig):
-        return cfg
-    if isinstance(cfg, dict):
-        d = cfg
-    elif dataclasses.is_dataclass(cfg):
-        d = dataclasses.asdict(cfg)
-    else:
-        d = {k: getattr(cfg, k) for k in UVConfig.__dataclass_fields__ if hasattr(cfg, k)}
-    for name in ("mudd", "bigram_rows", "conv_layers"):
-        if d.get(name):
-            raise L.UvmiError(f"this engine covers the attention-only presets; cfg.{name} is set")
-    if d.get("local_mixer", "attn") != "attn":
-        raise L.UvmiError(f"this engine covers the attention-only presets; cfg.local_mixer is {d['local_mixer']!r}")
-    return UVConfig(**{k: v for k, v in d.items() if k in UVConfig.__dataclass_fields__})
+    """engine.config.as_uvconfig with this module's error type."""
+    try:
+        return _as_uvconfig(cfg)
+    except ValueError as e:
+        raise L.UvmiError(str(e)) from None
 
 
 class KernelDecodeState(KVState):
@@ -49,7 +39,6 @@ class KernelDecodeState(KVState):
             raise L.UvmiError(f"kv_dtype {kv_dtype!r}: the KV layouts are 'int8' and 'fp16' (unquantized, in the compute dtype)")
         super().__init__(as_uvconfig(cfg), B, max_len, device, kv_dtype=kv_dtype, dtype=dtype)
         self.dtype = dtype
-        self.local_len = min(self.cfg.window, self.max_len)
         self.host_pos = np.zeros(B, dtype=np.int64)
 
 
@@ -62,10 +51,22 @@ def kv_bytes_per_seq(cfg, ctx: int, kv_dtype: str = "int8") -> int:
     return sum(2 * c.n_kv_heads * 2 * c.head_dim * (ctx if c.is_global(l) else min(ctx, c.window)) for l in range(c.n_layers))
 
 
+def _weights_stamp(model) -> tuple:
+    """Changes whenever a parameter of the model was written in place or replaced (torch bumps a tensor's version counter
+    on every in-place write - optimizer steps, copy_, sync_weights_inplace of scripts/rl_stream.py:22-36)."""
+    return tuple((id(t), t._version) for t in model.state_dict().values())
+
+
 def _engine(model) -> UVEngine:
+    """The engine bound to a patched model, with its fused device weights brought up to date first: the reference's patched
+    methods read the model's live fused weights (fast_decode.py:296-311), so a caller that updates the parameters in place
+    expects the next prefill / decode step to use them."""
     eng = model.__dict__.get("_uvmi_engine")
     if eng is None:
         raise L.UvmiError("model has not been patched: call patch_model(model) first")
+    stamp = _weights_stamp(model)
+    if stamp != model.__dict__.get("_uvmi_stamp"):
+        sync_patched_weights(model)
     return eng
 
 
@@ -92,6 +93,23 @@ def prefill_fast(self, idx: Tensor, starts: Tensor, st: KVState, rows: Tensor | 
 
 
 @torch.no_grad()
+def prefill_packed_host(self, prompts, rows, st: KVState, dev=None) -> Tensor:
+    """prompts (lists of token ids) prefilled into cache rows `rows` with every index table built on the host from the
+    prompt lengths - the reference's perf flag 'rfh' (fast_decode.py:210-269), which StreamGen's _refill_host calls
+    (ultraviolet/perf.py:620-648).  Left-padded positions (token j of a prompt of length n at T - n + j, T the longest
+    prompt of the call), so cache slots, st.pos / starts / host_pos and the returned logits of each prompt's last token
+    equal prefill_fast's on the left-padded batch.  `dev` is accepted for the reference's signature."""
+    eng = _engine(self)
+    rows_l = [int(r) for r in rows]
+    T = max(len(p) for p in prompts)
+    assert T <= st.max_len
+    h = eng.prefill([list(p) for p in prompts], rows_l, st, left_pad=True)
+    if hasattr(st, "host_pos"):
+        st.host_pos[np.asarray(rows_l)] = T
+    return eng.logits(h)
+
+
+@torch.no_grad()
 def decode_step_fast(self, tok: Tensor, st: KVState, g_len: int = 0, skip_attn: bool = False, num_splits: dict | None = None,
                      backend: str = "auto", return_hidden: bool = False) -> Tensor:
     """One token for all rows at st.pos, then st.pos += 1 (fast_decode.py:272-334).  g_len is accepted and ignored: the
@@ -106,7 +124,7 @@ def decode_step_fast(self, tok: Tensor, st: KVState, g_len: int = 0, skip_attn: 
     return h if return_hidden else eng.logits(h)
 
 
-def patch_model(model, kv_dtype: str = "int8", num_splits: dict | None = None, backend: str = "auto",
+def patch_model(model, kv_dtype: str = "fp16", num_splits: dict | None = None, backend: str = "auto",
                 dtype: torch.dtype = torch.bfloat16, max_tokens: int = 16384, device=None):
     """Bind the kernel decode path onto `model` (instance attributes only).  model.cfg and model.state_dict() must use
     the reference's names.  dtype: activation / weight dtype of the engine; max_tokens: largest number of token rows of
@@ -130,6 +148,7 @@ def patch_model(model, kv_dtype: str = "int8", num_splits: dict | None = None, b
         return decode_step_fast(self, tok, st, g_len, skip_attn, num_splits, backend)
 
     model.__dict__["_uvmi_engine"] = eng
+    model.__dict__["_uvmi_stamp"] = _weights_stamp(model)
     model.__dict__["new_state"] = types.MethodType(new_state, model)
     model.__dict__["prefill"] = types.MethodType(prefill_fast, model)
     model.__dict__["decode_step"] = types.MethodType(decode_step, model)
@@ -137,12 +156,18 @@ def patch_model(model, kv_dtype: str = "int8", num_splits: dict | None = None, b
 
 
 def unpatch_model(model):
-    for n in ("new_state", "prefill", "decode_step", "_uvmi_engine"):
+    for n in ("new_state", "prefill", "decode_step", "_uvmi_engine", "_uvmi_stamp"):
         model.__dict__.pop(n, None)
     return model
 
 
 @torch.no_grad()
 def sync_patched_weights(model) -> None:
-    """After model's parameters changed: refresh the engine's fused tensors in place from model.state_dict()."""
-    _engine(model).w.load_(model.state_dict())
+    """Refresh the engine's fused tensors in place from model.state_dict() (device addresses are kept, so captured graphs
+    stay valid).  Called by the patched methods themselves when a parameter's version counter moved; call it by hand
+    after replacing parameter storage in a way torch does not version (e.g. through .data of a view)."""
+    eng = model.__dict__.get("_uvmi_engine")
+    if eng is None:
+        raise L.UvmiError("model has not been patched: call patch_model(model) first")
+    eng.w.load_(model.state_dict())
+    model.__dict__["_uvmi_stamp"] = _weights_stamp(model)

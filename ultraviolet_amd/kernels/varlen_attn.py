@@ -126,3 +126,50 @@ def varlen_attention(q: Tensor, k: Tensor, v: Tensor, cu_seqlens: Tensor, max_se
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
         return _PackedAttention.apply(q[0], k[0], v[0], cu_seqlens, float(scale), int(window or 0))[None]
     return packed_attention(q[0], k[0], v[0], cu_seqlens, scale, window)[None]
+
+
+def _register_reference_ops():
+    """mathk::varlen_attn_fwd / mathk::varlen_attn_bwd with the reference's signatures (ultraviolet/kernels/varlen_attn.py:38-84)
+    for code that calls the ops directly: q (1, N, H, hd), k / v (1, N, K, hd).  The forward's logsumexp / seed / offset
+    outputs exist for the signature only (this backward recomputes the row statistics): they are empty tensors.  Skipped
+    when the names are already taken."""
+    try:
+        @torch.library.custom_op("mathk::varlen_attn_fwd", mutates_args=())
+        def fwd(q: Tensor, k: Tensor, v: Tensor, cu: Tensor, max_seqlen: int, window: int, scale: float) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+            o = packed_attention(q[0], k[0], v[0], cu, scale, window)[None]
+            e = lambda dt: torch.empty(0, dtype=dt, device=q.device)
+            return o, e(torch.float32), e(torch.int64), e(torch.int64)
+
+        @fwd.register_fake
+        def _(q, k, v, cu, max_seqlen, window, scale):
+            e = lambda dt: torch.empty(0, dtype=dt, device=q.device)
+            return torch.empty_like(q), e(torch.float32), e(torch.int64), e(torch.int64)
+
+        @torch.library.custom_op("mathk::varlen_attn_bwd", mutates_args=())
+        def bwd(go: Tensor, q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor, cu: Tensor, seed: Tensor, off: Tensor,
+                max_seqlen: int, window: int, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+            dq, dk, dv = packed_attention_backward(go[0], q[0], k[0], v[0], o[0], cu, scale, window)
+            return dq[None], dk[None], dv[None]
+
+        @bwd.register_fake
+        def _(go, q, k, v, o, lse, cu, seed, off, max_seqlen, window, scale):
+            return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+        def setup(ctx, inputs, output):
+            q, k, v, cu, max_seqlen, window, scale = inputs
+            o, lse, seed, off = output
+            ctx.save_for_backward(q, k, v, o, lse, cu, seed, off)
+            ctx.ms, ctx.window, ctx.scale = max_seqlen, window, scale
+
+        def backward(ctx, go, glse, gseed, goff):
+            q, k, v, o, lse, cu, seed, off = ctx.saved_tensors
+            dq, dk, dv = bwd(go, q, k, v, o, lse, cu, seed, off, ctx.ms, ctx.window, ctx.scale)
+            return dq, dk, dv, None, None, None, None
+
+        fwd.register_autograd(backward, setup_context=setup)
+        return fwd, bwd
+    except RuntimeError:
+        return None
+
+
+_reference_ops = _register_reference_ops()
