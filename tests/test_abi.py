@@ -191,3 +191,25 @@ def test_checkpoint_with_unsupported_layers_is_refused():
     with pytest.raises(ValueError):
         as_uvconfig(types.SimpleNamespace(**base, mudd=True))
     assert as_uvconfig(dict(base, mudd=False, local_mixer="attn")).d_model == base["d_model"]
+
+
+def test_integration_doc_stub_matches_the_binding():
+    """The maintainer's stub printed in INTEGRATION.md is executed as far as its declarations go (ctypes.CDLL replaced by
+    the loaded library) and compared with ultraviolet_amd/_lib.py: same dtype codes, same structure, same layout."""
+    import torch
+    from ultraviolet_amd import _lib
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = doc[doc.index("```python\nimport ctypes as C, torch"):]
+    block = block[len("```python\n"):block.index("\n```")]
+    block = block.replace('C.CDLL("libuvmi.so")', "LIB")
+    ns = {"LIB": _lib.lib()}
+    exec(compile(block, "INTEGRATION.md", "exec"), ns)
+    assert ns["_DT"] == {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32, torch.int8: _lib.I8,
+                         torch.int32: _lib.I32, torch.int64: _lib.I64}
+    assert ns["AttnArgs"]._fields_ == _lib.AttnArgs._fields_
+    assert C.sizeof(ns["AttnArgs"]) == C.sizeof(_lib.AttnArgs)
+    a = ns["_args"](torch.zeros(2, 8, 64, dtype=torch.bfloat16), torch.zeros(2, 1, 32, 64, dtype=torch.int8), torch.zeros(2, 1, 32, 64, dtype=torch.int8),
+                    torch.zeros(2, dtype=torch.long), torch.zeros(2, dtype=torch.long), 0.125, 0, False,
+                    torch.zeros(2, 1, 32, dtype=torch.float16), torch.zeros(2, 1, 32, dtype=torch.float16), 1, torch.zeros(2, 8, 64), None)
+    assert (a.B, a.H, a.KH, a.S, a.hd, a.q_dtype, a.kv_dtype, a.out_dtype, a.idx_dtype) == (2, 8, 1, 32, 64, 1, 3, 2, 5)
+    assert _lib.lib().uvmi_decode_attn_path(C.byref(a)) == 1    # CPU pointers are never dereferenced by the path predicate
