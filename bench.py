@@ -9,8 +9,10 @@ Philox sampling, per-sequence stop length min(Geom(1/600), 2048), random-init (p
 KV cache.  All prompts are prefilled (untimed, reported separately), W decode steps run untimed, then exactly K decode
 steps of the rollout are timed; a step is 10-layer trunk over the active rows -> tied head -> fused sampler -> commit,
 replayed from a captured graph (the active rows are compacted again when the bucket shrinks), with the inputs resident
-in HBM.  value = tokens generated in the timed steps /
-seconds.
+in HBM.  value = tokens generated in the timed steps / seconds.  With --steps K the timed window is decode steps
+W .. W + K of the rollout (right after admission: nearly all 2048 slots live, the shortest contexts); the same rollout
+is then run to completion and its whole-run figures are reported beside it as "full_rollout" (with --steps 0, the default,
+the timed region is the whole rollout itself).
 
 After the timed region the same rollout is replayed eagerly and, on a subsample of steps, the step's decode-attention
 launches are re-issued through the C ABI between HIP events on the launch stream to get the attention kernel's average
@@ -124,25 +126,43 @@ def bench_c5(args):
     tok1 = int(g.slot_cnt[g.slot_req >= 0].sum()) + g.n_tokens
     gen = tok1 - tok0
     value = gen / dt
+    active1 = g.n_active()
+    # ---- the rest of the same rollout, to completion: the whole-run figure next to the timed window's
+    rest = total_steps - W - K
+    dt_rest = 0.0
+    if rest > 0:
+        t0 = time.perf_counter()
+        run_steps(g, rest)
+        torch.cuda.synchronize()
+        dt_rest = time.perf_counter() - t0
+    tok2 = int(g.slot_cnt[g.slot_req >= 0].sum()) + g.n_tokens
+    steps_all, dt_all = K + rest, dt + dt_rest
 
     # ---- roofline of the dominant kernel: replay the same steps eagerly with events around the attention calls
-    roof = roofline_c5(make_rollout, eng, cfg, W, K)
+    roof, roof_full = roofline_c5(make_rollout, eng, cfg, W, K, total_steps - W)
     cpu = cpu_baseline_c5(cfg, prompts, limits)
+    full = {"tok_per_s": round((tok2 - tok0) / dt_all, 1), "steps": steps_all, "ms_per_step": round(dt_all * 1e3 / steps_all, 4),
+            "mean_active_rows": round((tok2 - tok0) / steps_all, 1), "tokens": tok2 - tok0, "active_at_end": g.n_active(),
+            "roofline_frac": roof_full["frac"], "roofline_achieved_GBs": roof_full["achieved"],
+            "attention_avg_launch_us": roof_full["avg_launch_us"], "attention_bytes_per_launch": roof_full["bytes_per_launch"]}
     out = {
         "metric": "decode tok/s, UV-50M ragged batch 2048", "value": round(value, 1), "unit": "tok/s", "n_gpus": 1,
         "steps": K, "warmup": W, "ms_per_step": round(dt * 1e3 / K, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C5 GRPO rollout: 256 prompts x 8 = 2048 sequences, prompts U{64..256}, T=1.0 Philox seed 0, "
                                "stop min(Geom(1/600), 2048), UV-50M (10L d640 8x64 MQA, vocab 32768) bf16, int8 KV",
-                   "slots": n_seq, "active_at_start": active0, "active_at_end": g.n_active(), "tokens_timed": gen,
+                   "timed_window": f"decode steps {W}..{W + K} of {total_steps} (whole rollout)" if rest <= 0 else
+                                   f"decode steps {W}..{W + K} of {total_steps}: the steps right after admission, all slots live, shortest "
+                                   f"contexts; the whole rollout is in full_rollout",
+                   "slots": n_seq, "active_at_start": active0, "active_at_end": active1, "tokens_timed": gen,
                    "prefill_tokens": prefill_tokens, "prefill_tokens_computed": prefill_unique, "prefill_s": round(prefill_s, 3),
                    "prefill_tok_per_s": round(prefill_unique / prefill_s, 1), "kv_cache_GB": round(g.st.nbytes() / 1e9, 3)},
-        "roofline": roof, "cpu_baseline": cpu,
+        "roofline": roof, "cpu_baseline": cpu, "full_rollout": full,
     }
     print(json.dumps(out))
 
 
-def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
+def roofline_c5(make_rollout, eng, cfg, W, K, K_all, every=16, reps=3):
     """Average launch duration and algorithmic bytes of the decode-attention kernel over the timed steps, by HIP events
     on the launch stream.  The same rollout is replayed eagerly; after every `every`-th timed step the step's ten
     attention launches are re-issued through the C ABI on that step's state, `reps` times back to back, between two
@@ -150,7 +170,9 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
     (~0.5 GB) exceeds the 256 MB last-level cache, so every launch streams from HBM as in the real step; re-issuing a
     single launch in a loop would be served from that cache.  Global-layer time = (A - B) / 2 per step.  The launches go
     through ctypes directly (a few microseconds each), so the host stays ahead of the GPU, and a fill kernel ahead of the
-    first event keeps the queue non-empty while the sequence is enqueued."""
+    first event keeps the queue non-empty while the sequence is enqueued.
+    Returns two roofline objects: over the samples of the timed window (steps W .. W + K) and over the samples of the
+    whole rollout (steps W .. W + K_all)."""
     import ctypes as C
     from ultraviolet_amd import _lib as L
     lib = L.lib()
@@ -179,7 +201,8 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
         e1.record()
         return e0, e1
 
-    for s in range(W + K):
+    in_window = []
+    for s in range(W + K_all):
         sampled = s >= W and (s - W) % every == 0
         if sampled:   # the step's own rows, tokens and positions (the step leaves the next step's in their place)
             n, act, tok, pos, starts = (t if isinstance(t, int) else t.clone() for t in g.step_inputs())
@@ -200,40 +223,47 @@ def roofline_c5(make_rollout, eng, cfg, W, K, every=16, reps=3):
             live = act.cpu().numpy() >= 0
             p, st = pos.cpu().numpy()[live], starts.cpu().numpy()[live]   # what the kernels saw (padding rows: no keys)
             samples.append((evA, evB, _attn_bytes(p, st, 0, n), _attn_bytes(p, st, cfg.window, n)))
+            in_window.append(s < W + K)
             del built
         if (s + 1) % g.ce == 0:
             g.poll()
     eng.qkvx_keep = None
-    tA = sum(a.elapsed_time(b) for (a, b), _, _, _ in samples) * 1e3 / reps      # us, all layers, summed over samples
-    tB = sum(a.elapsed_time(b) for _, (a, b), _, _ in samples) * 1e3 / reps      # us, ring layers only
-    ns = len(samples)
-    n_all = len(layers)
-    glob_us = (tA - tB) / (n_glob * ns)
-    ring_us = tB / (len(ring_layers) * ns)
-    all_us = tA / (n_all * ns)
-    glob_bytes = sum(x[2] for x in samples) / ns
-    ring_bytes = sum(x[3] for x in samples) / ns
-    all_bytes = (n_glob * glob_bytes + len(ring_layers) * ring_bytes) / n_all
-    gb, rb, ab = glob_bytes / glob_us / 1e3, ring_bytes / ring_us / 1e3, all_bytes / all_us / 1e3
-    # The headline figure covers every decode-attention launch of the step (sequence A as timed: two global-layer and
-    # eight ring-layer launches of the same kernel); the split by layer kind (A - B, B) is reported beside it.
-    extra = {}
-    if ev_plain:
-        plain_us = sum(a.elapsed_time(b) for a, b in ev_plain) * 1e3 / reps / (n_all * ns)
-        extra["attention_only_kernel"] = {
-            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=false> (the same launches without the fused QKV post-processing, which then "
-                      "costs a separate ~10 us launch per layer)",
-            "achieved": round(all_bytes / plain_us / 1e3, 1), "frac": round(all_bytes / plain_us / 1e3 / HBM_PEAK_GBS, 4),
-            "avg_launch_us": round(plain_us, 2), "launches_timed": n_all * ns * reps}
-    return {"bound": "hbm", "achieved": round(ab, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ab / HBM_PEAK_GBS, 4),
-            "traffic": int(all_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
-            "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=true> (bf16; all ten layers' launches of a step; the kernel also does the "
-                      "row's QKV post-processing and int8 append; WPR = 2 waves per row while 4 would not fit the device in one round, else 4)",
-            "avg_launch_us": round(all_us, 2), "bytes_per_launch": int(all_bytes), "steps_sampled": ns, "launches_timed": n_all * ns * reps,
-            "global_layers": {"achieved": round(gb, 1), "frac": round(gb / HBM_PEAK_GBS, 4), "avg_launch_us": round(glob_us, 2),
-                              "bytes_per_launch": int(glob_bytes), "launches_timed": n_glob * ns * reps},
-            "ring_layers": {"achieved": round(rb, 1), "frac": round(rb / HBM_PEAK_GBS, 4), "avg_launch_us": round(ring_us, 2),
-                            "bytes_per_launch": int(ring_bytes), "launches_timed": len(ring_layers) * ns * reps}, **extra}
+
+    def aggregate(sel):
+        smp = [x for x, k in zip(samples, sel) if k]
+        evp = [x for x, k in zip(ev_plain, sel) if k] if ev_plain else []
+        tA = sum(a.elapsed_time(b) for (a, b), _, _, _ in smp) * 1e3 / reps      # us, all layers, summed over samples
+        tB = sum(a.elapsed_time(b) for _, (a, b), _, _ in smp) * 1e3 / reps      # us, ring layers only
+        ns = len(smp)
+        n_all = len(layers)
+        glob_us = (tA - tB) / (n_glob * ns)
+        ring_us = tB / (len(ring_layers) * ns)
+        all_us = tA / (n_all * ns)
+        glob_bytes = sum(x[2] for x in smp) / ns
+        ring_bytes = sum(x[3] for x in smp) / ns
+        all_bytes = (n_glob * glob_bytes + len(ring_layers) * ring_bytes) / n_all
+        gb, rb, ab = glob_bytes / glob_us / 1e3, ring_bytes / ring_us / 1e3, all_bytes / all_us / 1e3
+        # The headline figure covers every decode-attention launch of the step (sequence A as timed: two global-layer and
+        # eight ring-layer launches of the same kernel); the split by layer kind (A - B, B) is reported beside it.
+        extra = {}
+        if evp:
+            plain_us = sum(a.elapsed_time(b) for a, b in evp) * 1e3 / reps / (n_all * ns)
+            extra["attention_only_kernel"] = {
+                "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=false> (the same launches without the fused QKV post-processing, which then "
+                          "costs a separate ~10 us launch per layer)",
+                "achieved": round(all_bytes / plain_us / 1e3, 1), "frac": round(all_bytes / plain_us / 1e3 / HBM_PEAK_GBS, 4),
+                "avg_launch_us": round(plain_us, 2), "launches_timed": n_all * ns * reps}
+        return {"bound": "hbm", "achieved": round(ab, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ab / HBM_PEAK_GBS, 4),
+                "traffic": int(all_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
+                "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=true> (bf16; all ten layers' launches of a step; the kernel also does the "
+                          "row's QKV post-processing and int8 append; WPR = 2 waves per row while 4 would not fit the device in one round, else 4)",
+                "avg_launch_us": round(all_us, 2), "bytes_per_launch": int(all_bytes), "steps_sampled": ns, "launches_timed": n_all * ns * reps,
+                "global_layers": {"achieved": round(gb, 1), "frac": round(gb / HBM_PEAK_GBS, 4), "avg_launch_us": round(glob_us, 2),
+                                  "bytes_per_launch": int(glob_bytes), "launches_timed": n_glob * ns * reps},
+                "ring_layers": {"achieved": round(rb, 1), "frac": round(rb / HBM_PEAK_GBS, 4), "avg_launch_us": round(ring_us, 2),
+                                "bytes_per_launch": int(ring_bytes), "launches_timed": len(ring_layers) * ns * reps}, **extra}
+
+    return aggregate(in_window), aggregate([True] * len(samples))
 
 
 def cpu_baseline_c5(cfg, prompts, limits, budget_s=15.0, rows=32):
@@ -369,22 +399,16 @@ def bench_c4(args):
                                  "prefill_attn_local_TFLOPs": round(fl_l / phases["prefill_attn_local_us"] / 1e6, 1)}}))
 
 
-def bench_c3(args):
-    """BASELINE configs[2]: 512 slots, contexts U{128..2048}, retire p = 0.01 per step, 64-token prompts admitted into freed
-    slots inside decode passes; 256 steps."""
-    from ultraviolet_amd.engine import UVEngine, UVWeights, make_config
+def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0):
+    """The C3 workload as a Rollout ready to step: B running slots whose contexts U{128..2048} are materialised in the cache
+    (request ids 0..B-1, one token generated so far), Bernoulli(0.01) retirement per slot and step on the device, and a
+    queue of 64-token prompts (ids B, B + 1, ..) long enough for n_steps steps, admitted inside decode passes."""
     from ultraviolet_amd.engine.rollout import Rollout
-    dev = "cuda:0"
-    cfg = make_config("uv-50m-alpha")
-    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02), max_tokens=2048)
-    rng = np.random.default_rng(0)
-    gen = torch.Generator(device=dev).manual_seed(0)
-    B = 512
-    K = args.steps if args.steps > 0 else 256
-    W = args.warmup
-    g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + K + W + 64, temperature=1.0, seed=0, eos_id=None, check_every=4, bucket=128,
-                retire_p=0.01, mixed=True, admit_cap=24, overlap_harvest=True)
-    # running slots with materialised contexts: request ids 0..B-1, one token generated so far
+    dev = eng.device
+    rng = np.random.default_rng(seed)
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + n_steps + 64, temperature=1.0, seed=seed, eos_id=None, check_every=4, bucket=128,
+                retire_p=0.01, mixed=True, admit_cap=24, overlap_harvest=True, use_graph=use_graph)
     rows = torch.arange(B, device=dev)
     _fill_cache(g.st, rows, torch.from_numpy(rng.integers(128, 2049, size=B)).to(dev), gen)
     g.slot_req.copy_(rows)
@@ -394,8 +418,23 @@ def bench_c3(args):
     g.free, g.next_req, g.n_active_host = [], B, B
     for r in range(B):
         g.meta[r] = (r, 0)
-    for i in range(int((W + K) * B * 0.01 * 2) + 64):
+    for i in range(int(n_steps * B * 0.01 * 2) + 64):
         g.add(rng.integers(1, cfg.vocab_size, size=64).tolist(), B + i)
+    return g
+
+
+def bench_c3(args):
+    """BASELINE configs[2]: 512 slots, contexts U{128..2048}, retire p = 0.01 per step, 64-token prompts admitted into freed
+    slots inside decode passes; 256 steps."""
+    from ultraviolet_amd.engine import UVEngine, UVWeights, make_config
+    from ultraviolet_amd.engine.rollout import Rollout
+    dev = "cuda:0"
+    cfg = make_config("uv-50m-alpha")
+    eng = UVEngine(UVWeights.random(cfg, seed=0, dtype=torch.bfloat16, device=dev, perturb=0.02), max_tokens=2048)
+    B = 512
+    K = args.steps if args.steps > 0 else 256
+    W = args.warmup
+    g = c3_rollout(eng, cfg, B, W + K)
     g.precapture()
 
     def run(n):
