@@ -169,12 +169,15 @@ int uvmi_decode_attn_path(const uvmi_attn_args* a);
 int uvmi_decode_attn_noalloc(const uvmi_attn_args* a, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------
- * Skinny 16-bit GEMM of a small decode step's projections: C (M, N) = A (M, K) . W (N, K)^T, fp32 accumulation, A, W, C
- * in `dtype` (F16 / BF16), rows contiguous with pitches lda, ldw, ldc (elements).  Replaces the F.linear calls of the
- * reference's fused inference path (ultraviolet/model.py:302-335 attention projections, 388-391 MLP) when M is a few
- * hundred rows: the weights are then the traffic, and the kernel requests a workgroup's whole weight strip and its
- * activation rows in one burst.  K % 64 == 0, K <= 1984; N % 16 == 0.
- * epilogue UVMI_GEMM_SWIGLU (K <= 960, N % 32 == 0): W holds w_gate and w_up interleaved in slabs of 16 rows ([gate 0..15 |
+ * 16-bit GEMM of a decode step's projections: C (M, N) = A (M, K) . W (N, K)^T, fp32 accumulation, A, W, C in `dtype`
+ * (F16 / BF16), rows contiguous with pitches lda, ldw, ldc (elements).  Replaces the F.linear calls of the reference's
+ * fused inference path (ultraviolet/model.py:302-335 attention projections, 388-391 MLP).  K % 64 == 0, K <= 8192;
+ * N % 16 == 0.  Two kernel families behind one entry point:
+ *   - skinny forms for steps of up to a few hundred rows, where the weights are the traffic: a workgroup requests its
+ *     whole weight strip and its activation rows in one burst (K <= 1984; 960 with SWIGLU);
+ *   - a tiled form (128 x 128 or 64 x 64 tiles, operand slabs double-buffered in LDS behind a ring of slabs in flight)
+ *     for steps of several hundred to a few thousand rows, where the product is bound by feeding the matrix cores.
+ * epilogue UVMI_GEMM_SWIGLU (N % 32 == 0): W holds w_gate and w_up interleaved in slabs of 16 rows ([gate 0..15 |
  * up 0..15 | gate 16..31 | ...], N = 2 f rows) and C (M, f) = silu(A w_gate^T) * (A w_up^T) with the roundings of the
  * separate SwiGLU pass (model.py:388-391).
  * ---------------------------------------------------------------------------------------------------------- */
@@ -198,8 +201,9 @@ typedef struct uvmi_gemm_args {
   int epilogue;
   int norm_a; float eps;
   const void* resid; int64_t ldr; float ca, cb;
-  int config;                              /* 0: built-in choice of the kernel form; 1: 64-row workgroups; 2: 16-row workgroups
-                                              whose waves split K (needs K % 128 == 0, else form 1) - for tuning and tests */
+  int config;                              /* 0: built-in choice of the kernel form by size; 1: skinny, 64-row workgroups; 2: skinny,
+                                              16-row workgroups whose waves split K (needs K % 128 == 0, else form 1); 3: tiled,
+                                              128 x 128; 4: tiled, 64 x 64 - for tuning and tests */
 } uvmi_gemm_args;
 int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream);
 

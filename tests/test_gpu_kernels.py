@@ -429,7 +429,7 @@ def test_rope_table_matches_rounded_cos_sin(dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,K,N", [(1, 640, 656), (64, 640, 656), (100, 512, 640), (128, 640, 3328), (257, 1664, 640), (384, 640, 48),
-                                   (65, 64, 16), (200, 960, 96), (77, 1984, 32)])
+                                   (65, 64, 16), (200, 960, 96), (77, 1984, 32), (700, 640, 656), (1030, 2048, 208)])
 def test_skinny_gemm_matches_fp32_reference(dtype, M, K, N):
     """uvmi_gemm_tn against a float64 product of the same 16-bit inputs: the result is the fp32-accumulated product rounded
     once to the activation type (tolerance: half a unit in the last place of the largest magnitude plus the accumulation
@@ -444,7 +444,9 @@ def test_skinny_gemm_matches_fp32_reference(dtype, M, K, N):
     ref = a.double() @ w.double().t()
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     tol = ulp * ref.abs().clamp_min(1.0) + 1e-5 * K ** 0.5
-    for config in (1, 2):     # 64-row workgroups; 16-row workgroups whose waves split K (the latter when K % 128 == 0)
+    # 64-row workgroups; 16-row workgroups whose waves split K (the latter when K % 128 == 0); the tiled kernel with 128 x 128
+    # and 64 x 64 tiles (any K); the library's own choice
+    for config in ((1, 2) if K <= 1984 else ()) + (3, 4, 0):
         out_full = torch.full((M, N + 4), 7.0, device="cuda", dtype=dtype)
         out = out_full[:, :N]
         gemm_tn(a, w, out, config=config)
@@ -454,7 +456,7 @@ def test_skinny_gemm_matches_fp32_reference(dtype, M, K, N):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,K,f", [(3, 640, 1664), (128, 640, 1664), (200, 128, 48)])
+@pytest.mark.parametrize("M,K,f", [(3, 640, 1664), (128, 640, 1664), (200, 128, 48), (600, 640, 1664)])
 def test_skinny_gemm_swiglu_epilogue(dtype, M, K, f):
     """The SWIGLU epilogue on interleaved gate / up rows equals the two-pass path (GEMM to the activation type, then
     silu(g) rounded, times u - ultraviolet/model.py:388-391) up to the GEMMs' own last-place differences."""
@@ -468,7 +470,7 @@ def test_skinny_gemm_swiglu_epilogue(dtype, M, K, f):
     ref = (gg * torch.sigmoid(gg)).to(dtype).double() * uu
     ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     tol = 4 * ulp * ref.abs().clamp_min(1.0) + 4 * ulp * (gg.abs() + uu.abs())   # g and u may each sit one rounding step off
-    for config in (1, 2):
+    for config in (1, 2, 3, 4):
         out = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU, config=config)
         assert out.shape == (M, f)
         assert bool(((out.double() - ref).abs() <= tol).all()), (config, float((out.double() - ref).abs().max()))
@@ -507,11 +509,16 @@ def test_skinny_gemm_rejects_what_it_cannot_do():
     from ultraviolet_amd.kernels.gemm import SWIGLU, gemm_supported, gemm_tn
     a = torch.zeros(4, 2048, device="cuda", dtype=torch.bfloat16)
     w = torch.zeros(32, 2048, device="cuda", dtype=torch.bfloat16)
-    assert not gemm_supported(a, w)            # K above 1984
+    assert gemm_supported(a, w)                # K above 1984: the tiled kernel only
+    gemm_tn(a, w)
+    for config in (1, 2):
+        with pytest.raises(L.UvmiError):
+            gemm_tn(a, w, config=config)
     with pytest.raises(L.UvmiError):
-        gemm_tn(a, w)
-    a, w = a[:, :1024], w[:, :1024]
-    assert gemm_supported(a, w) and not gemm_supported(a, w, SWIGLU)   # the SwiGLU strip needs K <= 960
+        gemm_tn(a[:, :1000], w[:, :1000])      # K % 64 != 0
+    with pytest.raises(L.UvmiError):
+        gemm_tn(a[:, :1024], w[:, :1024], epilogue=SWIGLU, config=1)   # the skinny SwiGLU strip needs K <= 960
+    gemm_tn(a[:, :1024], w[:, :1024], epilogue=SWIGLU)
     assert not gemm_supported(a.float(), w.float())
 
 
@@ -576,7 +583,7 @@ def test_truncated_sampler_off_equals_plain_and_seeded_draw():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,K,N", [(5, 640, 656), (128, 640, 3328), (200, 512, 640), (70, 1664, 640)])
+@pytest.mark.parametrize("M,K,N", [(5, 640, 656), (128, 640, 3328), (200, 512, 640), (70, 1664, 640), (900, 640, 3328), (515, 1664, 640)])
 def test_skinny_gemm_norm_and_resid_fusions(dtype, M, K, N):
     """norm_eps: the product of the RMS-normalised rows, against float64 (rmsnorm(a) @ w.T without intermediate rounding -
     the kernel applies the norm as an exact row scale); RESID: ca * r + cb * round(a @ w.T), rounded; and both with SwiGLU."""
@@ -594,11 +601,14 @@ def test_skinny_gemm_norm_and_resid_fusions(dtype, M, K, N):
     prod = (ad @ w.double().t()).to(dtype).double()
     want = 0.75 * r.double() + 1.25 * prod
     tol2 = ulp * want.abs().clamp_min(1.0) + 1.25 * 2 * ulp * prod.abs().clamp_min(1.0)
-    for config in (1, 2):
+    for config in (1, 2, 3, 4, 0):
         out = gemm_tn(a, w, norm_eps=eps, config=config)
         assert bool(((out.double() - ref).abs() <= tol).all()), (config, float((out.double() - ref).abs().max()))
         got = gemm_tn(a, w, epilogue=RESID, resid=r, ca=0.75, cb=1.25, config=config)
         assert bool(((got.double() - want).abs() <= tol2).all()), (config, float((got.double() - want).abs().max()))
+        inplace = r.clone()       # the residual update in place (C is R), as the engine's output projection runs it
+        gemm_tn(a, w, inplace, epilogue=RESID, resid=inplace, ca=0.75, cb=1.25, config=config)
+        assert torch.equal(inplace, got)
     if K <= 960 and N % 32 == 0:
         f = N // 2
         wg, wu = w[:f].contiguous(), w[f:].contiguous()
@@ -606,6 +616,6 @@ def test_skinny_gemm_norm_and_resid_fusions(dtype, M, K, N):
         uu = (an @ wu.double().t()).to(dtype).double()
         ra = (gg * torch.sigmoid(gg)).to(dtype).double() * uu
         tol3 = 4 * ulp * ra.abs().clamp_min(1.0) + 4 * ulp * (gg.abs() + uu.abs())
-        for config in (1, 2):
+        for config in (1, 2, 3, 4, 0):
             act = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU, norm_eps=eps, config=config)
             assert bool(((act.double() - ra).abs() <= tol3).all()), (config, float((act.double() - ra).abs().max()))

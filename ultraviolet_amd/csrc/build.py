@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["common.hip", "kv_quant.hip", "decode_attn.hip", "fused_sample.hip", "sched.hip", "model_ops.hip",
-           "prefill_attn.hip", "prefill_attn_bwd.hip", "gemm.hip"]
+           "prefill_attn.hip", "prefill_attn_bwd.hip", "gemm.hip", "gemm_tile.hip"]
 LIB = os.path.join(HERE, "libuvmi.so")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
@@ -36,7 +36,7 @@ def _hipcc() -> str:
 def _stale(obj: str, src: str) -> bool:
     if not os.path.exists(obj):
         return True
-    deps = [src, os.path.join(HERE, "common.h"), os.path.join(HERE, "sched_commit.h"), os.path.join(HERE, "..", "..", "include", "uvmi.h"), __file__]
+    deps = [src, os.path.join(HERE, "common.h"), os.path.join(HERE, "sched_commit.h"), os.path.join(HERE, "gemm_util.h"), os.path.join(HERE, "..", "..", "include", "uvmi.h"), __file__]
     return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps)
 
 

@@ -29,13 +29,9 @@
 //     once at the end - the normalised activations are never written (nor rounded to the activation type: the result is
 //     the exact row scale of the un-normalised product, a rounding step closer to exact than the two-pass path).
 #include "common.h"
+#include "gemm_util.h"
 
 namespace uvmi {
-
-typedef _Float16 gh8 __attribute__((ext_vector_type(8)));
-typedef __bf16 gb8 __attribute__((ext_vector_type(8)));
-typedef float gf4 __attribute__((ext_vector_type(4)));
-typedef unsigned int gu4 __attribute__((ext_vector_type(4)));
 
 struct SkinnyParams {
   const void* a; const void* w; void* c;
@@ -44,31 +40,6 @@ struct SkinnyParams {
   int M, N, K;
   int tiles_m, tiles_n;
 };
-
-template <int DT>
-__device__ __forceinline__ gf4 gmfma(gu4 a, gu4 b, gf4 c) {
-  if constexpr (DT == UVMI_F16) {
-    gh8 x, y;
-    __builtin_memcpy(&x, &a, 16);
-    __builtin_memcpy(&y, &b, 16);
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, c, 0, 0, 0);
-  } else {
-    gb8 x, y;
-    __builtin_memcpy(&x, &a, 16);
-    __builtin_memcpy(&y, &b, 16);
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, c, 0, 0, 0);
-  }
-}
-
-template <int DT> __device__ __forceinline__ float ground(float v) {
-  if constexpr (DT == UVMI_F16) return (float)(half_t)v;
-  else return bf16_to_float(float_to_bf16(v));
-}
-template <int DT> __device__ __forceinline__ uint32_t gpack(float a, float b) {
-  const uint32_t lo = DT == UVMI_BF16 ? float_to_bf16(a) : float_to_half_bits(a);
-  const uint32_t hi = DT == UVMI_BF16 ? float_to_bf16(b) : float_to_half_bits(b);
-  return lo | (hi << 16);
-}
 
 constexpr int SK_BM = 64;       // rows per workgroup
 constexpr int SK_RING = 16;     // activation K-steps (of 32) in flight per wave
@@ -399,6 +370,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_ksplit_kernel(const void* a_a
 
 using namespace uvmi;
 
+namespace uvmi { void gemm_tile_launch(const uvmi_gemm_args* a, bool big, hipStream_t st); }  // gemm_tile.hip
+
+// Rows from which the tiled kernel takes over from the skinny forms when config == 0 (measured on UV-50M's projections).
+constexpr int64_t TILE_MIN_ROWS = 448;
+
 static int skinny_bn(int K, int epilogue) {  // widest strip that fits 64 KB of LDS: 32 rows up to K = 960, else 16
   if (epilogue == UVMI_GEMM_SWIGLU) return K <= 960 ? 32 : 0;
   if (K <= 960) return 32;
@@ -408,7 +384,7 @@ static int skinny_bn(int K, int epilogue) {  // widest strip that fits 64 KB of 
 extern "C" int uvmi_gemm_tn_supported(int dtype, int64_t M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int epilogue) {
   if (dtype != UVMI_F16 && dtype != UVMI_BF16) return 0;
   if (epilogue != UVMI_GEMM_STORE && epilogue != UVMI_GEMM_SWIGLU && epilogue != UVMI_GEMM_RESID) return 0;
-  if (M < 0 || M > (1 << 16) || N <= 0 || K <= 0 || K % 64 != 0 || skinny_bn(K, epilogue) == 0) return 0;
+  if (M < 0 || M > (1 << 16) || N <= 0 || K <= 0 || K % 64 != 0 || K > 8192) return 0;  // (the skinny forms add K <= 1984 / 960)
   if (N % (epilogue == UVMI_GEMM_SWIGLU ? 32 : 16) != 0) return 0;
   if (lda < K || ldw < K || lda % 8 != 0 || ldw % 8 != 0 || ldc % 4 != 0) return 0;
   if (ldc < (epilogue == UVMI_GEMM_SWIGLU ? N / 2 : N)) return 0;
@@ -440,15 +416,27 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
   UVMI_REQUIRE(a && a->a && a->w && a->c, UVMI_EINVAL, "uvmi_gemm_tn: null pointer");
   UVMI_REQUIRE(uvmi_gemm_tn_supported(a->dtype, a->M, a->N, a->K, a->lda, a->ldw, a->ldc, a->epilogue), UVMI_EUNSUPPORTED,
                "uvmi_gemm_tn: unsupported problem (dtype %d, M %lld, N %d, K %d, lda %lld, ldw %lld, ldc %lld, epilogue %d): needs F16 / BF16, "
-               "K %% 64 == 0, K <= 1984 (960 with SWIGLU), N %% 16 == 0 (32 with SWIGLU), lda, ldw %% 8 == 0, ldc %% 4 == 0",
+               "K %% 64 == 0, N %% 16 == 0 (32 with SWIGLU), lda, ldw %% 8 == 0, ldc %% 4 == 0",
                a->dtype, (long long)a->M, a->N, a->K, (long long)a->lda, (long long)a->ldw, (long long)a->ldc, a->epilogue);
   UVMI_REQUIRE(((uintptr_t)a->a % 16) == 0 && ((uintptr_t)a->w % 16) == 0 && ((uintptr_t)a->c % 8) == 0, UVMI_EINVAL, "uvmi_gemm_tn: misaligned pointer");
   if (a->epilogue == UVMI_GEMM_RESID)
     UVMI_REQUIRE(a->resid && ((uintptr_t)a->resid % 8) == 0 && a->ldr % 4 == 0 && a->ldr >= a->N, UVMI_EINVAL,
                  "uvmi_gemm_tn: the RESID epilogue needs an 8-byte aligned residual with a pitch that is a multiple of 4 and >= N");
   UVMI_REQUIRE(!a->norm_a || a->eps >= 0.f, UVMI_EINVAL, "uvmi_gemm_tn: negative eps");
+  UVMI_REQUIRE(a->config >= 0 && a->config <= 4, UVMI_EINVAL, "uvmi_gemm_tn: config %d", a->config);
   if (a->M == 0) return UVMI_OK;
   const int BN = skinny_bn(a->K, a->epilogue);
+  UVMI_REQUIRE(BN != 0 || a->config == 0 || a->config >= 3, UVMI_EUNSUPPORTED, "uvmi_gemm_tn: K = %d is beyond the skinny forms (config 1, 2)", a->K);
+  if (a->config >= 3 || (a->config == 0 && (BN == 0 || a->M >= TILE_MIN_ROWS))) {
+    // tiled kernel: 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64
+    int cus = uvmi_device_cus();
+    if (cus <= 0) cus = 256;
+    const int64_t t128 = ((a->M + 127) / 128) * ((a->N + 127) / 128);
+    const bool big = a->config == 3 || (a->config == 0 && 4 * t128 >= 3 * cus);
+    gemm_tile_launch(a, big, (hipStream_t)stream);
+    UVMI_CHECK_LAUNCH("uvmi_gemm_tn(tiled)");
+    return UVMI_OK;
+  }
   // the smallest problems split K over the waves of a 16-row workgroup (more, shorter workgroups); config forces a form
   const bool can_split = a->K % 128 == 0;
   const int64_t t_split = ((a->M + 15) / 16) * ((a->N + BN - 1) / BN);

@@ -88,12 +88,15 @@ def rms_norm_eps(dtype: torch.dtype) -> float:
 
 
 class UVEngine:
-    def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 2048, fold_o_rows: int = 1024,
-                 lean: bool = True, fold: bool = True):
+    def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 1 << 30, fold_o_rows: int = 1 << 30,
+                 fold_gu_rows: int = 1 << 30, lean: bool = True, fold: bool = True, gemm_config: int = 0):
         """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens).
-        skinny_rows, fold_qkv_rows, fold_o_rows: row counts up to which a decode pass runs its projections on the skinny
-        GEMM (see below); lean / fold: the launch plans that drop the residual-add and norm launches (off: the general
-        path).  The defaults are the measured optimum on UV-50M; tests force the other plans through them."""
+        skinny_rows: passes of at most this many rows run every projection on the skinny GEMM; fold_qkv_rows, fold_o_rows,
+        fold_gu_rows: above skinny_rows, row counts up to which the QKV projection (with the pre-norm), the output
+        projection (with the residual update) and the gate-up projection (with the pre-norm and the SwiGLU) run on this
+        library's GEMM kernels instead of the vendor library's (see _trunk_folded); lean / fold: the launch plans that drop
+        the residual-add and norm launches (off: the general path); gemm_config: form of the hand-written GEMM (0: its own
+        choice by size; tests force the tiled forms at a few rows).  The defaults are the measured optimum on UV-50M."""
         self.w, self.cfg = weights, weights.cfg
         cfg, dt, dev = self.cfg, weights.dtype, weights.device
         assert cfg.head_dim == 64, "the fused kernels are written for head_dim 64"
@@ -117,8 +120,8 @@ class UVEngine:
         # above skinny_rows the skinny kernel still carries the QKV projection (with the pre-norm) and the output projection
         # (with the residual update) up to these many rows
         self.fold_qkv_rows = int(fold_qkv_rows)
-        self.fold_o_rows = int(fold_o_rows)
-        self.lean, self.fold = bool(lean), bool(fold)
+        self.fold_o_rows, self.fold_gu_rows = int(fold_o_rows), int(fold_gu_rows)
+        self.lean, self.fold, self.gemm_config = bool(lean), bool(fold), int(gemm_config)
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -380,16 +383,21 @@ class UVEngine:
 
     def _trunk_folded(self, n: int, fused_attn) -> Tensor:
         """The layers of _trunk for a pass of many rows whose every layer takes the fused attention; buf x and xn hold the
-        embedded rows and their norm on entry."""
+        embedded rows and their norm on entry.  Five launches per layer: QKV projection with the block's pre-norm as a row
+        scale, fused attention, output projection with the residual update in place, gate-up projection with the MLP's
+        pre-norm and the SwiGLU in its epilogue (the tiled GEMM of this library: the (n, 2 f) intermediate and the
+        normalised hidden are never written), down projection with the residual update (the vendor library's
+        C = alpha A B + beta C: at K = d_ff it is still the faster kernel)."""
         cfg, b = self.cfg, self.buf
         x, xn = b["x"][:n], b["xn"][:n]
-        sk_ok = cfg.d_model % 64 == 0 and cfg.d_model <= 960 and (cfg.n_heads * cfg.head_dim) % 64 == 0
+        gc = self.gemm_config
+        sk_ok = cfg.d_model % 64 == 0 and (cfg.n_heads * cfg.head_dim) % 64 == 0
         sk_qkv, sk_o = sk_ok and n <= self.fold_qkv_rows, sk_ok and n <= self.fold_o_rows
         for l, W in enumerate(self.w.layers):
-            if l == 0:
+            if l == 0:      # (the embedding's norm exists already: the same product as on the general path, bit for bit)
                 torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
             elif sk_qkv:
-                gemm_tn(x, W["wqkv_ext"], b["qkvx"][:n], norm_eps=self.eps)
+                gemm_tn(x, W["wqkv_ext"], b["qkvx"][:n], norm_eps=self.eps, config=gc)
             else:
                 self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
                 torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
@@ -398,11 +406,14 @@ class UVEngine:
             fused_attn(l)
             # x <- resid_attn * x + post_attn * (zg @ wo.T), in place (every element is read and written by the same lane)
             if sk_o:
-                gemm_tn(b["zg"][:n], W["wo"], x, epilogue=RESID, resid=x, ca=W["resid_attn"], cb=W["post_attn"])
+                gemm_tn(b["zg"][:n], W["wo"], x, epilogue=RESID, resid=x, ca=W["resid_attn"], cb=W["post_attn"], config=gc)
             else:
                 torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
-            torch.mm(x, W["gu"].t(), out=b["gu"][:n])
-            self._swiglu_norm(x, n)
+            if sk_ok and "gu_il" in W and n <= self.fold_gu_rows:
+                gemm_tn(x, W["gu_il"], b["act"][:n], epilogue=SWIGLU, norm_eps=self.eps, config=gc)
+            else:
+                torch.mm(x, W["gu"].t(), out=b["gu"][:n])
+                self._swiglu_norm(x, n)
             # x <- resid_mlp * x + post_mlp * (act @ down.T)
             torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
         self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
