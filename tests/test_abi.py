@@ -159,7 +159,7 @@ def test_reference_names_are_mirrored():
     for n in ("decode_attention", "default_splits", "dequantize_kv", "kv_write", "kv_write_rows", "quantize_kv"):
         assert callable(getattr(K, n))
     assert not hasattr(K, "decode_attention_ref") and not hasattr(fused_sample, "fused_sample_ref")
-    for n in ("KernelDecodeState", "prefill_fast", "decode_step_fast", "prefill_packed_host", "patch_model", "unpatch_model"):
+    for n in ("KernelDecodeState", "DecodeState", "prefill_fast", "decode_step_fast", "prefill_packed_host", "patch_model", "unpatch_model"):
         assert hasattr(fast_decode, n)
     for n in ("fused_sample", "fused_sample_ok"):
         assert callable(getattr(fused_sample, n))

@@ -539,3 +539,43 @@ def test_reference_op_name_runs_the_hip_kernels():
     a = torch.ops.mathk.decode_attn(q, k, v, pos, starts, 0.14125, 0, False, ks, vs, 2, 16, 1, "auto")
     b_ = decode_attention(q, k, v, pos, starts, 0.14125, k_scale=ks, v_scale=vs, num_splits=2)
     assert torch.equal(a, b_)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_uncompressed_decode_state_entry_points(dtype):
+    """The reference's SDPA-path entry points (MathLM.new_state -> DecodeState, prefill, decode_step with decode_impl "sdpa":
+    ultraviolet/model.py:861-1008, 1042-1072) bound by patch_model(kv_dtype=None): the state carries the reference's fields,
+    and prefill + decode over it give the logits of the dense causal forward of the whole sequence (the oracle's trunk in
+    the same 16-bit arithmetic) - the invariant the reference pins for this path (tests/test_math_model.py:73-85) - through
+    ring wrap-around, for left-padded rows as well."""
+    from ultraviolet_amd.kernels import fast_decode as fd
+    cfg, params, eng, OracleModel = _setup("uv-test", dtype=dtype, perturb=0.06, window=32)
+    m = fd.patch_model(_StubModel(cfg, params), kv_dtype=None, dtype=dtype, max_tokens=512)
+    B, L0, steps = 4, 20, 40
+    st = m.new_state(B, 96)
+    assert isinstance(st, fd.DecodeState) and st.kv_dtype is None and st.k[0].dtype == dtype and st.k[0].shape == (B, 1, 32, 64)
+    assert st.k[cfg.n_layers - 1].shape[2] == 96 and st.local_len == 32 and st.pos.dtype == torch.long and st.host_pos.shape == (B,)
+    assert st.nbytes() == sum(t.numel() * 2 for t in st.k + st.v)
+    seqs = np.random.default_rng(4).integers(1, cfg.vocab_size, size=(B, L0 + steps))
+    om = OracleModel(cfg, params, dtype=dtype)
+    hid, _ = om.trunk(torch.as_tensor(seqs))
+    ref = om.logits(hid).float().numpy()[:, L0 - 1:-1]
+    outs = [m.prefill(torch.as_tensor(seqs[:, :L0]).to(DEV), torch.zeros(B, dtype=torch.long, device=DEV), st).cpu()]
+    for t in range(steps - 1):
+        outs.append(m.decode_step(torch.as_tensor(seqs[:, L0 + t]).to(DEV), st, 96).cpu())
+    got = torch.stack(outs, 1).float().numpy()
+    assert st.pos.tolist() == [L0 + steps - 1] * B and st.host_pos.tolist() == [L0 + steps - 1] * B
+    d = np.abs(got - ref)
+    assert d.max() < (0.15 if dtype == torch.bfloat16 else 0.04) and (got.argmax(-1) == ref.argmax(-1)).mean() > 0.97, d.max()
+    # a left-padded refill of two rows (rows=...) leaves the other rows' caches and positions alone
+    st.set_pos(7)
+    assert st.pos.tolist() == [7] * B and st.host_pos.tolist() == [7] * B
+    k_before = st.k[0][[0, 3]].clone()
+    idx = torch.zeros(2, 9, dtype=torch.long)
+    idx[0, 4:], idx[1, :] = torch.as_tensor(seqs[0, :5]), torch.as_tensor(seqs[1, :9])
+    lg = m.prefill(idx.to(DEV), torch.tensor([4, 0], device=DEV), st, rows=torch.tensor([1, 2], device=DEV))
+    assert st.pos.tolist() == [7, 9, 9, 7] and st.starts.tolist() == [0, 4, 0, 0] and torch.equal(st.k[0][[0, 3]], k_before)
+    hid2, _ = om.trunk(torch.as_tensor(seqs[:2, :9]))
+    ref2 = om.logits(hid2).float().numpy()
+    assert np.abs(lg.float().cpu().numpy()[0] - ref2[0, 4]).max() < (0.15 if dtype == torch.bfloat16 else 0.04)   # 5 real tokens
+    assert np.abs(lg.float().cpu().numpy()[1] - ref2[1, 8]).max() < (0.15 if dtype == torch.bfloat16 else 0.04)

@@ -42,6 +42,28 @@ class KernelDecodeState(KVState):
         self.host_pos = np.zeros(B, dtype=np.int64)
 
 
+class DecodeState(KVState):
+    """DecodeState(cfg, B, max_len, dtype, device) of the reference (ultraviolet/model.py:1042-1072): the uncompressed cache
+    of its SDPA decode path - k[l], v[l] (B, K, S, hd) in `dtype`, S = max_len on global layers (rounded up to a multiple of
+    32 here) and min(window, max_len) ring slots on local ones, pos / starts (B,) int64 on the device, host_pos, kv_dtype =
+    None, set_pos, nbytes.  Where the reference attends such a cache through dense additive masks over all g_len slots
+    (model.py:968-1002), the engine reads each row's valid range lo..pos from it - the same keys.  16-bit dtypes."""
+    mix: dict = {}
+    prev = None
+
+    def __init__(self, cfg, B: int, max_len: int, dtype=torch.bfloat16, device="cuda"):
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise L.UvmiError("DecodeState keeps K / V in a 16-bit dtype (the engine's activation type)")
+        super().__init__(as_uvconfig(cfg), B, max_len, device, kv_dtype="fp16", dtype=dtype)
+        self.kv_dtype = None          # the reference's marker of the uncompressed state (model.py:1045)
+        self.dtype = dtype
+        self.host_pos = np.zeros(B, dtype=np.int64)
+
+    def set_pos(self, p: int):
+        self.pos.fill_(p)
+        self.host_pos[:] = p
+
+
 def kv_bytes_per_seq(cfg, ctx: int, kv_dtype: str = "int8") -> int:
     """Cache bytes of one sequence at context ctx (reference: fast_decode.py:60-67): hd + 2 bytes per key / value row
     with int8 + fp16 scale, 2 hd unquantized."""
@@ -124,11 +146,16 @@ def decode_step_fast(self, tok: Tensor, st: KVState, g_len: int = 0, skip_attn: 
     return h if return_hidden else eng.logits(h)
 
 
-def patch_model(model, kv_dtype: str = "fp16", num_splits: dict | None = None, backend: str = "auto",
+def patch_model(model, kv_dtype: str | None = "fp16", num_splits: dict | None = None, backend: str = "auto",
                 dtype: torch.dtype = torch.bfloat16, max_tokens: int = 16384, device=None):
     """Bind the kernel decode path onto `model` (instance attributes only).  model.cfg and model.state_dict() must use
     the reference's names.  dtype: activation / weight dtype of the engine; max_tokens: largest number of token rows of
-    one call (decode rows or packed prefill tokens)."""
+    one call (decode rows or packed prefill tokens).  kv_dtype None (or "sdpa") binds the reference's uncompressed
+    DecodeState instead of a KernelDecodeState: the entry points of its SDPA path - MathLM.new_state / prefill / decode_step
+    with decode_impl "sdpa" (ultraviolet/model.py:861-872, 880-1008) - on the same kernels."""
+    sdpa = kv_dtype in (None, "sdpa")
+    if sdpa:
+        kv_dtype = "fp16"
     if kv_dtype not in ("int8", "fp16"):
         raise L.UvmiError(f"kv_dtype {kv_dtype!r}: the KV layouts are 'int8' and 'fp16' (unquantized, in the compute dtype)")
     if kv_dtype == "fp16" and dtype not in (torch.float16, torch.bfloat16):
@@ -142,6 +169,8 @@ def patch_model(model, kv_dtype: str = "fp16", num_splits: dict | None = None, b
 
     def new_state(self, batch, max_len, dtype=torch.float16, device=None):
         # (an unquantized cache is kept in the engine's activation dtype, whatever the caller's compute dtype is called)
+        if sdpa:
+            return DecodeState(cfg, batch, max_len, eng.dtype, device or dev)
         return KernelDecodeState(cfg, batch, max_len, eng.dtype if kv_dtype == "fp16" else dtype, device or dev, kv_dtype)
 
     def decode_step(self, tok, st, g_len=0, skip_attn=False):
