@@ -173,4 +173,5 @@ def test_c5_long_rollout_sixteen_sequences_teacher_forced_through_the_oracle():
     d = np.concatenate(diffs)
     assert np.isfinite(d).all()
     print("teacher-forced log-prob gap: mean %.4f p99 %.4f max %.4f over %d tokens" % (d.mean(), np.quantile(d, 0.99), d.max(), d.size))
-    assert d.mean() < 0.06 and np.quantile(d, 0.99) < 0.3 and d.max() < 1.0, (d.mean(), np.quantile(d, 0.99), d.max())
+    # measured: mean 0.006, p99 0.020, max 0.031 (bf16 logits of magnitude ~10 carry 2^-5 spacing); the bars are twice that
+    assert d.mean() < 0.015 and np.quantile(d, 0.99) < 0.05 and d.max() < 0.1, (d.mean(), np.quantile(d, 0.99), d.max())
