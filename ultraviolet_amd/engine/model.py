@@ -89,7 +89,8 @@ def rms_norm_eps(dtype: torch.dtype) -> float:
 
 class UVEngine:
     def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 1 << 30, fold_o_rows: int = 1 << 30,
-                 fold_gu_rows: int = 1 << 30, lean: bool = True, fold: bool = True, gemm_config: int = 0):
+                 fold_gu_rows: int = 1 << 30, lean: bool = True, fold: bool = True, gemm_config: int = 0,
+                 tiled_prefill: bool = True):
         """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens).
         skinny_rows: passes of at most this many rows run every projection on the skinny GEMM; fold_qkv_rows, fold_o_rows,
         fold_gu_rows: above skinny_rows, row counts up to which the QKV projection (with the pre-norm), the output
@@ -122,6 +123,7 @@ class UVEngine:
         self.fold_qkv_rows = int(fold_qkv_rows)
         self.fold_o_rows, self.fold_gu_rows = int(fold_o_rows), int(fold_gu_rows)
         self.lean, self.fold, self.gemm_config = bool(lean), bool(fold), int(gemm_config)
+        self.tiled_prefill = bool(tiled_prefill)
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -329,6 +331,8 @@ class UVEngine:
         if folded:
             return self._trunk_folded(n, fused_attn)
         fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and self.fold
+        tiled_gu = (fold_mlp and self.tiled_prefill and n >= 448 and cfg.d_model % 64 == 0
+                    and all("gu_il" in W for W in self.w.layers))
         x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
@@ -358,8 +362,11 @@ class UVEngine:
                 # on the hidden in place and the MLP's pre-norm is the row scale inside the SwiGLU launch; the block ends
                 # with the norm the next block's projection and post-processing read
                 torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
-                torch.mm(x, W["gu"].t(), out=b["gu"][:n])
-                self._swiglu_norm(x, n)
+                if tiled_gu:   # the tiled GEMM with the pre-norm and the SwiGLU in it: the (n, 2 f) product is never written
+                    gemm_tn(x, W["gu_il"], b["act"][:n], epilogue=SWIGLU, norm_eps=self.eps, config=self.gemm_config)
+                else:
+                    torch.mm(x, W["gu"].t(), out=b["gu"][:n])
+                    self._swiglu_norm(x, n)
                 torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
                 self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
                 continue
