@@ -15,14 +15,16 @@
 //     key 4g+j of tile A (j < 4) or of tile B (j >= 4): probabilities never move between lanes;
 //   * V^T operands come from 8-byte loads (lane = dims 4m..4m+3 of 8 keys) regrouped with v_perm_b32 into four
 //     operands whose row m is head dim 4m + t; they are built once per super-tile and shared by the wave's 4 heads,
-//     as are the K operands (16-byte loads, lane = key m, dims 8g..8g+7 of each half);
-//   * loads are raw buffer loads with per-lane row offsets clamped to the last row; the next super-tile is requested
-//     before the current one is used;
+//     as are the K operands (16-byte reads, lane = key m, dims 8g..8g+7 of each half);
+//   * the 4 waves of a workgroup are 2 consecutive query blocks x 2 head groups (4 blocks x 1 group for up to 4 query
+//     heads per kv head) of one kv head and walk the same keys, so a super-tile of K and V is fetched once per workgroup:
+//     each thread requests 16 bytes of K and of V two tiles ahead into registers, parks them in one of two LDS halves
+//     (K rows chunk-swizzled, so the 16-byte operand reads are conflict-free) and the waves take their operands from
+//     there, one barrier per tile; a wave skips the tiles outside its own block's key range;
 //   * online softmax per (row, head) in the exp2 domain; tiles that every row of the block sees completely skip the
 //     mask arithmetic (one branch per tile, so the four heads of a tile form one block the scheduler interleaves);
-//   * the 4 waves of a workgroup are independent (2 query blocks x 2 head groups), so K/V of a block are fetched
-//     from L2 once per pair of waves; workgroup ids are remapped so that each XCD (one L2 each) owns a contiguous
-//     range of query blocks and therefore whole sequences.
+//   * workgroup ids are remapped so that each XCD (one L2 each) owns a contiguous range of query blocks and therefore
+//     whole sequences.
 //
 // Everything else (fp32 K/V, other head dims) goes token by token through the decode kernel's generic path with the
 // packed K/V as a batch-stride-0 "cache".
@@ -45,8 +47,8 @@ struct PrefillParams {
   const void* q; const void* k; const void* v; void* out;
   const int32_t* seg_start;  // (N,) packed index of the first token of each token's sequence
   int64_t sqn, sqh, skn, skh, svn, svh, son, soh;
-  int N, H, KH, G, window, n_hg;
-  int64_t n_items;
+  int N, H, KH, G, window, n_hg;   // n_hg: head groups of 4 query heads per kv head, 1 or 2
+  int n_wg;                        // workgroups with work: ceil(query blocks / (4 / n_hg)) * KH
   float scale_log2;
   const float* post_vhat; const float* post_gate; const float* post_xsa;  // fused Attention.post epilogue when post_vhat != null
 };
@@ -116,25 +118,32 @@ struct PTile {   // one 32-key super-tile as loaded (32 dwords per lane)
 
 constexpr int HPW = 4;  // query heads per wave
 
+constexpr int RING = 2;  // super-tiles requested ahead of the one being parked in LDS
+
 template <int DT, int ODT>
 __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][4096];  // [half][K, V][32 keys x 128 B]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // gridDim.x is a multiple of 8; ids congruent mod 8 run on one XCD and get a contiguous range of work
   const int per = gridDim.x >> 3;
   const int bid = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  const int64_t item = (int64_t)bid * 4 + wave;
-  if (item >= P.n_items) return;
-  const int hg = (int)(item % P.n_hg);
-  const int64_t rest = item / P.n_hg;
-  const int kvh = (int)(rest % P.KH);
-  const int qb = (int)(rest / P.KH);
+  if (bid >= P.n_wg) return;   // (the whole workgroup: no barrier is left waiting)
+  const int kvh = bid % P.KH;
+  const int qg = bid / P.KH;               // group of 4 / n_hg consecutive query blocks
+  const int hsh = P.n_hg - 1;              // n_hg is 1 or 2
+  const int qbw = 4 >> hsh;
+  const int hg = wave & hsh;
+  const int qb = qg * qbw + (wave >> hsh);
   const int m = lane & 15, g = lane >> 4;
   const int G = P.G;
   const float c = P.scale_log2;
 
-  // ---- this lane's query row (accumulator column m) and its key range
+  // ---- this lane's query row (accumulator column m) and its key range; a wave whose block starts past the last token
+  // (the tail of the last group) has an empty range and only helps with the loads
   const int r0 = qb * 16;
+  const bool wave_ok = r0 < P.N;
   const int row = r0 + m;
   const bool row_ok = row < P.N;
   const int rowc = row_ok ? row : P.N - 1;
@@ -143,8 +152,15 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
   if (!row_ok) lo_n = INT_MAX;
   const int rl = min(r0 + 15, P.N - 1);                                       // last real row of the block
   const int lo_first = __builtin_amdgcn_readfirstlane(lo_n);                  // lo is non-decreasing in the row
-  const int lo_last = __builtin_amdgcn_readfirstlane(__shfl(lo_n, rl - r0, 64));
-  const int kbeg = lo_first & ~31, kend = rl + 1;
+  const int lo_last = __builtin_amdgcn_readfirstlane(__shfl(lo_n, wave_ok ? rl - r0 : 0, 64));
+  const int kbeg = wave_ok ? lo_first & ~31 : 0, kend = wave_ok ? rl + 1 : 0;
+  // ---- the workgroup's key range: from the first row's lower bound (the smallest of the group) to its last row
+  const int row0 = qg * qbw * 16;          // < N
+  int lo0 = P.seg_start[row0];
+  if (P.window > 0 && row0 - P.window + 1 > lo0) lo0 = row0 - P.window + 1;
+  const int kbeg_wg = __builtin_amdgcn_readfirstlane(lo0) & ~31;
+  const int kend_wg = min(row0 + qbw * 16, P.N);
+  const int nk = (kend_wg - kbeg_wg + 31) >> 5;   // >= 1
 
   // ---- Q^T operands: lane (row m, group g) holds q[row][head][32 s + 8 g .. + 8] for s = 0, 1
   pu4 Q[HPW][2];
@@ -176,20 +192,37 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
   const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)((uint32_t)(P.N - 1) * skn2 + 128), 0x00020000);
   const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (int)((uint32_t)(P.N - 1) * svn2 + 128), 0x00020000);
 
-  // Rows are addressed per lane and clamped to N - 1 (the scalar offset of a buffer load is not part of its bounds
-  // check, so a tile reaching past row N must not rely on the descriptor); clamped rows are masked keys.
-  auto load_tile = [&](int tb_in, PTile& T) {
-    const int tb = __builtin_amdgcn_readfirstlane(tb_in);
-    const int last = P.N - 1;
-    const uint32_t ka = (uint32_t)min(tb + m, last) * skn2 + 16 * g, kb = (uint32_t)min(tb + 16 + m, last) * skn2 + 16 * g;
-    T.k[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, ka, 0, 0);
-    T.k[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, ka + 64, 0, 0);
-    T.k[2] = __builtin_amdgcn_raw_buffer_load_b128(rK, kb, 0, 0);
-    T.k[3] = __builtin_amdgcn_raw_buffer_load_b128(rK, kb + 64, 0, 0);
+  // ---- K / V super-tiles go global -> registers (RING tiles ahead) -> LDS (two halves) -> MFMA operands.  Thread t moves
+  // 16 bytes of K and of V per tile: key t / 8, chunk t % 8 of the 128-byte row.  Rows are clamped to N - 1 (the keys of a
+  // clamped row are masked); tiles past the group's last are re-reads of the last one.  K rows are stored with their
+  // 16-byte chunks XOR-swizzled by (key / 2) % 8, which makes both the stores and the operand reads (lane = key m, chunk
+  // 4 s + g) free of bank conflicts; V rows are stored as they are (an operand read takes whole 128-byte rows).
+  pu4 rk[RING], rv[RING];
+  const int lkey = tid >> 3, lch = tid & 7;
+  const uint32_t kst = (uint32_t)lkey * 128 + (uint32_t)((lch ^ ((lkey >> 1) & 7)) << 4), vst = (uint32_t)lkey * 128 + (uint32_t)lch * 16;
+  auto fetch = [&](int k, int slot) {
+    const int tb = kbeg_wg + 32 * min(k, nk - 1);
+    const uint32_t r = (uint32_t)min(tb + lkey, P.N - 1);
+    rk[slot] = __builtin_amdgcn_raw_buffer_load_b128(rK, r * skn2 + 16 * lch, 0, 0);
+    rv[slot] = __builtin_amdgcn_raw_buffer_load_b128(rV, r * svn2 + 16 * lch, 0, 0);
+  };
+  auto park = [&](int slot, int half) {
+    *(pu4*)(&smem[half][0][kst]) = rk[slot];
+    *(pu4*)(&smem[half][1][vst]) = rv[slot];
+  };
+  const uint32_t kld0 = (uint32_t)m * 128 + (uint32_t)((g ^ ((m >> 1) & 7)) << 4), kld1 = (uint32_t)m * 128 + (uint32_t)(((4 + g) ^ ((m >> 1) & 7)) << 4);
+  const uint32_t vld = (uint32_t)(4 * g) * 128 + 8 * m;
+  auto read_tile = [&](int half, PTile& T) {
+    const unsigned char* sk = smem[half][0];
+    const unsigned char* sv = smem[half][1];
+    T.k[0] = *(const pu4*)(sk + kld0);
+    T.k[1] = *(const pu4*)(sk + kld1);
+    T.k[2] = *(const pu4*)(sk + 2048 + kld0);
+    T.k[3] = *(const pu4*)(sk + 2048 + kld1);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      T.v[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, (uint32_t)min(tb + 4 * g + j, last) * svn2 + 8 * m, 0, 0);
-      T.v[4 + j] = __builtin_amdgcn_raw_buffer_load_b64(rV, (uint32_t)min(tb + 16 + 4 * g + j, last) * svn2 + 8 * m, 0, 0);
+      T.v[j] = *(const pu2*)(sv + vld + 128 * j);
+      T.v[4 + j] = *(const pu2*)(sv + 2048 + vld + 128 * j);
     }
   };
 
@@ -256,20 +289,32 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
     // a tile needs no mask when every row of the block sees all of it: it starts at or after the last row's lower
     // bound and ends at or before the first row
     auto edge_of = [&](int tb) { return !(tb >= lo_last && tb + 31 <= r0); };
-    auto next_of = [&](int tb) { return tb + 32 < kend ? tb + 32 : tb; };  // past the end: re-read (a cache hit)
-    int tb = kbeg;
-    PTile TA, TB;
-    load_tile(tb, TA);
-    while (true) {
-      load_tile(next_of(tb), TB);
-      step(TA, tb, edge_of(tb));
-      tb += 32;
-      if (tb >= kend) break;
-      load_tile(next_of(tb), TA);
-      step(TB, tb, edge_of(tb));
-      tb += 32;
-      if (tb >= kend) break;
+    // iteration k: this wave's operands of tile k come out of LDS half k % 2 (when the tile lies in the wave's own range),
+    // tile k + 1 is parked in the other half, tile k + 1 + RING is requested into the ring slot that frees, then the
+    // arithmetic of tile k runs; the barrier lets the next iteration overwrite the half just read
+    auto iteration = [&](int k, int d) {
+      const int tb = kbeg_wg + 32 * k;
+      const bool act = tb >= kbeg && tb < kend;   // wave-uniform
+      PTile T;
+      if (act) read_tile(k & 1, T);
+      park((d + 1) % RING, (k + 1) & 1);
+      fetch(k + 1 + RING, (d + 1) % RING);
+      if (act) step(T, tb, edge_of(tb));
+      __syncthreads();
+    };
+#pragma unroll
+    for (int d = 0; d < RING; d++) fetch(d, d);
+    park(0, 0);
+    fetch(RING, 0);
+    __syncthreads();
+    int k = 0;
+    for (; k + RING <= nk; k += RING) {
+#pragma unroll
+      for (int d = 0; d < RING; d++) iteration(k + d, d);
     }
+#pragma unroll
+    for (int d = 0; d < RING - 1; d++)
+      if (k + d < nk) iteration(k + d, d);   // workgroup-uniform
   }
 
   // ---- normalise and store: lane (row m, group g) holds head dims 16g .. 16g+15 (O[t][i] is dim 16g + 4i + t)
@@ -413,12 +458,14 @@ extern "C" int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream) 
   P.q = a->q; P.k = a->k; P.v = a->v; P.out = a->out; P.seg_start = seg_start;
   P.sqn = a->sqn; P.sqh = a->sqh; P.skn = a->skn; P.skh = a->skh; P.svn = a->svn; P.svh = a->svh; P.son = a->son; P.soh = a->soh;
   P.N = a->N; P.H = a->H; P.KH = a->KH; P.G = a->H / a->KH; P.window = a->window;
-  P.n_hg = (P.G + HPW - 1) / HPW;
-  P.n_items = (int64_t)((a->N + 15) / 16) * a->KH * P.n_hg;
+  P.n_hg = (P.G + HPW - 1) / HPW;   // 1 or 2 (G <= 8)
+  const int64_t n_qb = (a->N + 15) / 16, qbw = 4 / P.n_hg;
+  const int64_t n_wg = (n_qb + qbw - 1) / qbw * a->KH;
   P.scale_log2 = a->scale * 1.4426950408889634f;
   P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa;
-  UVMI_REQUIRE(P.n_items < (1LL << 31), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: too many work items");
-  const unsigned nblk = (unsigned)(((P.n_items + 3) / 4 + 7) / 8 * 8);
+  UVMI_REQUIRE(n_wg < (1LL << 30), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: too many work items");
+  P.n_wg = (int)n_wg;
+  const unsigned nblk = (unsigned)((n_wg + 7) / 8 * 8);
   const dim3 grid(nblk), blk(256);
   const int od = a->out_dtype;
 #define UVMI_L(QD)                                                                                                \
