@@ -74,6 +74,35 @@ def test_few_and_many_rows_on_long_caches(dtype, B, S, ring):
     _attn_check(q, k, v, ks, vs, pos, starts, 1.13 / 8, window=S if ring else 0, ring=ring)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,S,ring,G", [(3, 1056, False, 8), (200, 1056, False, 8), (300, 2080, False, 4), (40, 1024, True, 8), (64, 256, True, 2),
+                                        (50, 100, False, 8)])
+def test_unquantized_cache_on_the_mfma_kernel(dtype, B, S, ring, G):
+    """K / V cached unquantized in the q dtype (the reference's accuracy baseline, fast_decode.py:21-57 with kv_dtype fp16):
+    head_dim 64 runs on the MFMA kernel too - 1, 2 and 4 waves per row, ring wrap-around, left-padded starts, a cache that
+    ends inside a super-tile - and slots outside lo..pos may hold NaN patterns."""
+    from ultraviolet_amd.kernels import decode_attention
+    from ultraviolet_amd.kernels.decode_attn import supported
+    q, k, v, _, _ = attn_case(B, 1, G, 64, S, False, dtype=dtype, seed=B)
+    g = torch.Generator().manual_seed(B + S)
+    pos = torch.randint(0, S if not ring else 5 * S, (B,), generator=g)
+    pos[0], pos[1 % B] = (S - 1 if not ring else 3 * S + 17), 0
+    starts = (torch.rand(B, generator=g) * (pos + 1).float()).long()
+    starts[0] = 0
+    d = lambda t: t.to(DEV)
+    assert supported(d(q), d(k))
+    o32, ref = _attn_check(q, k, v, None, None, pos, starts, 1.13 / 8, window=S if ring else 0, ring=ring)
+    if not ring:   # poison what no row may read
+        k2, v2 = k.clone(), v.clone()
+        for b in range(B):
+            bad = torch.ones(S, dtype=torch.bool)
+            bad[starts[b]:pos[b] + 1] = False
+            k2[b, 0, bad] = float("nan")
+            v2[b, 0, bad] = float("nan")
+        out = decode_attention(d(q), d(k2), d(v2), d(pos), d(starts), 1.13 / 8, out_fp32=True)
+        assert torch.equal(out.cpu(), torch.from_numpy(o32))
+
+
 @pytest.mark.parametrize("int8", [False, True])
 @pytest.mark.parametrize("W,hd,G", [(128, 128, 5), (256, 64, 8), (1024, 128, 4), (100, 128, 4), (64, 64, 8),
                                     (100, 64, 8)])

@@ -30,6 +30,7 @@
 #include "common.h"
 
 #include <cstdlib>
+#include <type_traits>
 #include <mutex>
 
 namespace uvmi {
@@ -162,6 +163,25 @@ struct Tile {             // one 32-key super-tile as loaded from HBM (26 dwords
   uint2 ksc, vsc;         // fp16 scales of keys 4g..4g+3 of this lane's stream
 };
 
+struct Tile16 {           // the same super-tile of a 16-bit cache (32 dwords per lane)
+  u4 kA[2], kB[2];        // key m of stream A / B, dims 16g..16g+7 and 16g+8..16g+15
+  u2 vA[4], vB[4];        // keys 4g+j of stream A / B, dims 4m..4m+3
+};
+
+// 16x16x32 MFMA on operand words of the 16-bit type DT (the int8 path always multiplies in fp16)
+template <int DT>
+__device__ __forceinline__ f4 mfma_kv(const h8& a, const h8& b, f4 acc) {
+  if constexpr (DT == UVMI_BF16) {
+    typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+    b8 x, y;
+    __builtin_memcpy(&x, &a, 16);
+    __builtin_memcpy(&y, &b, 16);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, acc, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+  }
+}
+
 struct AttnState {
   f4 O[4];                // O''^T tiles: 2^-24 * sum (v + 128) P'
   float mrun, lrun, psum; // running max (score units before scale), sum p, sum of the fp16-rounded P'
@@ -177,7 +197,10 @@ struct AttnState {
 // The arguments ahead of the parameter block are what a wave needs before it can request anything - the index arrays of
 // the row's plan, the q (or projection) pointer and the item arithmetic: as leading scalar arguments they are preloaded
 // into SGPRs with the wave, so the plan's loads go out without first waiting for a load of the kernel arguments.
-template <int QDT, int ODT, int WPR, bool FUSE>
+// KV16: the cache holds K / V unquantized in the q dtype (no scales): the same work split, plan, online softmax, merge and
+// epilogue around tiles that go into the MFMAs as they are loaded - no conversion, no bias terms, probabilities rounded to
+// the cache type (a tile is 32 dwords per lane, still 4 waves per SIMD).  Not combined with FUSE.
+template <int QDT, int ODT, int WPR, bool FUSE, bool KV16 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_rows, const void* a_q, int64_t a_items, int a_idx64,
                        int a_splits, int a_kh, AttnParams P) {
@@ -266,7 +289,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   auto set_q = [&]() {
     QA0 = as_h8(qr[0] & mA, qr[1] & mA, qr[2] & mA, qr[3] & mA); QA1 = as_h8(qr[4] & mA, qr[5] & mA, qr[6] & mA, qr[7] & mA);
     QB0 = as_h8(qr[0] & mB, qr[1] & mB, qr[2] & mB, qr[3] & mB); QB1 = as_h8(qr[4] & mB, qr[5] & mB, qr[6] & mB, qr[7] & mB);
-    cinit = qmask ? -1152.0f * qsum : 0.f;
+    cinit = !KV16 && qmask ? -1152.0f * qsum : 0.f;
   };
   // unfused: q arrives normalised and rotated, 16 dims per lane in the operand layout
   auto prep_q = [&]() {
@@ -277,9 +300,13 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       float f0, f1;
       if (QDT == UVMI_BF16) { f0 = __uint_as_float(w[i] << 16); f1 = __uint_as_float(w[i] & 0xffff0000u); }
       else { f0 = half_bits_to_float(w[i] & 0xffff); f1 = half_bits_to_float(w[i] >> 16); }
-      const uint16_t l16 = float_to_half_bits(f0), h16 = float_to_half_bits(f1);
-      qr[i] = (uint32_t)l16 | ((uint32_t)h16 << 16);
-      qsum += half_bits_to_float(l16) + half_bits_to_float(h16);
+      if constexpr (KV16) {
+        qr[i] = w[i];   // the product runs in the q dtype itself
+      } else {
+        const uint16_t l16 = float_to_half_bits(f0), h16 = float_to_half_bits(f1);
+        qr[i] = (uint32_t)l16 | ((uint32_t)h16 << 16);
+        qsum += half_bits_to_float(l16) + half_bits_to_float(h16);
+      }
     }
     qsum = xsum32(xsum16(qsum));  // all 64 dims of this head
     set_q();
@@ -404,21 +431,22 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
 
   // ---- addressing: wave-uniform row base + wave-uniform tile offset (scalar) + lane-invariant 32-bit offsets
   const int64_t cb = rp.cb;
-  const int8_t* kbase = (const int8_t*)P.kc + cb * P.skb + (int64_t)h * P.skh;
-  const int8_t* vbase = (const int8_t*)P.vc + cb * P.svb + (int64_t)h * P.svh;
+  constexpr int ES = KV16 ? 2 : 1;   // bytes per cache element
+  const int8_t* kbase = (const int8_t*)P.kc + (cb * P.skb + (int64_t)h * P.skh) * ES;
+  const int8_t* vbase = (const int8_t*)P.vc + (cb * P.svb + (int64_t)h * P.svh) * ES;
   const uint16_t* ksb = (const uint16_t*)P.ks + cb * P.ssb + (int64_t)h * P.ssh;
   const uint16_t* vsb = (const uint16_t*)P.vs + cb * P.stb + (int64_t)h * P.sth;
   const int S = P.S;
-  const uint32_t sks = (uint32_t)P.sks, svs = (uint32_t)P.svs;
+  const uint32_t sks = (uint32_t)P.sks * ES, svs = (uint32_t)P.svs * ES;   // row strides in bytes
   const uint32_t usks = __builtin_amdgcn_readfirstlane(sks), usvs = __builtin_amdgcn_readfirstlane(svs);
-  const uint32_t koA = m * sks + 16 * g, koB = koA + 16 * sks;  // K: key m of stream A / B, bytes 16g..
-  const uint32_t voA = 4 * g * svs + 4 * m;     // V: key 4g (+j via the scalar offset), bytes 4m..
+  const uint32_t koA = m * sks + 16 * ES * g, koB = koA + 16 * sks;  // K: key m of stream A / B, dims 16g..
+  const uint32_t voA = 4 * g * svs + 4 * ES * m;     // V: key 4g (+j via the scalar offset), dims 4m..
   const uint32_t so = 16 * strm + 4 * g;  // scale offset (elements) inside the super-tile
 
   // Buffer descriptors (wave-uniform, one per row stream): a load is descriptor base + lane-invariant VGPR offset +
   // scalar tile offset, so the loop spends no VALU work on addresses.  num_records covers exactly the row's bytes.
-  const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (S - 1) * (int)sks + 64, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (S - 1) * (int)svs + 64, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rK = __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (S - 1) * (int)sks + 64 * ES, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rV = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, (S - 1) * (int)svs + 64 * ES, 0x00020000);
   const __amdgpu_buffer_rsrc_t rKS = __builtin_amdgcn_make_buffer_rsrc((void*)ksb, 0, S * 2, 0x00020000);
   const __amdgpu_buffer_rsrc_t rVS = __builtin_amdgcn_make_buffer_rsrc((void*)vsb, 0, S * 2, 0x00020000);
   const uint32_t so2 = so * 2;
@@ -426,9 +454,21 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   // slot0: cache slot of absolute position tb (a multiple of 32).  Ring caches have S % 32 == 0 (host-checked), so a
   // super-tile never wraps.  load_tile needs slot0 + 32 <= S; a linear cache that ends inside its last super-tile
   // takes load_tail (per-lane clamped rows) for that one tile, outside the pipelined loop.
-  auto load_tile = [&](int slot_in, Tile& T) {
+  using TileX = std::conditional_t<KV16, Tile16, Tile>;
+  auto load_tile = [&](int slot_in, TileX& T) {
     const int slot0 = __builtin_amdgcn_readfirstlane(slot_in);  // wave-uniform by construction
     const uint32_t ok = (uint32_t)slot0 * usks, ov = (uint32_t)slot0 * usvs, os = (uint32_t)slot0 * 2;
+    if constexpr (KV16) {
+      T.kA[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koA, ok, 0);
+      T.kA[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koA + 16, ok, 0);
+      T.kB[0] = __builtin_amdgcn_raw_buffer_load_b128(rK, koB, ok, 0);
+      T.kB[1] = __builtin_amdgcn_raw_buffer_load_b128(rK, koB + 16, ok, 0);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        T.vA[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + j * usvs, 0);
+        T.vB[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + (16 + j) * usvs, 0);
+      }
+    } else {
     u4 ka = __builtin_amdgcn_raw_buffer_load_b128(rK, koA, ok, 0);
     u4 kb = __builtin_amdgcn_raw_buffer_load_b128(rK, koB, ok, 0);
     T.kA = uint4{ka.x, ka.y, ka.z, ka.w};
@@ -442,9 +482,21 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     u2 c2 = __builtin_amdgcn_raw_buffer_load_b64(rVS, so2, os, 0);
     T.ksc = uint2{a.x, a.y};
     T.vsc = uint2{c2.x, c2.y};
+    }
   };
-  auto load_tail = [&](int slot0, Tile& T) {
+  auto load_tail = [&](int slot0, TileX& T) {
     const int smax = S - 1;
+    if constexpr (KV16) {
+      const int8_t* ka = kbase + (int64_t)min(slot0 + m, smax) * sks + 32 * g;
+      const int8_t* kb = kbase + (int64_t)min(slot0 + 16 + m, smax) * sks + 32 * g;
+      T.kA[0] = *(const u4*)ka; T.kA[1] = *(const u4*)(ka + 16);
+      T.kB[0] = *(const u4*)kb; T.kB[1] = *(const u4*)(kb + 16);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        T.vA[j] = *(const u2*)(vbase + (int64_t)min(slot0 + 4 * g + j, smax) * svs + 8 * m);
+        T.vB[j] = *(const u2*)(vbase + (int64_t)min(slot0 + 16 + 4 * g + j, smax) * svs + 8 * m);
+      }
+    } else {
     T.kA = *(const uint4*)(kbase + (int64_t)min(slot0 + m, smax) * P.sks + 16 * g);
     T.kB = *(const uint4*)(kbase + (int64_t)min(slot0 + 16 + m, smax) * P.sks + 16 * g);
 #pragma unroll
@@ -455,12 +507,27 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     const int ss = min(slot0 + (int)so, S - 4);  // S % 4 == 0: a clamped group is entirely past the cache end
     T.ksc = *(const uint2*)(ksb + ss);
     T.vsc = *(const uint2*)(vsb + ss);
+    }
   };
 
-  auto step = [&](const Tile& T, int tb, bool edge) {
-    // ---- S^T = K' . Q^T - 1152 sum(q), K' = 1024 + (k ^ 0x80) as fp16 0x64uu
+  auto step = [&](const TileX& T, int tb, bool edge) {
+    // ---- S^T = K' . Q^T - 1152 sum(q), K' = 1024 + (k ^ 0x80) as fp16 0x64uu (16-bit cache: K as loaded, no bias)
     f4 acc = f4{cinit, cinit, cinit, cinit};
-    {
+    if constexpr (KV16) {
+      // An accumulator column sums one stream's products and the other stream's products with zeros, so on an edge tile
+      // the rows of keys outside the range are cleared first: a slot never written may hold a NaN or Inf pattern, and
+      // 0 x NaN would reach the score of the other stream's valid key.
+      u4 a0 = T.kA[0], a1 = T.kA[1], b0 = T.kB[0], b1 = T.kB[1];
+      if (edge) {
+        const u4 z = u4{0u, 0u, 0u, 0u};
+        if (tb + m < lo_eff || tb + m >= s1) { a0 = z; a1 = z; }
+        if (tb + 16 + m < lo_eff || tb + 16 + m >= s1) { b0 = z; b1 = z; }
+      }
+      acc = mfma_kv<QDT>(as_h8(a0.x, a0.y, a0.z, a0.w), QA0, acc);
+      acc = mfma_kv<QDT>(as_h8(a1.x, a1.y, a1.z, a1.w), QA1, acc);
+      acc = mfma_kv<QDT>(as_h8(b0.x, b0.y, b0.z, b0.w), QB0, acc);
+      acc = mfma_kv<QDT>(as_h8(b1.x, b1.y, b1.z, b1.w), QB1, acc);
+    } else {
       const uint32_t a0 = T.kA.x ^ 0x80808080u, a1 = T.kA.y ^ 0x80808080u, a2 = T.kA.z ^ 0x80808080u, a3 = T.kA.w ^ 0x80808080u;
       const uint32_t b0 = T.kB.x ^ 0x80808080u, b1 = T.kB.y ^ 0x80808080u, b2 = T.kB.z ^ 0x80808080u, b3 = T.kB.w ^ 0x80808080u;
       constexpr uint32_t C64 = 0x64646464u, LO = 0x04010400u, HI = 0x04030402u;
@@ -470,11 +537,17 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_h8(perm(C64, b2, LO), perm(C64, b2, HI), perm(C64, b3, LO), perm(C64, b3, HI)), QB1, acc, 0, 0, 0);
     }
     // ---- t_i = (q.k_int) * kscale_i for the lane's keys 4g+i of its stream (softmax scale applied inside exp2)
-    h2 ks01, ks23, vs01, vs23;
-    __builtin_memcpy(&ks01, &T.ksc.x, 4); __builtin_memcpy(&ks23, &T.ksc.y, 4);
-    __builtin_memcpy(&vs01, &T.vsc.x, 4); __builtin_memcpy(&vs23, &T.vsc.y, 4);
-    float t[4] = {acc[0] * (float)ks01[0], acc[1] * (float)ks01[1], acc[2] * (float)ks23[0], acc[3] * (float)ks23[1]};
-    float vsf[4] = {(float)vs01[0], (float)vs01[1], (float)vs23[0], (float)vs23[1]};
+    float t[4], vsf[4];
+    if constexpr (KV16) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) { t[i] = acc[i]; vsf[i] = 1.f; }
+    } else {
+      h2 ks01, ks23, vs01, vs23;
+      __builtin_memcpy(&ks01, &T.ksc.x, 4); __builtin_memcpy(&ks23, &T.ksc.y, 4);
+      __builtin_memcpy(&vs01, &T.vsc.x, 4); __builtin_memcpy(&vs23, &T.vsc.y, 4);
+      t[0] = acc[0] * (float)ks01[0]; t[1] = acc[1] * (float)ks01[1]; t[2] = acc[2] * (float)ks23[0]; t[3] = acc[3] * (float)ks23[1];
+      vsf[0] = (float)vs01[0]; vsf[1] = (float)vs01[1]; vsf[2] = (float)vs23[0]; vsf[3] = (float)vs23[1];
+    }
     if (edge) {  // keys outside [lo_eff, s1): no score, and their (possibly stale, non-finite) V scale must not meet p = 0
       const int t0 = tb + 16 * strm + 4 * g;
 #pragma unroll
@@ -497,18 +570,58 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
 #pragma unroll
     for (int i = 0; i < 4; i++) p[i] = __builtin_amdgcn_exp2f(fmaf(t[i], c, -mc));
     st.lrun += (p[0] + p[1]) + (p[2] + p[3]);
-    // ---- P' = fp16(p * vscale), placed in this stream's half of the contraction slots
-    const h2 p01 = h2{(_Float16)(p[0] * vsf[0]), (_Float16)(p[1] * vsf[1])};
-    const h2 p23 = h2{(_Float16)(p[2] * vsf[2]), (_Float16)(p[3] * vsf[3])};
-    const h2 ones = h2{(_Float16)1.0f, (_Float16)1.0f};
-    st.psum = __builtin_amdgcn_fdot2(p23, ones, __builtin_amdgcn_fdot2(p01, ones, st.psum, false), false);
+    // ---- P' = fp16(p * vscale) (16-bit cache: p rounded to the cache type), placed in this stream's half of the
+    // contraction slots
     uint32_t u01, u23;
-    __builtin_memcpy(&u01, &p01, 4);
-    __builtin_memcpy(&u23, &p23, 4);
+    [[maybe_unused]] uint32_t l01 = 0, l23 = 0;
+    if constexpr (KV16 && QDT == UVMI_BF16) {
+      // a bf16 cache: p goes in as two bf16 terms, p = hi + lo (16 significant bits, where a single bf16 has 8), and P V is
+      // two MFMAs per operand - the matrix pipe has the room, and the result stays within the fp16 path's error
+      typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+      const b2 p01 = b2{(__bf16)p[0], (__bf16)p[1]}, p23 = b2{(__bf16)p[2], (__bf16)p[3]};
+      const b2 q01 = b2{(__bf16)(p[0] - (float)p01[0]), (__bf16)(p[1] - (float)p01[1])};
+      const b2 q23 = b2{(__bf16)(p[2] - (float)p23[0]), (__bf16)(p[3] - (float)p23[1])};
+      __builtin_memcpy(&u01, &p01, 4);
+      __builtin_memcpy(&u23, &p23, 4);
+      __builtin_memcpy(&l01, &q01, 4);
+      __builtin_memcpy(&l23, &q23, 4);
+    } else {
+      const h2 p01 = h2{(_Float16)(p[0] * vsf[0]), (_Float16)(p[1] * vsf[1])};
+      const h2 p23 = h2{(_Float16)(p[2] * vsf[2]), (_Float16)(p[3] * vsf[3])};
+      if constexpr (!KV16) {
+        const h2 ones = h2{(_Float16)1.0f, (_Float16)1.0f};
+        st.psum = __builtin_amdgcn_fdot2(p23, ones, __builtin_amdgcn_fdot2(p01, ones, st.psum, false), false);
+      }
+      __builtin_memcpy(&u01, &p01, 4);
+      __builtin_memcpy(&u23, &p23, 4);
+    }
     const h8 PB = as_h8(u01 & mA, u23 & mA, u01 & mB, u23 & mB);
     // ---- O''^T += V'' . P'^T with V'' = (v ^ 0x80) * 2^-24 (fp16 subnormal 0x00uu; the MFMA takes subnormals);
     // tile tt, operand row m is head dim 4m + tt
-    {
+    if constexpr (KV16) {
+      // V as loaded: dword pairs (dims 4m..4m+3) of 8 keys; operand tt takes half tt of each pair.  On an edge tile the
+      // values of keys outside the range are cleared: a slot never written may hold a NaN pattern, and 0 x NaN is NaN.
+      u2 va_[4], vb_[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) { va_[j] = T.vA[j]; vb_[j] = T.vB[j]; }
+      if (edge) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int ka = tb + 4 * g + j, kb = ka + 16;
+          if (ka < lo_eff || ka >= s1) va_[j] = u2{0u, 0u};
+          if (kb < lo_eff || kb >= s1) vb_[j] = u2{0u, 0u};
+        }
+      }
+      constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) {
+        const uint32_t sel = (tt & 1) ? HI : LO;
+        const int e = tt >> 1;
+        const h8 va = as_h8(perm(va_[1][e], va_[0][e], sel), perm(va_[3][e], va_[2][e], sel), perm(vb_[1][e], vb_[0][e], sel), perm(vb_[3][e], vb_[2][e], sel));
+        st.O[tt] = mfma_kv<QDT>(va, PB, st.O[tt]);
+        if constexpr (QDT == UVMI_BF16) st.O[tt] = mfma_kv<QDT>(va, as_h8(l01 & mA, l23 & mA, l01 & mB, l23 & mB), st.O[tt]);
+      }
+    } else {
       uint32_t xa[4], xb[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) { xa[j] = T.vA[j] ^ 0x80808080u; xb[j] = T.vB[j] ^ 0x80808080u; }
@@ -557,7 +670,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     // follows it on every path and waits for q only.  (Requesting two tiles here was measured on the fused path, with no
     // spills: 20.5 us against 19.2 us per launch on ~2000 rows x ~215 keys - all waves' first two tiles then leave in
     // one burst of more than half the launch's bytes.)
-    Tile TA, TB;
+    TileX TA, TB;
     load_tile(slot, TA);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!FUSE) {
@@ -592,7 +705,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       }
     }
     if (tb < s1) {  // linear cache ending inside this super-tile (at most one wave of the item gets here)
-      Tile TT;
+      TileX TT;
       load_tail(tb, TT);
       step(TT, tb, true);
     }
@@ -605,8 +718,8 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   const float ms = mm == -INFINITY ? 0.f : mm;
   const float w_s = __builtin_amdgcn_exp2f(m2 - ms), w_o = __builtin_amdgcn_exp2f(m_o - ms);
   const float lm = lsum * w_s + l_o * w_o;
-  const float pm = 128.0f * (ps * w_s + ps_o * w_o);
-  const float w_s24 = w_s * 16777216.0f, w_o24 = w_o * 16777216.0f;
+  const float pm = KV16 ? 0.f : 128.0f * (ps * w_s + ps_o * w_o);
+  const float w_s24 = KV16 ? w_s : w_s * 16777216.0f, w_o24 = KV16 ? w_o : w_o * 16777216.0f;
   float o[16];  // head dims 16g .. 16g+15: O[t][i] is dim 16g + 4i + t
 #pragma unroll
   for (int t = 0; t < 4; t++)
@@ -936,6 +1049,24 @@ static bool mfma_ok(const uvmi_attn_args* a) {
   return true;
 }
 
+// The MFMA kernel on a cache that holds K / V unquantized in the q dtype.
+static bool mfma16_ok(const uvmi_attn_args* a) {
+  const int G = a->H / a->KH;
+  if (a->hd != 64 || G > 8 || a->kv_dtype != a->q_dtype || (a->q_dtype != UVMI_F16 && a->q_dtype != UVMI_BF16)) return false;
+  if (a->fuse) return false;
+  if (!(a->scale > 0.f)) return false;
+  if (a->ring && (a->S % 32 != 0)) return false;
+  if (a->S < 32) return false;  // a whole 32-key tile at slot 0 must exist
+  if (a->sks > (1 << 19) || a->svs > (1 << 19) || a->sks < 0 || a->svs < 0) return false;  // 32-bit tile offsets in bytes
+  auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
+  if (!al(a->q, 16) || a->sqb % 8 || a->sqh % 8) return false;
+  if (!al(a->k_cache, 16) || a->skb % 8 || a->skh % 8 || a->sks % 8) return false;   // 16-byte K loads
+  if (!al(a->v_cache, 8) || a->svb % 4 || a->svh % 4 || a->svs % 4) return false;    // 8-byte V loads
+  const int ob = a->out_dtype == UVMI_F32 ? 4 : 2;
+  if (!al(a->out, 16) || (a->sob * ob) % 16 || (a->soh * ob) % 16) return false;
+  return true;
+}
+
 }  // namespace uvmi
 
 using namespace uvmi;
@@ -965,7 +1096,7 @@ extern "C" int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus) {
 extern "C" int uvmi_decode_attn_path(const uvmi_attn_args* a) {
   int rc = check_common(a);
   if (rc) return rc;
-  return mfma_ok(a) ? 1 : 0;
+  return mfma_ok(a) || mfma16_ok(a) ? 1 : 0;
 }
 
 // The launch sequence of uvmi_decode_attn with the split partials in `ws` (ws_bytes of device memory; unused when
@@ -1005,8 +1136,8 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     P.post_vhat = nullptr; P.post_gate = nullptr;
   }
   if (a->post_vhat && !a->fuse) {
-    UVMI_REQUIRE(mfma_ok(a) && a->num_splits == 1, UVMI_EUNSUPPORTED,
-                 "uvmi_decode_attn: the fused post epilogue needs the MFMA kernel (head_dim 64, int8 cache) and num_splits == 1");
+    UVMI_REQUIRE((mfma_ok(a) || mfma16_ok(a)) && a->num_splits == 1, UVMI_EUNSUPPORTED,
+                 "uvmi_decode_attn: the fused post epilogue needs the MFMA kernel (head_dim 64, int8 cache or one of the q dtype) and num_splits == 1");
     UVMI_REQUIRE(is_float_dtype(a->post_round_dtype) && ((uintptr_t)a->post_vhat % 16) == 0, UVMI_EINVAL, "uvmi_decode_attn: bad post arguments");
   }
   if (a->num_splits > 1) {
@@ -1019,7 +1150,8 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     P.ws_l = P.ws_m + rows;
   }
   UVMI_REQUIRE(P.n_items < (1LL << 31), UVMI_EUNSUPPORTED, "uvmi_decode_attn: too many work items");
-  if (mfma_ok(a)) {
+  const bool kv16 = !mfma_ok(a) && mfma16_ok(a);
+  if (mfma_ok(a) || kv16) {
     // Waves per work item.  Long rows are streamed by all 4 waves of a workgroup, short ones by 2 or 1; and when 4 waves
     // per item would need more wave slots than the device has at this kernel's occupancy (4 per SIMD), 2 per item keep
     // the whole launch resident in one round instead of two (measured: 2000 rows x ~230 keys, 15.6 us against 18.9 us).
@@ -1048,8 +1180,20 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true>), grid, blk, 0, st, UVMI_LEAD, P);  \
     else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true>), grid, blk, 0, st, UVMI_LEAD, P);                \
   } while (0)
+#define UVMI_L16(QD, OD)                                                                              \
+  do {                                                                                                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 4, false, true>), grid, blk, 0, st, UVMI_LEAD, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2, false, true>), grid, blk, 0, st, UVMI_LEAD, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1, false, true>), grid, blk, 0, st, UVMI_LEAD, P);               \
+  } while (0)
     const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
-    if (a->fuse) {
+    if (kv16) {
+      if (a->q_dtype == UVMI_F16) {
+        if (od == UVMI_F16) UVMI_L16(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L16(UVMI_F16, UVMI_BF16); else UVMI_L16(UVMI_F16, UVMI_F32);
+      } else {
+        if (od == UVMI_F16) UVMI_L16(UVMI_BF16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L16(UVMI_BF16, UVMI_BF16); else UVMI_L16(UVMI_BF16, UVMI_F32);
+      }
+    } else if (a->fuse) {
       if (a->q_dtype == UVMI_F16) UVMI_LF(UVMI_F16); else UVMI_LF(UVMI_BF16);
     } else if (a->q_dtype == UVMI_F16) {
       if (od == UVMI_F16) UVMI_L(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(UVMI_F16, UVMI_BF16); else UVMI_L(UVMI_F16, UVMI_F32);
@@ -1058,6 +1202,7 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     }
 #undef UVMI_L
 #undef UVMI_LF
+#undef UVMI_L16
 #undef UVMI_LEAD
   } else {
     const dim3 grid((unsigned)P.n_items), blk(64);

@@ -220,15 +220,17 @@ class UVEngine:
     # ------------------------------------------------------------------------------------------------ trunk
     def cache_attention(self, l: int, q: Tensor, st: KVState, pos: Tensor, starts: Tensor, n: int, rows: Tensor | None = None,
                         off: int = 0):
-        """Decode attention of layer l over the int8 cache with the fused XSA + gate epilogue for the n rows that sit at
+        """Decode attention of layer l over the cache (int8, or unquantized) with the fused XSA + gate epilogue for the n rows that sit at
         off..off+n of the call's buffers (q is already that slice); writes buf zg[off:off+n] and returns None, or, where
         the fused epilogue does not apply, returns the plain attention output for _attn_post."""
         cfg, b, W = self.cfg, self.buf, self.w.layers[l]
         glob = cfg.is_global(l)
         S = st.k[l].size(2)
         kw = dict(window=0 if glob else cfg.window, ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=rows)
-        # the MFMA kernel (which carries the epilogue) streams 32-key tiles: rings need S % 32 == 0, linear caches S % 4 == 0
-        if st.quantized and cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0:
+        # the MFMA kernel (which carries the epilogue) streams 32-key tiles: rings need S % 32 == 0, linear int8 caches
+        # S % 4 == 0; it serves int8 caches and caches in the q dtype
+        mfma_cache = st.quantized or (st.k[l].dtype == q.dtype and q.dtype in (torch.float16, torch.bfloat16))
+        if mfma_cache and cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0 and S >= 32:
             out = b["zg"][off:off + n].view(n, cfg.n_heads, cfg.head_dim)
             decode_attention_post(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, vhat=b["vhat"][off:off + n],
                                   gate=None if W["attn_gate"] is None else b["gate"][off:off + n], xsa=W["xsa"], out=out, **kw)

@@ -30,10 +30,11 @@ def default_splits(n_bk: int, ctx: int, device=None, min_chunk: int = 256, waves
 
 def supported(q: Tensor, k_cache: Tensor) -> bool:
     """True when the MFMA kernel serves this geometry (reference: decode_attn_cuda.supported,
-    decode_attn_cuda.py:265-270).  Other geometries run the generic kernel."""
+    decode_attn_cuda.py:265-270): head_dim 64, up to 8 query heads per kv head, an int8 cache or one in the q dtype.  Other
+    geometries run the generic kernel."""
     H, hd = q.shape[-2], q.shape[-1]
     G = H // k_cache.shape[1]
-    return bool(q.is_cuda and hd == 64 and 1 <= G <= 8 and k_cache.dtype == torch.int8
+    return bool(q.is_cuda and hd == 64 and 1 <= G <= 8 and k_cache.dtype in (torch.int8, q.dtype)
                 and q.dtype in (torch.float16, torch.bfloat16))
 
 
@@ -193,7 +194,7 @@ def decode_attention_post(q: Tensor, k_cache: Tensor, v_cache: Tensor, pos: Tens
     """decode_attention followed by the reference's Attention.post up to the output projection (XSA with the
     unquantized current v, per-head sigmoid gate; ultraviolet/model.py:321-333) in the same kernel.  vhat (B, K, hd) fp32
     is v / max(|v|, eps) and gate (B, H) fp32 the gate values, both produced by the qkv_post kernel; out (B, H, hd) in
-    the activation dtype is written in place.  int8 cache, head_dim 64, one chunk per row."""
+    the activation dtype is written in place.  int8 cache or a cache in the q dtype, head_dim 64, one chunk per row."""
     L.require_cuda(q, k_cache, pos)
     if rows is not None:
         rows = rows.to(pos.dtype).contiguous()
