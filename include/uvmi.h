@@ -107,7 +107,8 @@ typedef struct uvmi_attn_args {
                                               decode_attn.py:42-44); > 0: chunks of at least this many keys, so short
                                               rows use fewer work items and a row that fits one chunk skips the combine */
   void* workspace; size_t workspace_bytes; /* >= uvmi_decode_attn_workspace_bytes(...) when num_splits > 1 */
-  /* Optional fused epilogue, used when post_vhat != NULL (needs head_dim 64, int8 cache, num_splits == 1): Attention.post
+  /* Optional fused epilogue, used when post_vhat != NULL (needs the MFMA kernel - head_dim 64, an int8 cache or one in
+   * the q dtype - and num_splits == 1): Attention.post
    * before the output projection (ultraviolet/model.py:321-333): XSA z -= xsa[h] (z . v_hat) v_hat with the unquantized
    * current v, then z *= 2 sigmoid(gate_w[h] . xn[:gate_ch]); out then holds that result in out_dtype. */
   const float* post_vhat;                  /* (B, KH, hd) fp32 normalized current v (uvmi_qkv_post vhat_out); enables the epilogue */
@@ -151,8 +152,9 @@ size_t uvmi_decode_attn_workspace_bytes(int B, int H, int KH, int hd, int num_sp
 /* default_splits (decode_attn.py:121-129) re-derived for 256 CUs x wave64: enough (row, kv head, split) work
  * items to fill the device, each chunk >= min_chunk keys, at most 64.  n_cus <= 0: query the current device. */
 int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus);
-/* 1 if uvmi_decode_attn runs the MFMA kernel for these arguments, 0 if the generic kernel (any hd <= 256,
- * G <= 16), negative if unsupported.  Mirrors decode_attn_cuda.supported (decode_attn_cuda.py:265-270). */
+/* 1 if uvmi_decode_attn runs the MFMA kernel for these arguments (head_dim 64, up to 8 query heads per kv head, an
+ * int8 cache with fp16 scales or a cache held unquantized in the q dtype, aligned rows), 0 if the generic kernel (any
+ * hd <= 256, G <= 16), negative if unsupported.  Mirrors decode_attn_cuda.supported (decode_attn_cuda.py:265-270). */
 int uvmi_decode_attn_path(const uvmi_attn_args* a);
 
 /* uvmi_decode_attn for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
