@@ -217,6 +217,33 @@ def test_backward_ragged_and_edges(dtype, lens, H, K, window):
         assert np.abs(a - b).max() <= 2 * ulp * max(np.abs(b).max(), 1e-3) + 1e-6, (np.abs(a - b).max(), np.abs(b).max())
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,K,window", [(8, 1, None), (8, 2, 256), (4, 1, 100), (16, 1, 64)])
+def test_backward_many_tiles_and_padding_tokens(dtype, H, K, window):
+    """Sequences of several 32-key tiles and 64-key workgroups (interior tiles take the unmasked path), a group of 16 heads
+    (beyond the matrix-core kernels' 8: the plain kernels), and 37 tokens past cu[-1]: padding, whose gradients are zero and
+    which no real key may see."""
+    from oracle.varlen_attn import varlen_attention_grad_ref
+    from ultraviolet_amd.kernels.varlen_attn import packed_attention, packed_attention_backward
+    lens, pad = [512, 700, 300, 5], 37
+    q, k, v, cu = _case(lens, H, K, 64, dtype, seed=11)
+    N = q.size(0)
+    gen = torch.Generator().manual_seed(12)
+    go = torch.randn(q.shape, generator=gen).to(dtype)
+    ext = lambda t: torch.cat([t, torch.randn(pad, *t.shape[1:], generator=gen).to(dtype)]).to(DEV)
+    qd, kd, vd, god = ext(q), ext(k), ext(v), ext(go)
+    o = packed_attention(qd, kd, vd, cu.to(DEV), SC, window)
+    dq, dk, dv = packed_attention_backward(god, qd, kd, vd, o, cu.to(DEV), SC, window)
+    torch.cuda.synchronize()
+    ref = varlen_attention_grad_ref(to_np(q), to_np(k), to_np(v), to_np(go), to_np(cu), SC, window)
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for a, b in zip((dq, dk, dv), ref):
+        a = to_np(a).astype(np.float64)
+        assert np.isfinite(a).all() and (a[N:] == 0).all()
+        assert np.abs(a[:N] - b).max() <= 2 * ulp * np.abs(b).max() + 1e-6, (np.abs(a[:N] - b).max(), np.abs(b).max())
+        assert np.linalg.norm(a[:N] - b) / np.linalg.norm(b) < (5e-3 if dtype == torch.float16 else 2e-2)
+
+
 def test_backward_rejects_what_it_cannot_do():
     from ultraviolet_amd import _lib as L
     from ultraviolet_amd.kernels.varlen_attn import packed_attention_backward

@@ -36,7 +36,7 @@ def _hipcc() -> str:
 def _stale(obj: str, src: str) -> bool:
     if not os.path.exists(obj):
         return True
-    deps = [src, os.path.join(HERE, "common.h"), os.path.join(HERE, "sched_commit.h"), os.path.join(HERE, "gemm_util.h"), os.path.join(HERE, "..", "..", "include", "uvmi.h"), __file__]
+    deps = [src, os.path.join(HERE, "common.h"), os.path.join(HERE, "sched_commit.h"), os.path.join(HERE, "gemm_util.h"), os.path.join(HERE, "attn_mfma_util.h"), os.path.join(HERE, "..", "..", "include", "uvmi.h"), __file__]
     return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps)
 
 

@@ -29,19 +29,12 @@
 // Everything else (fp32 K/V, other head dims) goes token by token through the decode kernel's generic path with the
 // packed K/V as a batch-stride-0 "cache".
 #include "common.h"
+#include "attn_mfma_util.h"
 
 #include <climits>
 #include <type_traits>
 
 namespace uvmi {
-
-typedef _Float16 ph8 __attribute__((ext_vector_type(8)));
-typedef _Float16 ph2 __attribute__((ext_vector_type(2)));
-typedef __bf16 pb8 __attribute__((ext_vector_type(8)));
-typedef __bf16 pb2 __attribute__((ext_vector_type(2)));
-typedef float pf4 __attribute__((ext_vector_type(4)));
-typedef unsigned int pu4 __attribute__((ext_vector_type(4)));
-typedef unsigned int pu2 __attribute__((ext_vector_type(2)));
 
 struct PrefillParams {
   const void* q; const void* k; const void* v; void* out;
@@ -51,6 +44,7 @@ struct PrefillParams {
   int n_wg;                        // workgroups with work: ceil(query blocks / (4 / n_hg)) * KH
   float scale_log2;
   const float* post_vhat; const float* post_gate; const float* post_xsa;  // fused Attention.post epilogue when post_vhat != null
+  float* lse_out; int64_t lse_stride;  // optional (H, lse_stride) fp32: log2 of each row's sum of exp2(scale_log2 s) (the backward's statistics)
 };
 
 // seg_start[i] = cu[s] for the last s with cu[s] <= i (empty sequences are skipped); pidx[i] = i.
@@ -64,51 +58,6 @@ __global__ __launch_bounds__(256) void prefill_segments(const void* cu, int idx6
   }
   seg_start[i] = (int32_t)load_index(cu, idx64, lo);
   pidx[i] = i;
-}
-
-template <int DT>
-__device__ __forceinline__ pf4 mfma16(pu4 a, pu4 b, pf4 c) {
-  if constexpr (DT == UVMI_F16) {
-    ph8 x, y;
-    __builtin_memcpy(&x, &a, 16);
-    __builtin_memcpy(&y, &b, 16);
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, c, 0, 0, 0);
-  } else {
-    pb8 x, y;
-    __builtin_memcpy(&x, &a, 16);
-    __builtin_memcpy(&y, &b, 16);
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, c, 0, 0, 0);
-  }
-}
-
-template <int DT>
-__device__ __forceinline__ uint32_t pack2(float a, float b) {  // two fp32 -> one dword of 16-bit values, round to nearest even
-  uint32_t r;
-  if constexpr (DT == UVMI_F16) {
-    const ph2 v = ph2{(_Float16)a, (_Float16)b};
-    __builtin_memcpy(&r, &v, 4);
-  } else {
-    const pb2 v = pb2{(__bf16)a, (__bf16)b};
-    __builtin_memcpy(&r, &v, 4);
-  }
-  return r;
-}
-
-__device__ __forceinline__ float pmax16(float v) {
-  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float pmax32(float v) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float psum16(float v) {
-  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-__device__ __forceinline__ float psum32(float v) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 struct PTile {   // one 32-key super-tile as loaded (32 dwords per lane)
@@ -336,6 +285,9 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_hd64(PrefillParams P) {
     const int hq = hg * HPW + hh;
     const float l = psum32(psum16(lrun[hh]));
     const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (P.lse_out && g == 0 && hq < G && row_ok)   // (+inf for a row without keys: its probabilities come out as 0)
+      P.lse_out[(int64_t)(kvh * G + hq) * P.lse_stride + row] = l > 0.f ? mrun[hh] * c + __builtin_amdgcn_logf(l) : INFINITY;
+    if (P.out == nullptr) continue;   // statistics only
     float o[16];
 #pragma unroll
     for (int t = 0; t < 4; t++)
@@ -398,6 +350,17 @@ static int check_prefill(const uvmi_prefill_attn_args* a) {
   return UVMI_OK;
 }
 
+static bool prefill_mfma_ok_stats(const uvmi_prefill_attn_args* a) {   // (as below, without an output tensor)
+  if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype) return false;
+  if (!(a->scale > 0.f)) return false;
+  auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
+  if (!al(a->q, 16) || a->sqn % 8 || a->sqh % 8) return false;
+  if (!al(a->k, 16) || a->skn % 8 || a->skh % 8 || !al(a->v, 16) || a->svn % 8 || a->svh % 8) return false;
+  if (a->skn <= 0 || a->svn <= 0) return false;
+  if ((int64_t)a->N * a->skn * 2 >= (1LL << 31) || (int64_t)a->N * a->svn * 2 >= (1LL << 31)) return false;
+  return true;
+}
+
 static bool prefill_mfma_ok(const uvmi_prefill_attn_args* a) {
   if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype) return false;
   if (!(a->scale > 0.f)) return false;  // the running maximum is tracked before the (positive) softmax scale
@@ -409,6 +372,48 @@ static bool prefill_mfma_ok(const uvmi_prefill_attn_args* a) {
   const int ob = a->out_dtype == UVMI_F32 ? 4 : 2;
   if (!al(a->out, 16) || (a->son * ob) % 16 || (a->soh * ob) % 16) return false;
   return true;
+}
+
+static int launch_mfma(const uvmi_prefill_attn_args* a, const int32_t* seg_start, float* lse_out, int64_t lse_stride, hipStream_t st) {
+  PrefillParams P;
+  P.q = a->q; P.k = a->k; P.v = a->v; P.out = a->out; P.seg_start = seg_start;
+  P.sqn = a->sqn; P.sqh = a->sqh; P.skn = a->skn; P.skh = a->skh; P.svn = a->svn; P.svh = a->svh; P.son = a->son; P.soh = a->soh;
+  P.N = a->N; P.H = a->H; P.KH = a->KH; P.G = a->H / a->KH; P.window = a->window;
+  P.n_hg = (P.G + HPW - 1) / HPW;   // 1 or 2 (G <= 8)
+  const int64_t n_qb = (a->N + 15) / 16, qbw = 4 / P.n_hg;
+  const int64_t n_wg = (n_qb + qbw - 1) / qbw * a->KH;
+  P.scale_log2 = a->scale * 1.4426950408889634f;
+  P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa;
+  P.lse_out = lse_out; P.lse_stride = lse_stride;
+  UVMI_REQUIRE(n_wg < (1LL << 30), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: too many work items");
+  P.n_wg = (int)n_wg;
+  const unsigned nblk = (unsigned)((n_wg + 7) / 8 * 8);
+  const dim3 grid(nblk), blk(256);
+  const int od = a->out_dtype;
+#define UVMI_L(QD)                                                                                                \
+  do {                                                                                                            \
+    if (od == UVMI_F16) hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_F16>), grid, blk, 0, st, P);          \
+    else if (od == UVMI_BF16) hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_BF16>), grid, blk, 0, st, P);   \
+    else hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_F32>), grid, blk, 0, st, P);                         \
+  } while (0)
+  if (a->q_dtype == UVMI_F16) UVMI_L(UVMI_F16); else UVMI_L(UVMI_BF16);
+#undef UVMI_L
+  UVMI_CHECK_LAUNCH("uvmi_prefill_attn");
+  return UVMI_OK;
+}
+
+// For the backward (prefill_attn_bwd.hip): the segment table of cu_seqlens into seg_start (N ints; pidx: N ints of scratch) and
+// the rows' softmax statistics into lse (H, lse_stride), from one forward pass that stores no output.  a->out may be null.
+int prefill_attn_stats(const uvmi_prefill_attn_args* a, int32_t* seg_start, int32_t* pidx, float* lse, int64_t lse_stride, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(prefill_segments, dim3((unsigned)((a->N + 255) / 256)), dim3(256), 0, st, a->cu_seqlens, a->idx_dtype == UVMI_I64 ? 1 : 0,
+                     a->n_seg, a->N, seg_start, pidx);
+  UVMI_CHECK_LAUNCH("uvmi_prefill_attn_bwd(segments)");
+  uvmi_prefill_attn_args b = *a;
+  b.out = nullptr; b.out_dtype = a->q_dtype; b.son = (int64_t)a->H * 64; b.soh = 64;
+  b.post_vhat = nullptr; b.post_gate = nullptr; b.post_xsa = nullptr;
+  UVMI_REQUIRE(prefill_mfma_ok_stats(&b), UVMI_EUNSUPPORTED, "uvmi_prefill_attn_bwd: q / k / v layout not served by the MFMA kernels");
+  return launch_mfma(&b, seg_start, lse, lse_stride, st);
 }
 
 }  // namespace uvmi
@@ -454,28 +459,6 @@ extern "C" int uvmi_prefill_attn(const uvmi_prefill_attn_args* a, void* stream) 
     d.scale = a->scale; d.window = a->window; d.ring = 0; d.num_splits = 1;
     return uvmi_decode_attn(&d, stream);
   }
-  PrefillParams P;
-  P.q = a->q; P.k = a->k; P.v = a->v; P.out = a->out; P.seg_start = seg_start;
-  P.sqn = a->sqn; P.sqh = a->sqh; P.skn = a->skn; P.skh = a->skh; P.svn = a->svn; P.svh = a->svh; P.son = a->son; P.soh = a->soh;
-  P.N = a->N; P.H = a->H; P.KH = a->KH; P.G = a->H / a->KH; P.window = a->window;
-  P.n_hg = (P.G + HPW - 1) / HPW;   // 1 or 2 (G <= 8)
-  const int64_t n_qb = (a->N + 15) / 16, qbw = 4 / P.n_hg;
-  const int64_t n_wg = (n_qb + qbw - 1) / qbw * a->KH;
-  P.scale_log2 = a->scale * 1.4426950408889634f;
-  P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa;
-  UVMI_REQUIRE(n_wg < (1LL << 30), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: too many work items");
-  P.n_wg = (int)n_wg;
-  const unsigned nblk = (unsigned)((n_wg + 7) / 8 * 8);
-  const dim3 grid(nblk), blk(256);
-  const int od = a->out_dtype;
-#define UVMI_L(QD)                                                                                                \
-  do {                                                                                                            \
-    if (od == UVMI_F16) hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_F16>), grid, blk, 0, st, P);          \
-    else if (od == UVMI_BF16) hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_BF16>), grid, blk, 0, st, P);   \
-    else hipLaunchKernelGGL((prefill_attn_mfma_hd64<QD, UVMI_F32>), grid, blk, 0, st, P);                         \
-  } while (0)
-  if (a->q_dtype == UVMI_F16) UVMI_L(UVMI_F16); else UVMI_L(UVMI_BF16);
-#undef UVMI_L
-  UVMI_CHECK_LAUNCH("uvmi_prefill_attn");
-  return UVMI_OK;
+  return launch_mfma(a, seg_start, nullptr, 0, st);
 }
+
