@@ -386,6 +386,20 @@ def bench_c4(args):
         e1.record()
         torch.cuda.synchronize()
         phases[name] = round(e0.elapsed_time(e1) * 1e3 / 20, 1)
+    # the backward of the same packed attention (the trainer side's first kernel): output gradient -> dq, dk, dv
+    from ultraviolet_amd.kernels.varlen_attn import packed_attention_backward
+    go = torch.randn(N, cfg.n_heads, cfg.head_dim, device=dev, generator=gen).to(torch.bfloat16)
+    qc, kc, vc = (b[n_][:N].contiguous() for n_ in ("q", "k", "v"))
+    for name, w in (("prefill_attn_bwd_global_us", 0), ("prefill_attn_bwd_local_us", cfg.window)):
+        o = packed_attention(qc, kc, vc, pk["cu"], cfg.attn_scale, w)
+        for _ in range(3):
+            packed_attention_backward(go, qc, kc, vc, o, pk["cu"], cfg.attn_scale, w)
+        e0.record()
+        for _ in range(10):
+            packed_attention_backward(go, qc, kc, vc, o, pk["cu"], cfg.attn_scale, w)
+        e1.record()
+        torch.cuda.synchronize()
+        phases[name] = round(e0.elapsed_time(e1) * 1e3 / 10, 1)
     fl_g = 4 * 8 * 64 * npf * (512 * 513 // 2)
     fl_l = 4 * 8 * 64 * npf * (512 * 256 - 256 * 255 // 2)
     ntok = N + nd
@@ -396,7 +410,9 @@ def bench_c4(args):
                                              "fused) packed with 448 decode rows, contexts U{256..2048}; one forward pass per step, eager launches",
                                  "token_rows": ntok, "wall_ms_per_step": round(wall * 1e3 / it, 4), **phases,
                                  "prefill_attn_global_TFLOPs": round(fl_g / phases["prefill_attn_global_us"] / 1e6, 1),
-                                 "prefill_attn_local_TFLOPs": round(fl_l / phases["prefill_attn_local_us"] / 1e6, 1)}}))
+                                 "prefill_attn_local_TFLOPs": round(fl_l / phases["prefill_attn_local_us"] / 1e6, 1),
+                                 "prefill_attn_bwd_global_TFLOPs": round(2.5 * fl_g / phases["prefill_attn_bwd_global_us"] / 1e6, 1),
+                                 "prefill_attn_bwd_local_TFLOPs": round(2.5 * fl_l / phases["prefill_attn_bwd_local_us"] / 1e6, 1)}}))
 
 
 def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0):
