@@ -78,15 +78,16 @@ def test_fp32_engine_matches_oracle_logits_and_cache():
 
 def test_first_layer_cache_is_bit_exact():
     """Layer 0 sees only embedding -> norm -> QKV GEMM -> QK-norm / RoPE before the quantizer; with fp32 GEMMs its int8
-    bytes and fp16 scales must equal the oracle's almost everywhere (GEMM summation order can flip a tie)."""
+    bytes and fp16 scales must equal the oracle's (GEMM summation order can flip a tie: none does on this case)."""
     cfg, params, eng, OracleModel = _setup(window=16)
     prompts = _prompts(cfg, (16, 16, 16, 16), seed=3)
     cont = np.random.default_rng(4).integers(1, cfg.vocab_size, size=(4, 8))
     _, st = _teacher_forced(eng, prompts, cont, 32)
     _, ost = _oracle_teacher_forced(OracleModel(cfg, params, torch.float32), prompts, cont, 32)
     k = st.k[0].cpu().numpy()
-    assert (k != ost.k[0]).mean() < 2e-3
-    assert (st.k_scale[0].cpu().numpy().view(np.uint16) != ost.ks[0].view(np.uint16)).mean() < 2e-2
+    dk, ds = (k != ost.k[0]).mean(), (st.k_scale[0].cpu().numpy().view(np.uint16) != ost.ks[0].view(np.uint16)).mean()
+    # measured: no differing code, no differing scale; the bars leave room for one flipped round-half-even tie per 10^4 codes
+    assert dk <= 1e-4 and ds <= 1e-3, (dk, ds)
 
 
 @pytest.mark.parametrize("name,over", [("uv-test", dict(window=16)), ("uv-50m-alpha", dict())])
