@@ -194,7 +194,7 @@ def test_checkpoint_with_unsupported_layers_is_refused():
 
 
 def test_integration_doc_stub_matches_the_binding():
-    """The maintainer's stub printed in INTEGRATION.md is executed as far as its declarations go (ctypes.CDLL replaced by
+    """The maintainer's stub printed in the integration notes at the repository root is executed as far as its declarations go (ctypes.CDLL replaced by
     the loaded library) and compared with ultraviolet_amd/_lib.py: same dtype codes, same structure, same layout."""
     import torch
     from ultraviolet_amd import _lib
