@@ -713,7 +713,8 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   // ---- reduce l and sum P' over the 4 lane groups, merge stream B into stream A (lanes n and n^8), undo the bias
   float lsum = xsum32(xsum16(st.lrun)), ps = xsum32(xsum16(st.psum));
   const float m2 = st.mrun == -INFINITY ? -INFINITY : st.mrun * c;  // exp2 domain
-  const float m_o = __shfl_xor(m2, 8, 64), l_o = __shfl_xor(lsum, 8, 64), ps_o = __shfl_xor(ps, 8, 64);
+  // (lane ^ 8 is a rotation by 8 inside a row of 16 lanes: a DPP move on the vector ALU, where __shfl_xor would go through the LDS crossbar)
+  const float m_o = dpp_mov<0x128>(m2), l_o = dpp_mov<0x128>(lsum), ps_o = dpp_mov<0x128>(ps);
   const float mm = fmaxf(m2, m_o);
   const float ms = mm == -INFINITY ? 0.f : mm;
   const float w_s = __builtin_amdgcn_exp2f(m2 - ms), w_o = __builtin_amdgcn_exp2f(m_o - ms);
@@ -726,7 +727,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const float mine = st.O[t][i];
-      const float oth = __shfl_xor(mine, 8, 64);
+      const float oth = dpp_mov<0x128>(mine);
       o[4 * i + t] = (mine * w_s24 + oth * w_o24) - pm;
     }
   float mfin = mm, lfin = lm;
