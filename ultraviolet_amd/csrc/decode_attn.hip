@@ -90,13 +90,22 @@ __device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b, bool own
   r.a0 = lo & ~31;
   int span = p + 1 - r.a0;
   if (span < 0) span = 0;
-  const int gr = P.gran;  // multiple of 32
-  int chunk = (((span + P.splits - 1) / P.splits) + gr - 1) / gr * gr;
+  // (integer divisions by run-time values cost a few dozen instructions each, here on the way to the row's first tile
+  // request: the granule is a power of two, and an uncut row - every decode step of the engine - divides by nothing)
+  const int gr = P.gran;  // 32, 64 or 128
+  const int per = P.splits == 1 ? span : (int)(((uint32_t)span + (uint32_t)P.splits - 1u) / (uint32_t)P.splits);
+  int chunk = (per + gr - 1) & ~(gr - 1);
   if (chunk < P.chunk_keys) chunk = P.chunk_keys;
   if (chunk < gr) chunk = gr;
   r.chunk = chunk;
-  r.nsplit = span > 0 ? (span + chunk - 1) / chunk : 1;
+  r.nsplit = span > chunk ? (int)(((uint32_t)span + (uint32_t)chunk - 1u) / (uint32_t)chunk) : 1;
   return r;
+}
+
+// Cache slot of position t >= 0: t itself, or t mod S on a ring (a mask when S is a power of two, as every window is).
+__device__ __forceinline__ int ring_slot(const AttnParams& P, int t) {
+  if (!P.ring) return t;
+  return (P.S & (P.S - 1)) == 0 ? (t & (P.S - 1)) : (int)((uint32_t)t % (uint32_t)P.S);
 }
 
 // ---------------------------------------------------------------------------------------------------- MFMA kernel
@@ -223,9 +232,12 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     if (WPR == 1) return;
     item = P.n_items - 1;  // keep the wave for the barrier below; it does no work
   }
-  const int sid = (int)(item % P.splits);
-  const int64_t bk = item / P.splits;
-  const int b = __builtin_amdgcn_readfirstlane((int)(bk / P.KH)), h = __builtin_amdgcn_readfirstlane((int)(bk % P.KH));
+  // (items fit 31 bits, host-checked; one split and one kv head - the engine's shape - need no division)
+  const uint32_t it32 = (uint32_t)item;
+  const int sid = P.splits == 1 ? 0 : (int)(it32 % (uint32_t)P.splits);
+  const uint32_t bk = P.splits == 1 ? it32 : it32 / (uint32_t)P.splits;
+  const int b = __builtin_amdgcn_readfirstlane((int)(P.KH == 1 ? bk : bk / (uint32_t)P.KH));
+  const int h = __builtin_amdgcn_readfirstlane((int)(P.KH == 1 ? 0u : bk % (uint32_t)P.KH));
   const int m = lane & 15, g = lane >> 4;  // A/B operand (row, group) == accumulator (column, group)
   const int strm = m >> 3, head = m & 7;
   const int G = P.G;
@@ -381,7 +393,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     }
     uint16_t sbk;
     const float kq = quant1(k, sbk);
-    const int slot = P.ring ? rp.pc % P.S : rp.pc;
+    const int slot = ring_slot(P, rp.pc);
     if (slot < P.S) {
       ((int8_t*)P.kc)[(int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + lane] = (int8_t)(int)kq;
       if (lane == 0) ((uint16_t*)P.ks)[(int64_t)rp.cb * P.ssb + (int64_t)h * P.ssh + slot] = sbk;
@@ -413,7 +425,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     const float nv = fmaxf(sqrtf(bfly_sum(v * v)), P.f_xsa_eps);
     uint16_t sbv;
     const float vq = quant1(v, sbv);
-    const int slot = P.ring ? rp.pc % P.S : rp.pc;
+    const int slot = ring_slot(P, rp.pc);
     if (slot < P.S) {
       ((int8_t*)P.vc)[(int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + lane] = (int8_t)(int)vq;
       if (lane == 0) ((uint16_t*)P.vs)[(int64_t)rp.cb * P.stb + (int64_t)h * P.sth + slot] = sbv;
@@ -642,7 +654,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     const int s1f = P.ring ? s1 : min(s1, S & ~31);
     int tb = s0 + 32 * wsub;
     const bool has = tb < s1f;
-    int slot = has ? (P.ring ? tb % S : tb) : 0;
+    int slot = has ? ring_slot(P, tb) : 0;
     auto next_slot = [&](int sl, int t) {
       if (t + STEP >= s1f) return sl;
       sl += STEP;
