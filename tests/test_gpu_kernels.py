@@ -648,3 +648,37 @@ def test_skinny_gemm_norm_and_resid_fusions(dtype, M, K, N):
         for config in (1, 2, 3, 4, 0):
             act = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU, norm_eps=eps, config=config)
             assert bool(((act.double() - ra).abs() <= tol3).all()), (config, float((act.double() - ra).abs().max()))
+
+
+@pytest.mark.gpu
+def test_tiled_gemm_at_prefill_row_counts():
+    """The projections of a packed prefill pass at its size (33 216 rows, the mixed-batch config): gate-up with the pre-norm
+    and SwiGLU, and the output projection with the residual update in place, on both tile shapes and on the shape the
+    library picks, against float64 - thousands of tiles per XCD run, row and column tails (33 216 = 259.5 x 128)."""
+    from ultraviolet_amd.kernels.gemm import RESID, SWIGLU, gemm_tn, interleave_gate_up
+    dtype, M, K, f = torch.bfloat16, 33216, 640, 1664
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = (torch.randn(M, K, device="cuda", generator=g) * 2).to(dtype)
+    wg = (torch.randn(f, K, device="cuda", generator=g) / K ** 0.5).to(dtype)
+    wu = (torch.randn(f, K, device="cuda", generator=g) / K ** 0.5).to(dtype)
+    ulp, eps = 2.0 ** -8, 1e-6
+    ad = a.double()
+    an = ad * torch.rsqrt((ad * ad).mean(-1, keepdim=True) + eps)
+    gg = (an @ wg.double().t()).to(dtype).double()
+    uu = (an @ wu.double().t()).to(dtype).double()
+    ra = (gg * torch.sigmoid(gg)).to(dtype).double() * uu
+    tol = 4 * ulp * ra.abs().clamp_min(1.0) + 4 * ulp * (gg.abs() + uu.abs())
+    del an
+    for config in (3, 4, 0):
+        act = gemm_tn(a, interleave_gate_up(wg, wu), epilogue=SWIGLU, norm_eps=eps, config=config)
+        assert bool(((act.double() - ra).abs() <= tol).all()), (config, float((act.double() - ra).abs().max()))
+    del gg, uu, ra, tol
+    z = (torch.randn(M, 512, device="cuda", generator=g)).to(dtype)
+    wo = (torch.randn(K, 512, device="cuda", generator=g) / 512 ** 0.5).to(dtype)
+    prod = (z.double() @ wo.double().t()).to(dtype).double()
+    want = 0.75 * a.double() + 1.25 * prod
+    tol2 = ulp * want.abs().clamp_min(1.0) + 1.25 * 2 * ulp * prod.abs().clamp_min(1.0)
+    for config in (3, 4, 0):
+        x = a.clone()
+        gemm_tn(z, wo, x, epilogue=RESID, resid=x, ca=0.75, cb=1.25, config=config)
+        assert bool(((x.double() - want).abs() <= tol2).all()), (config, float((x.double() - want).abs().max()))
