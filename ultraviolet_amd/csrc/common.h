@@ -120,12 +120,56 @@ __device__ __forceinline__ float rope_rot(float x, float y, float c, float s, bo
 template <class R>
 __device__ __forceinline__ float ve_add(float v, float g, float e, R rnd) { return rnd(add_sep(v, rnd(mul_sep(g, e)))); }
 
+// ---- cross-lane exchanges of a wave64 without the LDS crossbar where the hardware has another way: lanes l ^ 32 and l ^ 16 by
+// the permlane swaps, l ^ 8 as a rotation inside a row of 16 (DPP), l ^ 4 by ds_swizzle, l ^ 2 and l ^ 1 as quad permutes (DPP)
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_mov_dpp((int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_xor1(float v) { return dpp_mov<0xb1>(v); }   // quad_perm [1, 0, 3, 2]
+__device__ __forceinline__ float lane_xor2(float v) { return dpp_mov<0x4e>(v); }   // quad_perm [2, 3, 0, 1]
+__device__ __forceinline__ float lane_xor4(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_ds_swizzle((int)__float_as_uint(v), 0x101f));
+}
+__device__ __forceinline__ float lane_xor8(float v) { return dpp_mov<0x128>(v); }  // row_ror:8
+__device__ __forceinline__ float lane_xor16(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_ds_swizzle((int)__float_as_uint(v), 0x401f));
+}
+__device__ __forceinline__ float xmax16(float v) {  // max over lanes l, l ^ 16
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xmax32(float v) {  // max over lanes l, l ^ 32
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// (the sums below add with contraction off: a reduction's first step must not fuse with the multiply that produced its
+// argument - wave_sum(k * k) sums rounded squares wherever it is written)
+__device__ __forceinline__ float xsum16(float v) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return add_sep(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xsum32(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return add_sep(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// Butterfly reductions over the 64 lanes, pairing lane ^ 32, 16, 8, 4, 2, 1 in that order: every kernel that sums or maximises
+// over a wave goes through these, so that the same values round the same way wherever they are reduced.
 __device__ __forceinline__ float wave_max(float v) {
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  v = xmax32(v);
+  v = xmax16(v);
+  v = fmaxf(v, lane_xor8(v));
+  v = fmaxf(v, lane_xor4(v));
+  v = fmaxf(v, lane_xor2(v));
+  v = fmaxf(v, lane_xor1(v));
   return v;
 }
 __device__ __forceinline__ float wave_sum(float v) {
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  v = xsum32(v);
+  v = xsum16(v);
+  v = add_sep(v, lane_xor8(v));
+  v = add_sep(v, lane_xor4(v));
+  v = add_sep(v, lane_xor2(v));
+  v = add_sep(v, lane_xor1(v));
   return v;
 }
 

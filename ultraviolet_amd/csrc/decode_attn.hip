@@ -118,53 +118,10 @@ __device__ __forceinline__ h8 as_h8(uint32_t a, uint32_t b, uint32_t c, uint32_t
   return v;
 }
 
-__device__ __forceinline__ float xmax16(float v) {  // max over lanes l, l^16
-  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float xmax32(float v) {  // max over lanes l, l^32
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float xsum16(float v) {
-  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-__device__ __forceinline__ float xsum32(float v) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-// Butterfly reductions over the 64 lanes with the pairing order of wave_sum / wave_max (lane ^ 32, 16, 8, 4, 2, 1), so
-// that a sum formed here rounds exactly as the one in the standalone post-processing kernel; the steps use the lane-swap,
-// DPP and swizzle forms instead of six LDS permutes.
-__device__ __forceinline__ float lane_xor16(float v) {  // value of lane l ^ 16
-  return __uint_as_float((uint32_t)__builtin_amdgcn_ds_swizzle((int)__float_as_uint(v), 0x401f));
-}
-template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
-  return __uint_as_float((uint32_t)__builtin_amdgcn_mov_dpp((int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float lane_xor4(float v) {
-  return __uint_as_float((uint32_t)__builtin_amdgcn_ds_swizzle((int)__float_as_uint(v), 0x101f));
-}
-__device__ __forceinline__ float bfly_sum(float v) {
-  v = xsum32(v);
-  v = xsum16(v);
-  v += dpp_mov<0x128>(v);  // row_ror:8 == lane ^ 8 inside a row of 16
-  v += lane_xor4(v);
-  v += dpp_mov<0x4e>(v);   // quad_perm [2, 3, 0, 1] == lane ^ 2
-  v += dpp_mov<0xb1>(v);   // quad_perm [1, 0, 3, 2] == lane ^ 1
-  return v;
-}
-__device__ __forceinline__ float bfly_max(float v) {
-  v = xmax32(v);
-  v = xmax16(v);
-  v = fmaxf(v, dpp_mov<0x128>(v));
-  v = fmaxf(v, lane_xor4(v));
-  v = fmaxf(v, dpp_mov<0x4e>(v));
-  v = fmaxf(v, dpp_mov<0xb1>(v));
-  return v;
-}
+// (the lane exchanges and the 64-lane butterflies - pairing lane ^ 32, 16, 8, 4, 2, 1, the order every kernel of this library
+// reduces in - live in common.h)
+__device__ __forceinline__ float bfly_sum(float v) { return wave_sum(v); }
+__device__ __forceinline__ float bfly_max(float v) { return wave_max(v); }
 
 struct Tile {             // one 32-key super-tile as loaded from HBM (26 dwords per lane)
   uint4 kA, kB;           // key m of stream A / B, bytes 16g..16g+15

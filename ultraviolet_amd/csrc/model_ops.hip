@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       float ss = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; j++) ss += x[j] * x[j];
-      ss += __shfl_xor(ss, 1, 64); ss += __shfl_xor(ss, 2, 64); ss += __shfl_xor(ss, 4, 64);
+      ss += lane_xor1(ss); ss += lane_xor2(ss); ss += lane_xor4(ss);
       const float rs = rsqrtf(ss * (1.0f / 64.0f) + A.eps);
 #pragma unroll
       for (int j = 0; j < 8; j++) x[j] = round_t<DT>(x[j] * rs);
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
         const bool first = 8 * c < np_, rot = 8 * c < 2 * np_;
         float y[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) y[j] = __shfl_xor(x[j], pl, 64);  // partner chunk: c <-> c ^ pl inside the head
+        for (int j = 0; j < 8; j++) y[j] = pl == 2 ? lane_xor2(x[j]) : __shfl_xor(x[j], pl, 64);  // partner chunk: c <-> c ^ pl inside the head
         if (rot) {
 #pragma unroll
           for (int j = 0; j < 8; j++) x[j] = rope_rot(x[j], y[j], cs[j], sn[j], first, [](float f) { return round_t<DT>(f); });
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
             for (int j = 0; j < cpl; j++) dot += elem<DT>::ld(A.xn, r * A.d + c * cpl + j) * A.gate_w[h * A.gate_ch + c * cpl + j];
           }
         }
-        dot += __shfl_xor(dot, 1, 64); dot += __shfl_xor(dot, 2, 64); dot += __shfl_xor(dot, 4, 64);
+        dot += lane_xor1(dot); dot += lane_xor2(dot); dot += lane_xor4(dot);
         dot = round_t<DT>(dot);
         if (h < A.H && c == 0) A.gate_out[r * A.H + h] = round_t<DT>(2.0f * round_t<DT>(1.0f / (1.0f + __expf(-dot))));
       }
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       const float rs = rsqrtf(wave_sum(k * k) * (1.0f / 64.0f) + A.eps);
       k = round_t<DT>(k * rs);
       if (A.rope) {
-        const float other = __shfl_xor(k, np_, 64);
+        const float other = np_ == 16 ? lane_xor16(k) : __shfl_xor(k, np_, 64);
         if (rot1) k = rope_rot(k, other, cs1, sn1, lane < np_, [](float f) { return round_t<DT>(f); });
       }
     }
