@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const void* a_a, const
 #pragma unroll
       for (int t = 0; t < 4; t++) {
         const float gv = ground<DT>(gt[t]), uv = ground<DT>(up[t]);
-        o[t] = ground<DT>(gv / (1.0f + __expf(-gv))) * uv;
+        o[t] = silu_round<DT>(gv) * uv;
       }
       uint16_t* cp = (uint16_t*)P.c + (int64_t)arow * P.ldc + (n0 >> 1) + 4 * g;
       *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_ksplit_kernel(const void* a_a
 #pragma unroll
       for (int t = 0; t < 4; t++) {
         const float gv = ground<DT>(gt[t]), uv = ground<DT>(up[t]);
-        o[t] = ground<DT>(gv / (1.0f + __expf(-gv))) * uv;
+        o[t] = silu_round<DT>(gv) * uv;
       }
       uint16_t* cp = (uint16_t*)a_c + (int64_t)arow * a_ldc + (n0 >> 1) + 4 * g;
       *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};

@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(TileParams P) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
           const float gv = ground<DT>(acc[i][j][t] * rn), uv = ground<DT>(acc[i][j + 1][t] * rn);
-          o[t] = ground<DT>(gv / (1.0f + __expf(-gv))) * uv;
+          o[t] = silu_round<DT>(gv) * uv;
         }
         uint16_t* cp = (uint16_t*)P.c + (int64_t)row * P.ldc + (n >> 1) + 4 * g;
         *(uint2*)cp = uint2{gpack<DT>(o[0], o[1]), gpack<DT>(o[2], o[3])};

@@ -29,6 +29,13 @@ template <int DT> __device__ __forceinline__ float ground(float v) {
   if constexpr (DT == UVMI_F16) return (float)(half_t)v;
   else return bf16_to_float(float_to_bf16(v));
 }
+// silu(g) rounded to the activation type, for a g already on that type's grid.  bf16 divides through the hardware reciprocal
+// (1 ulp in fp32, ahead of a rounding to 8 bits), as the standalone SwiGLU kernel does: a full IEEE division is ten
+// instructions per element of the gate-up epilogue.
+template <int DT> __device__ __forceinline__ float silu_round(float gv) {
+  if constexpr (DT == UVMI_BF16) return ground<DT>(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
+  else return ground<DT>(gv / (1.0f + __expf(-gv)));
+}
 template <int DT> __device__ __forceinline__ uint32_t gpack(float a, float b) {
   const uint32_t lo = DT == UVMI_BF16 ? float_to_bf16(a) : float_to_half_bits(a);
   const uint32_t hi = DT == UVMI_BF16 ? float_to_bf16(b) : float_to_half_bits(b);
