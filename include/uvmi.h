@@ -174,11 +174,13 @@ int uvmi_decode_attn_noalloc(const uvmi_attn_args* a, void* stream);
  * 16-bit GEMM of a decode step's projections: C (M, N) = A (M, K) . W (N, K)^T, fp32 accumulation, A, W, C in `dtype`
  * (F16 / BF16), rows contiguous with pitches lda, ldw, ldc (elements).  Replaces the F.linear calls of the reference's
  * fused inference path (ultraviolet/model.py:302-335 attention projections, 388-391 MLP).  K % 64 == 0, K <= 8192;
- * N % 16 == 0.  Two kernel families behind one entry point:
+ * N % 16 == 0.  Three kernel families behind one entry point:
  *   - skinny forms for steps of up to a few hundred rows, where the weights are the traffic: a workgroup requests its
  *     whole weight strip and its activation rows in one burst (K <= 1984; 960 with SWIGLU);
  *   - a tiled form (128 x 128 or 64 x 64 tiles, operand slabs double-buffered in LDS behind a ring of slabs in flight)
- *     for steps of several hundred to a few thousand rows, where the product is bound by feeding the matrix cores.
+ *     for steps of several hundred to a few thousand rows, where the product is bound by feeding the matrix cores;
+ *   - a 256 x 256 tile form (slabs loaded from global memory straight into LDS, 128 x 64 per wave) for the passes of many
+ *     thousand rows - a packed prefill, a mixed prefill + decode pass - where L2 and LDS bandwidth per flop decide.
  * epilogue UVMI_GEMM_SWIGLU (N % 32 == 0): W holds w_gate and w_up interleaved in slabs of 16 rows ([gate 0..15 |
  * up 0..15 | gate 16..31 | ...], N = 2 f rows) and C (M, f) = silu(A w_gate^T) * (A w_up^T) with the roundings of the
  * separate SwiGLU pass (model.py:388-391).
@@ -205,7 +207,8 @@ typedef struct uvmi_gemm_args {
   const void* resid; int64_t ldr; float ca, cb;
   int config;                              /* 0: built-in choice of the kernel form by size; 1: skinny, 64-row workgroups; 2: skinny,
                                               16-row workgroups whose waves split K (needs K % 128 == 0, else form 1); 3: tiled,
-                                              128 x 128; 4: tiled, 64 x 64 - for tuning and tests */
+                                              128 x 128; 4: tiled, 64 x 64; 5: 256 x 256 tiles (needs K >= 128, C and resid
+                                              16-byte aligned, ldc, ldr % 8 == 0) - for tuning and tests */
 } uvmi_gemm_args;
 int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream);
 

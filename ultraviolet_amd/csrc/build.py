@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["common.hip", "kv_quant.hip", "decode_attn.hip", "fused_sample.hip", "sched.hip", "model_ops.hip",
-           "prefill_attn.hip", "prefill_attn_bwd.hip", "gemm.hip", "gemm_tile.hip"]
+           "prefill_attn.hip", "prefill_attn_bwd.hip", "gemm.hip", "gemm_tile.hip", "gemm_big.hip"]
 LIB = os.path.join(HERE, "libuvmi.so")
 ARCH = "gfx950"
 FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",

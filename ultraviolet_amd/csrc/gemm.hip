@@ -370,10 +370,24 @@ __global__ __launch_bounds__(256) void gemm_skinny_ksplit_kernel(const void* a_a
 
 using namespace uvmi;
 
-namespace uvmi { void gemm_tile_launch(const uvmi_gemm_args* a, bool big, hipStream_t st); }  // gemm_tile.hip
+namespace uvmi {
+void gemm_tile_launch(const uvmi_gemm_args* a, bool big, hipStream_t st);  // gemm_tile.hip
+void gemm_big_launch(const uvmi_gemm_args* a, hipStream_t st);             // gemm_big.hip
+}
 
 // Rows from which the tiled kernel takes over from the skinny forms when config == 0 (measured on UV-50M's projections).
 constexpr int64_t TILE_MIN_ROWS = 448;
+// Rows from which the 256 x 256 tile of gemm_big.hip takes over (one workgroup per compute unit: it needs several rounds of
+// tiles to pay; measured on UV-50M's projections at 2 k - 33 k rows: from ~12 k rows it is the fastest form for every
+// projection, for the wide gate-up projection with its SwiGLU epilogue already from 4 k).
+constexpr int64_t BIG_MIN_ROWS = 12288, BIG_MIN_ROWS_SWIGLU = 4096;
+
+// what the 256 x 256 kernel assumes beyond uvmi_gemm_tn_supported: two slabs at least, 16-byte stores and residual loads
+static bool big_ok(const uvmi_gemm_args* a) {
+  if (a->K < 128 || ((uintptr_t)a->c % 16) != 0 || a->ldc % 8 != 0) return false;
+  if (a->epilogue == UVMI_GEMM_RESID && (((uintptr_t)a->resid % 16) != 0 || a->ldr % 8 != 0)) return false;
+  return true;
+}
 
 static int skinny_bn(int K, int epilogue) {  // widest strip that fits 64 KB of LDS: 32 rows up to K = 960, else 16
   if (epilogue == UVMI_GEMM_SWIGLU) return K <= 960 ? 32 : 0;
@@ -423,10 +437,17 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
     UVMI_REQUIRE(a->resid && ((uintptr_t)a->resid % 8) == 0 && a->ldr % 4 == 0 && a->ldr >= a->N, UVMI_EINVAL,
                  "uvmi_gemm_tn: the RESID epilogue needs an 8-byte aligned residual with a pitch that is a multiple of 4 and >= N");
   UVMI_REQUIRE(!a->norm_a || a->eps >= 0.f, UVMI_EINVAL, "uvmi_gemm_tn: negative eps");
-  UVMI_REQUIRE(a->config >= 0 && a->config <= 4, UVMI_EINVAL, "uvmi_gemm_tn: config %d", a->config);
+  UVMI_REQUIRE(a->config >= 0 && a->config <= 5, UVMI_EINVAL, "uvmi_gemm_tn: config %d", a->config);
   if (a->M == 0) return UVMI_OK;
   const int BN = skinny_bn(a->K, a->epilogue);
   UVMI_REQUIRE(BN != 0 || a->config == 0 || a->config >= 3, UVMI_EUNSUPPORTED, "uvmi_gemm_tn: K = %d is beyond the skinny forms (config 1, 2)", a->K);
+  if (a->config == 5 || (a->config == 0 && a->M >= (a->epilogue == UVMI_GEMM_SWIGLU ? BIG_MIN_ROWS_SWIGLU : BIG_MIN_ROWS) && big_ok(a))) {
+    UVMI_REQUIRE(big_ok(a), UVMI_EUNSUPPORTED,
+                 "uvmi_gemm_tn: config 5 (256 x 256 tiles) needs K >= 128, C (and the residual) 16-byte aligned, ldc (ldr) %% 8 == 0");
+    gemm_big_launch(a, (hipStream_t)stream);
+    UVMI_CHECK_LAUNCH("uvmi_gemm_tn(256 x 256)");
+    return UVMI_OK;
+  }
   if (a->config >= 3 || (a->config == 0 && (BN == 0 || a->M >= TILE_MIN_ROWS))) {
     // tiled kernel: 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64
     int cus = uvmi_device_cus();

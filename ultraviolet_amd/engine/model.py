@@ -90,14 +90,17 @@ def rms_norm_eps(dtype: torch.dtype) -> float:
 class UVEngine:
     def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 1 << 30, fold_o_rows: int = 1 << 30,
                  fold_gu_rows: int = 1 << 30, lean: bool = True, fold: bool = True, gemm_config: int = 0,
-                 tiled_prefill: bool = True):
+                 tiled_prefill: bool = True, big_rows: int = 12288):
         """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens).
         skinny_rows: passes of at most this many rows run every projection on the skinny GEMM; fold_qkv_rows, fold_o_rows,
         fold_gu_rows: above skinny_rows, row counts up to which the QKV projection (with the pre-norm), the output
         projection (with the residual update) and the gate-up projection (with the pre-norm and the SwiGLU) run on this
         library's GEMM kernels instead of the vendor library's (see _trunk_folded); lean / fold: the launch plans that drop
         the residual-add and norm launches (off: the general path); gemm_config: form of the hand-written GEMM (0: its own
-        choice by size; tests force the tiled forms at a few rows).  The defaults are the measured optimum on UV-50M."""
+        choice by size; tests force the tiled forms at a few rows); big_rows: passes of at least this many rows (a packed
+        prefill, a mixed pass) run all four projections of a block on this library's GEMM, whose 256 x 256 tile form is
+        faster than the vendor library there, with the residual updates in the epilogues.  The defaults are the measured
+        optimum on UV-50M."""
         self.w, self.cfg = weights, weights.cfg
         cfg, dt, dev = self.cfg, weights.dtype, weights.device
         assert cfg.head_dim == 64, "the fused kernels are written for head_dim 64"
@@ -124,6 +127,7 @@ class UVEngine:
         self.fold_o_rows, self.fold_gu_rows = int(fold_o_rows), int(fold_gu_rows)
         self.lean, self.fold, self.gemm_config = bool(lean), bool(fold), int(gemm_config)
         self.tiled_prefill = bool(tiled_prefill)
+        self.big_rows = int(big_rows)
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -335,6 +339,11 @@ class UVEngine:
         fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and self.fold
         tiled_gu = (fold_mlp and self.tiled_prefill and n >= 448 and cfg.d_model % 64 == 0
                     and all("gu_il" in W for W in self.w.layers))
+        # the largest passes: every projection on this library's GEMM (its 256 x 256 tile form), residual updates in place
+        own = (fold_mlp and tiled_gu and n >= self.big_rows and (cfg.n_heads * cfg.head_dim) % 64 == 0 and cfg.d_ff % 64 == 0
+               and cfg.d_model % 8 == 0)
+        if own:
+            mm = lambda a, w, out: gemm_tn(a, w, out, config=self.gemm_config)
         x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
@@ -363,13 +372,19 @@ class UVEngine:
                 # 16-bit passes of any size and attention path: both residual updates are the library's C = alpha A B + beta C
                 # on the hidden in place and the MLP's pre-norm is the row scale inside the SwiGLU launch; the block ends
                 # with the norm the next block's projection and post-processing read
-                torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
+                if own:
+                    gemm_tn(b["zg"][:n], W["wo"], x, epilogue=RESID, resid=x, ca=W["resid_attn"], cb=W["post_attn"], config=self.gemm_config)
+                else:
+                    torch.addmm(x, b["zg"][:n], W["wo"].t(), beta=W["resid_attn"], alpha=W["post_attn"], out=x)
                 if tiled_gu:   # the tiled GEMM with the pre-norm and the SwiGLU in it: the (n, 2 f) product is never written
                     gemm_tn(x, W["gu_il"], b["act"][:n], epilogue=SWIGLU, norm_eps=self.eps, config=self.gemm_config)
                 else:
                     torch.mm(x, W["gu"].t(), out=b["gu"][:n])
                     self._swiglu_norm(x, n)
-                torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
+                if own:
+                    gemm_tn(b["act"][:n], W["down"], x, epilogue=RESID, resid=x, ca=W["resid_mlp"], cb=W["post_mlp"], config=self.gemm_config)
+                else:
+                    torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
                 self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
                 continue
             else:
