@@ -179,8 +179,10 @@ int uvmi_decode_attn_noalloc(const uvmi_attn_args* a, void* stream);
  *     whole weight strip and its activation rows in one burst (K <= 1984; 960 with SWIGLU);
  *   - a tiled form (128 x 128 or 64 x 64 tiles, operand slabs double-buffered in LDS behind a ring of slabs in flight)
  *     for steps of several hundred to a few thousand rows, where the product is bound by feeding the matrix cores;
- *   - a 256 x 256 tile form (slabs loaded from global memory straight into LDS, 128 x 64 per wave) for the passes of many
- *     thousand rows - a packed prefill, a mixed prefill + decode pass - where L2 and LDS bandwidth per flop decide.
+ *   - a form whose slabs go from global memory straight into LDS, with operand reads pipelined ahead of the MFMAs and
+ *     whole-line stores: 256 x 256 tiles (128 x 64 per wave) for the passes of many thousand rows - a packed prefill, a
+ *     mixed prefill + decode pass - where L2 and LDS bandwidth per flop decide, and 128 x 128 tiles in place of the
+ *     tiled form's wherever C is 16-byte aligned.
  * epilogue UVMI_GEMM_SWIGLU (N % 32 == 0): W holds w_gate and w_up interleaved in slabs of 16 rows ([gate 0..15 |
  * up 0..15 | gate 16..31 | ...], N = 2 f rows) and C (M, f) = silu(A w_gate^T) * (A w_up^T) with the roundings of the
  * separate SwiGLU pass (model.py:388-391).
@@ -207,8 +209,9 @@ typedef struct uvmi_gemm_args {
   const void* resid; int64_t ldr; float ca, cb;
   int config;                              /* 0: built-in choice of the kernel form by size; 1: skinny, 64-row workgroups; 2: skinny,
                                               16-row workgroups whose waves split K (needs K % 128 == 0, else form 1); 3: tiled,
-                                              128 x 128; 4: tiled, 64 x 64; 5: 256 x 256 tiles (needs K >= 128, C and resid
-                                              16-byte aligned, ldc, ldr % 8 == 0) - for tuning and tests */
+                                              128 x 128; 4: tiled, 64 x 64; 5: 256 x 256 tiles, 6: 128 x 128 tiles, both with slabs
+                                              loaded straight into LDS (need K >= 128, C and resid 16-byte aligned, ldc,
+                                              ldr % 8 == 0) - for tuning and tests */
 } uvmi_gemm_args;
 int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream);
 

@@ -690,7 +690,7 @@ def test_tiled_gemm_at_prefill_row_counts():
 @pytest.mark.parametrize("M,K,N", [(1, 128, 16), (300, 640, 656), (257, 1664, 640), (1000, 512, 640), (700, 640, 3328), (1030, 2048, 224),
                                    (5000, 640, 672), (513, 192, 512)])
 def test_big_tile_gemm_matches_float64(dtype, M, K, N):
-    """The 256 x 256 tile form (config 5) with every epilogue against float64 on the same 16-bit inputs: ragged M and N (rows
+    """The direct-to-LDS forms (config 5: 256 x 256 tiles, 6: 128 x 128) with every epilogue against float64 on the same 16-bit inputs: ragged M and N (rows
     and weight rows past the end are read clamped and never stored), odd and even slab counts (K / 64), one tile and many,
     padded row pitches, nothing written past column N; to the same bars as the other forms."""
     from ultraviolet_amd.kernels.gemm import RESID, SWIGLU, gemm_tn, interleave_gate_up
@@ -703,22 +703,24 @@ def test_big_tile_gemm_matches_float64(dtype, M, K, N):
     ref = ad @ wd.t()
     tol = ulp * ref.abs().clamp_min(1.0) + 1e-5 * K ** 0.5
     out_full = torch.full((M, N + 8), 7.0, device="cuda", dtype=dtype)
-    gemm_tn(a, w, out_full[:, :N], config=5)
-    assert bool(((out_full[:, :N].double() - ref).abs() <= tol).all()), float((out_full[:, :N].double() - ref).abs().max())
-    assert bool((out_full[:, N:] == 7.0).all())
     an = ad * torch.rsqrt((ad * ad).mean(-1, keepdim=True) + eps)
     refn = an @ wd.t()
-    out = gemm_tn(a, w, norm_eps=eps, config=5)
-    assert bool(((out.double() - refn).abs() <= ulp * refn.abs().clamp_min(1.0) + 1e-5 * K ** 0.5).all())
     r = torch.randn(M, N, device="cuda", generator=g).to(dtype)
     prod = ref.to(dtype).double()
     want = 0.75 * r.double() + 1.25 * prod
     tol2 = ulp * want.abs().clamp_min(1.0) + 1.25 * 2 * ulp * prod.abs().clamp_min(1.0)
-    got = gemm_tn(a, w, epilogue=RESID, resid=r, ca=0.75, cb=1.25, config=5)
-    assert bool(((got.double() - want).abs() <= tol2).all()), float((got.double() - want).abs().max())
-    inplace = r.clone()
-    gemm_tn(a, w, inplace, epilogue=RESID, resid=inplace, ca=0.75, cb=1.25, config=5)
-    assert torch.equal(inplace, got)
+    for config in (5, 6):   # 256 x 256 and 128 x 128 tiles
+        out_full = torch.full((M, N + 8), 7.0, device="cuda", dtype=dtype)
+        gemm_tn(a, w, out_full[:, :N], config=config)
+        assert bool(((out_full[:, :N].double() - ref).abs() <= tol).all()), (config, float((out_full[:, :N].double() - ref).abs().max()))
+        assert bool((out_full[:, N:] == 7.0).all())
+        out = gemm_tn(a, w, norm_eps=eps, config=config)
+        assert bool(((out.double() - refn).abs() <= ulp * refn.abs().clamp_min(1.0) + 1e-5 * K ** 0.5).all()), config
+        got = gemm_tn(a, w, epilogue=RESID, resid=r, ca=0.75, cb=1.25, config=config)
+        assert bool(((got.double() - want).abs() <= tol2).all()), (config, float((got.double() - want).abs().max()))
+        inplace = r.clone()
+        gemm_tn(a, w, inplace, epilogue=RESID, resid=inplace, ca=0.75, cb=1.25, config=config)
+        assert torch.equal(inplace, got)
     if N % 32 == 0:
         f = N // 2
         wg, wu = w[:f].contiguous(), w[f:].contiguous()
@@ -727,21 +729,23 @@ def test_big_tile_gemm_matches_float64(dtype, M, K, N):
             uu = (src @ wu.double().t()).to(dtype).double()
             ra = (gg * torch.sigmoid(gg)).to(dtype).double() * uu
             tol3 = 4 * ulp * ra.abs().clamp_min(1.0) + 4 * ulp * (gg.abs() + uu.abs())
-            act_full = torch.full((M, f + 8), 7.0, device="cuda", dtype=dtype)
-            gemm_tn(a, interleave_gate_up(wg, wu), act_full[:, :f], epilogue=SWIGLU, norm_eps=nrm, config=5)
-            assert bool(((act_full[:, :f].double() - ra).abs() <= tol3).all()), (nrm, float((act_full[:, :f].double() - ra).abs().max()))
-            assert bool((act_full[:, f:] == 7.0).all())
+            for config in (5, 6):
+                act_full = torch.full((M, f + 8), 7.0, device="cuda", dtype=dtype)
+                gemm_tn(a, interleave_gate_up(wg, wu), act_full[:, :f], epilogue=SWIGLU, norm_eps=nrm, config=config)
+                assert bool(((act_full[:, :f].double() - ra).abs() <= tol3).all()), (config, nrm, float((act_full[:, :f].double() - ra).abs().max()))
+                assert bool((act_full[:, f:] == 7.0).all())
 
 
 @pytest.mark.gpu
 def test_big_tile_gemm_rejects_what_it_cannot_do():
-    """config 5 needs two K slabs and 16-byte rows of C: asked for anything else it raises instead of running another form."""
+    """configs 5 and 6 need two K slabs and 16-byte rows of C: asked for anything else they raise instead of running another form."""
     from ultraviolet_amd._lib import UvmiError
     from ultraviolet_amd.kernels.gemm import gemm_tn
     a = torch.randn(300, 128, device="cuda").to(torch.bfloat16)
     w = torch.randn(64, 128, device="cuda").to(torch.bfloat16)
-    with pytest.raises(UvmiError):
-        gemm_tn(a[:, :64], w[:, :64], config=5)                                   # one slab
-    with pytest.raises(UvmiError):
-        gemm_tn(a, w, torch.empty(300, 68, device="cuda", dtype=torch.bfloat16)[:, :64], config=5)   # pitch 68
-    gemm_tn(a, w, config=5)
+    for config in (5, 6):
+        with pytest.raises(UvmiError):
+            gemm_tn(a[:, :64], w[:, :64], config=config)                                   # one slab
+        with pytest.raises(UvmiError):
+            gemm_tn(a, w, torch.empty(300, 68, device="cuda", dtype=torch.bfloat16)[:, :64], config=config)   # pitch 68
+        gemm_tn(a, w, config=config)

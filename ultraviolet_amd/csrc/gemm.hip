@@ -372,7 +372,7 @@ using namespace uvmi;
 
 namespace uvmi {
 void gemm_tile_launch(const uvmi_gemm_args* a, bool big, hipStream_t st);  // gemm_tile.hip
-void gemm_big_launch(const uvmi_gemm_args* a, hipStream_t st);             // gemm_big.hip
+void gemm_big_launch(const uvmi_gemm_args* a, int tile, hipStream_t st);   // gemm_big.hip
 }
 
 // Rows from which the tiled kernel takes over from the skinny forms when config == 0 (measured on UV-50M's projections).
@@ -437,15 +437,22 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
     UVMI_REQUIRE(a->resid && ((uintptr_t)a->resid % 8) == 0 && a->ldr % 4 == 0 && a->ldr >= a->N, UVMI_EINVAL,
                  "uvmi_gemm_tn: the RESID epilogue needs an 8-byte aligned residual with a pitch that is a multiple of 4 and >= N");
   UVMI_REQUIRE(!a->norm_a || a->eps >= 0.f, UVMI_EINVAL, "uvmi_gemm_tn: negative eps");
-  UVMI_REQUIRE(a->config >= 0 && a->config <= 5, UVMI_EINVAL, "uvmi_gemm_tn: config %d", a->config);
+  UVMI_REQUIRE(a->config >= 0 && a->config <= 6, UVMI_EINVAL, "uvmi_gemm_tn: config %d", a->config);
   if (a->M == 0) return UVMI_OK;
   const int BN = skinny_bn(a->K, a->epilogue);
   UVMI_REQUIRE(BN != 0 || a->config == 0 || a->config >= 3, UVMI_EUNSUPPORTED, "uvmi_gemm_tn: K = %d is beyond the skinny forms (config 1, 2)", a->K);
   if (a->config == 5 || (a->config == 0 && a->M >= (a->epilogue == UVMI_GEMM_SWIGLU ? BIG_MIN_ROWS_SWIGLU : BIG_MIN_ROWS) && big_ok(a))) {
     UVMI_REQUIRE(big_ok(a), UVMI_EUNSUPPORTED,
                  "uvmi_gemm_tn: config 5 (256 x 256 tiles) needs K >= 128, C (and the residual) 16-byte aligned, ldc (ldr) %% 8 == 0");
-    gemm_big_launch(a, (hipStream_t)stream);
+    gemm_big_launch(a, 256, (hipStream_t)stream);
     UVMI_CHECK_LAUNCH("uvmi_gemm_tn(256 x 256)");
+    return UVMI_OK;
+  }
+  if (a->config == 6) {
+    UVMI_REQUIRE(big_ok(a), UVMI_EUNSUPPORTED,
+                 "uvmi_gemm_tn: config %d (tiles loaded straight into LDS) needs K >= 128, C (and the residual) 16-byte aligned, ldc (ldr) %% 8 == 0", a->config);
+    gemm_big_launch(a, 128, (hipStream_t)stream);
+    UVMI_CHECK_LAUNCH("uvmi_gemm_tn(128 x 128, direct)");
     return UVMI_OK;
   }
   if (a->config >= 3 || (a->config == 0 && (BN == 0 || a->M >= TILE_MIN_ROWS))) {
@@ -454,6 +461,11 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
     if (cus <= 0) cus = 256;
     const int64_t t128 = ((a->M + 127) / 128) * ((a->N + 127) / 128);
     const bool big = a->config == 3 || (a->config == 0 && 4 * t128 >= 3 * cus);
+    if (big && a->config == 0 && big_ok(a)) {   // the 128 x 128 tile in its direct-to-LDS form (gemm_big.hip): faster wherever it applies
+      gemm_big_launch(a, 128, (hipStream_t)stream);
+      UVMI_CHECK_LAUNCH("uvmi_gemm_tn(128 x 128, direct)");
+      return UVMI_OK;
+    }
     gemm_tile_launch(a, big, (hipStream_t)stream);
     UVMI_CHECK_LAUNCH("uvmi_gemm_tn(tiled)");
     return UVMI_OK;

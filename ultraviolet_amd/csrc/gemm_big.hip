@@ -65,10 +65,14 @@ template <int DT> __device__ __forceinline__ void unpack2(uint32_t w, float& lo,
 
 // EPI 0: C = A W^T (M, N).  EPI 1: W rows are [gate 16 | up 16] slabs; C = silu(gate) * up, (M, N / 2).
 // EPI 2: C = ca * R + cb * (A W^T).  NORM: A stands for its RMS-normalised rows.
-template <int DT, int EPI, bool NORM>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// FI: 16-row fragments per wave along M: 8 - the 256 x 256 tile on 8 waves (2 x 4); 4 - a 128 x 128 tile on 4 waves (2 x 2,
+// 64 x 64 per wave, two workgroups per compute unit) for passes whose 256 x 256 tiles would not fill the device.  (A
+// 64 x 64 tile on 2 waves was measured too: no faster than the tiled kernel's 64 x 64 form at 2 k rows.)
+template <int DT, int EPI, bool NORM, int FI>
+__global__ __launch_bounds__(64 * FI) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_big_kernel(BigParams P) {
-  constexpr int BM = 256, BN = 256;
+  constexpr int WN = FI / 2;                   // waves along N (2 along M)
+  constexpr int BM = 32 * FI, BN = 64 * WN;
   // one array per stage and operand: the compiler can then tell that the operand reads of one stage do not touch the
   // stage a load in flight is writing, and does not wait for that load
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * 128];
@@ -86,8 +90,8 @@ void gemm_big_kernel(BigParams P) {
   const int m0 = bm * BM, n0 = bn * BN;
   const int nk = P.K / 64;
 
-  // ---- loader: wave w fills blocks 4 w .. 4 w + 3 (8 rows each) of A and of W.  Rows past M / N repeat the last row:
-  // what they produce is never stored.
+  // ---- loader: wave w fills blocks 4 w .. 4 w + 3 (8 rows each) of A and of W (BM = BN = 32 x the number of waves).  Rows
+  // past M / N repeat the last row: what they produce is never stored.
   uint32_t offA[4], offB[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -112,20 +116,20 @@ void gemm_big_kernel(BigParams P) {
       __builtin_amdgcn_global_load_lds(UVMI_GLBP(gw + offB[i] + ko), UVMI_LDSP(sb + (4 * wave + i) * 1024), 16, 0, 0);
   };
 
-  // ---- reader: wave (wm, wn) owns rows 128 wm .., columns 64 wn ..; lane (r, g) reads chunk (4 s + g) ^ ((r / 2) % 8) of
+  // ---- reader: wave (wm, wn) owns rows 16 FI wm .., columns 64 wn ..; lane (r, g) reads chunk (4 s + g) ^ ((r / 2) % 8) of
   // row r of a 16-row fragment for K-step s
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave / WN, wn = wave % WN;
   const int r = lane & 15, g = lane >> 4;
   uint32_t a_off[2], b_off[2];
 #pragma unroll
   for (int s = 0; s < 2; s++) {
     const uint32_t lo = (uint32_t)r * 128 + (uint32_t)((((4 * s + g) ^ ((r >> 1) & 7))) << 4);
-    a_off[s] = (uint32_t)wm * 16384 + lo;
+    a_off[s] = (uint32_t)wm * (16 * FI * 128) + lo;
     b_off[s] = (uint32_t)wn * 8192 + lo;
   }
-  gf4 acc[8][4];
+  gf4 acc[FI][4];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int i = 0; i < FI; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = gf4{0.f, 0.f, 0.f, 0.f};
 
@@ -147,7 +151,7 @@ void gemm_big_kernel(BigParams P) {
     for (int j = 0; j < 4; j++) acc[i + 1][j] = gmfma<DT>(w[j], f[1], acc[i + 1][j]);
   };
   // NORM: the squares of the rows are summed from the operand fragments as they pass: wave (wm, wn) takes row pair wn of
-  // each K-step (rows 128 wm + 32 wn + 16 u + r, u = 0, 1; lane (r, g) sees 8 of a row's 32 values)
+  // each K-step (rows 16 FI wm + 32 wn + 16 u + r, u = 0, 1; lane (r, g) sees 8 of a row's 32 values)
   float ss[2] = {0.f, 0.f};
   auto sumsq = [&](int pair, const gu4* f) {
     if (NORM && wn == pair) {
@@ -190,20 +194,42 @@ void gemm_big_kernel(BigParams P) {
     read_b(SBN, 0, w0); read_a(SAN, 0, 0, f0); UVMI_SB();                                                                \
     mm1(6, f1, w1); mm7(6, f1, w1); sumsq(3, f1); UVMI_SB();                                                             \
   } while (0)
+  // FI = 4: 4 groups per slab; the first operands of the next slab arrive in the buffer the iteration's second group used,
+  // so two iterations alternate the roles of f0 and f1
+#define UVMI_ITER4(SA, SB_, SAN, SBN, k, X, Y)                                                                           \
+  do {                                                                                                                   \
+    mm1(0, X, w0); UVMI_SB(); read_a(SA, 0, 2, Y); UVMI_SB(); mm7(0, X, w0); sumsq(0, X); UVMI_SB();                     \
+    mm1(2, Y, w0); UVMI_SB(); read_b(SB_, 1, w1); read_a(SA, 1, 0, f2); UVMI_SB(); mm7(2, Y, w0); sumsq(1, Y); UVMI_SB(); \
+    mm1(0, f2, w1); UVMI_SB(); read_a(SA, 1, 2, X); UVMI_SB(); mm7(0, f2, w1); sumsq(0, f2); UVMI_SB();                  \
+    __builtin_amdgcn_s_waitcnt(0x0f70);                                                                                  \
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");                                                      \
+    issue(SA, SB_, (k) + 2);                                                                                             \
+    read_b(SBN, 0, w0); read_a(SAN, 0, 0, Y); UVMI_SB();                                                                 \
+    mm1(2, X, w1); mm7(2, X, w1); sumsq(1, X); UVMI_SB();                                                                \
+  } while (0)
   int k = 0;
-  for (; k + 2 <= nk; k += 2) {
-    UVMI_ITER(sA0, sB0, sA1, sB1, k);
-    UVMI_ITER(sA1, sB1, sA0, sB0, k + 1);
+  if constexpr (FI == 8) {
+    for (; k + 2 <= nk; k += 2) {
+      UVMI_ITER(sA0, sB0, sA1, sB1, k);
+      UVMI_ITER(sA1, sB1, sA0, sB0, k + 1);
+    }
+    if (k < nk) UVMI_ITER(sA0, sB0, sA1, sB1, k);
+  } else {
+    for (; k + 2 <= nk; k += 2) {
+      UVMI_ITER4(sA0, sB0, sA1, sB1, k, f0, f1);
+      UVMI_ITER4(sA1, sB1, sA0, sB0, k + 1, f1, f0);
+    }
+    if (k < nk) UVMI_ITER4(sA0, sB0, sA1, sB1, k, f0, f1);
   }
-  if (k < nk) UVMI_ITER(sA0, sB0, sA1, sB1, k);
+#undef UVMI_ITER4
 #undef UVMI_ITER
 #undef UVMI_SB
   __builtin_amdgcn_s_waitcnt(0x0f70);   // the loads past the last slab have landed before LDS is reused or the wave ends
 
   // ---- row scales of the pre-norm: the 4 lane groups of a row add their sums; LDS carries the scales to every wave
-  float rn[8];
+  float rn[FI];
 #pragma unroll
-  for (int i = 0; i < 8; i++) rn[i] = 1.0f;
+  for (int i = 0; i < FI; i++) rn[i] = 1.0f;
   if (NORM) {
     float* sRS = (float*)sA0;
     __syncthreads();   // every wave's loads have landed and its operand reads are done
@@ -212,17 +238,17 @@ void gemm_big_kernel(BigParams P) {
       float v = ss[u];
       v += lane_xor16(v);
       v = xsum32(v);
-      if (g == 0) sRS[128 * wm + 32 * wn + 16 * u + r] = rsqrtf(v / (float)P.K + P.eps);
+      if (g == 0) sRS[16 * FI * wm + 32 * wn + 16 * u + r] = rsqrtf(v / (float)P.K + P.eps);
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 8; i++) rn[i] = sRS[128 * wm + 16 * i + r];
+    for (int i = 0; i < FI; i++) rn[i] = sRS[16 * FI * wm + 16 * i + r];
   }
 
-  // ---- epilogue: accumulator (i, j): lane (r, g) holds C[m0 + 128 wm + 16 i + r][n0 + 64 wn + 16 j + 4 g + t], t = 0..3
+  // ---- epilogue: accumulator (i, j): lane (r, g) holds C[m0 + 16 FI wm + 16 i + r][n0 + 64 wn + 16 j + 4 g + t], t = 0..3
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const int row = m0 + 128 * wm + 16 * i + r;
+  for (int i = 0; i < FI; i++) {
+    const int row = m0 + 16 * FI * wm + 16 * i + r;
     if (EPI == 1) {
       // gate slab j, up slab j + 1 -> 4 outputs per slab pair; after the 2 x 2 transpose lane (r, g) holds the 8 consecutive
       // output columns 16 (g % 2) + 8 (g / 2) .. of the wave's 32
@@ -278,11 +304,11 @@ void gemm_big_kernel(BigParams P) {
   }
 }
 
-template <int DT>
+template <int DT, int FI>
 static void launch_big(const uvmi_gemm_args* a, const BigParams& P, hipStream_t st) {
   const int T = P.tiles_m * P.tiles_n;
-  const dim3 grid((unsigned)(((T + 7) / 8) * 8)), blk(512);
-#define UVMI_GO(EPI, NORM) hipLaunchKernelGGL((gemm_big_kernel<DT, EPI, NORM>), grid, blk, 0, st, P)
+  const dim3 grid((unsigned)(((T + 7) / 8) * 8)), blk(64 * FI);
+#define UVMI_GO(EPI, NORM) hipLaunchKernelGGL((gemm_big_kernel<DT, EPI, NORM, FI>), grid, blk, 0, st, P)
   const bool norm = a->norm_a != 0;
   if (a->epilogue == UVMI_GEMM_RESID) { if (norm) UVMI_GO(2, true); else UVMI_GO(2, false); }
   else if (a->epilogue == UVMI_GEMM_SWIGLU) { if (norm) UVMI_GO(1, true); else UVMI_GO(1, false); }
@@ -290,19 +316,19 @@ static void launch_big(const uvmi_gemm_args* a, const BigParams& P, hipStream_t 
 #undef UVMI_GO
 }
 
-// Arguments are validated by the caller (uvmi_gemm_tn_ex), which also checks K >= 128.
-void gemm_big_launch(const uvmi_gemm_args* a, hipStream_t st) {
+// Arguments are validated by the caller (uvmi_gemm_tn_ex), which also checks K >= 128.  tile: 256 or 128.
+void gemm_big_launch(const uvmi_gemm_args* a, int tile, hipStream_t st) {
   BigParams P;
   P.a = a->a; P.w = a->w; P.c = a->c; P.r = a->resid;
   P.lda2 = (uint32_t)a->lda * 2; P.ldw2 = (uint32_t)a->ldw * 2; P.ldc = a->ldc; P.ldr = a->ldr;
   P.M = (int)a->M; P.N = a->N; P.K = a->K;
-  P.tiles_m = (int)((a->M + 255) / 256);
-  P.tiles_n = (a->N + 255) / 256;
+  P.tiles_m = (int)((a->M + tile - 1) / tile);
+  P.tiles_n = (a->N + tile - 1) / tile;
   P.eps = a->eps; P.ca = a->ca; P.cb = a->cb;
   const double bytes_a = (double)a->M * a->K, bytes_w = (double)a->N * a->K;
   P.rowsplit = bytes_a / 8 + bytes_w < bytes_a + bytes_w / 8;
-  if (a->dtype == UVMI_F16) launch_big<UVMI_F16>(a, P, st);
-  else launch_big<UVMI_BF16>(a, P, st);
+  if (a->dtype == UVMI_F16) { if (tile == 256) launch_big<UVMI_F16, 8>(a, P, st); else launch_big<UVMI_F16, 4>(a, P, st); }
+  else { if (tile == 256) launch_big<UVMI_BF16, 8>(a, P, st); else launch_big<UVMI_BF16, 4>(a, P, st); }
 }
 
 }  // namespace uvmi
