@@ -346,6 +346,11 @@ typedef struct uvmi_qkv_post_args {
   /* optional: uvmi_rope_table's output in dtype's rounding for positions 0 .. rope_positions - 1; tokens at those positions
    * read their cos / sin from it (the same values the kernel would compute), others compute them */
   const float* rope_table; int rope_positions;
+  /* optional: the projection output carries the gates' logits behind q, k, v, as the extended projection of the decode
+   * step forms them (columns (H + 2 KH) * hd .. : H output-gate logits, then KH value-embedding gate logits, in dtype).
+   * qkv_ld: row pitch of qkv in elements (0: (H + 2 KH) * hd).  ext_logits != 0: the logits are read from those columns
+   * instead of being computed from xn, gate_w and ve_gate, which may then be NULL. */
+  int64_t qkv_ld; int ext_logits;
 } uvmi_qkv_post_args;
 int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream);
 

@@ -102,7 +102,8 @@ class QkvPostArgs(C.Structure):
                 ("H", C.c_int), ("KH", C.c_int), ("hd", C.c_int), ("d", C.c_int), ("ve_ch", C.c_int),
                 ("n_pairs", C.c_int), ("S", C.c_int), ("ring", C.c_int), ("has_ve", C.c_int), ("rope", C.c_int),
                 ("eps", C.c_float), ("gate_w", C.c_void_p), ("gate_ch", C.c_int), ("gate_out", C.c_void_p),
-                ("vhat_out", C.c_void_p), ("xsa_eps", C.c_float), ("rope_table", C.c_void_p), ("rope_positions", C.c_int)]
+                ("vhat_out", C.c_void_p), ("xsa_eps", C.c_float), ("rope_table", C.c_void_p), ("rope_positions", C.c_int),
+                ("qkv_ld", C.c_int64), ("ext_logits", C.c_int)]
 
 
 class SchedState(C.Structure):

@@ -144,6 +144,7 @@ struct QkvArgs {
   int H, KH, d, ve_ch, n_pairs, S, ring, has_ve, rope, q_dt, gate_ch;
   float eps, xsa_eps;
   const float* rope_tab; int rope_n;   // optional table of the rounded cos / sin per position (row: cos[n_pairs], sin[n_pairs])
+  int64_t ld; int ext;                 // row pitch of qkv; gate logits read from columns W .. of the row instead of formed from xn
 };
 
 template <int DT>
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= A.n) return;
   const int W = (A.H + 2 * A.KH) * 64;
-  const int64_t base = r * W;
+  const int64_t base = r * A.ld;
   const int64_t p = A.pos[r];
   const int np_ = A.n_pairs;
   const float* tab = A.rope_tab && p >= 0 && p < A.rope_n ? A.rope_tab + p * 2 * np_ : nullptr;   // (wave-uniform)
@@ -221,7 +222,9 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       for (int h0 = 0; h0 < A.H; h0 += 8) {
         const int h = h0 + hh;
         float dot = 0.f;
-        if (h < A.H) {
+        if (A.ext) {   // the projection formed the logit (already rounded to the activation type)
+          if (h < A.H && c == 0) dot = elem<DT>::ld(A.qkv, base + W + h);
+        } else if (h < A.H) {
           if (cpl % 8 == 0 && (A.d % 8) == 0) {
             for (int j = 0; j < cpl; j += 8) {
               float xv[8];
@@ -269,8 +272,11 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
     float v = elem<DT>::ld(A.qkv, base + (A.H + A.KH + kh) * 64 + lane);
     if (A.has_ve) {  // v += 2 sigmoid(W xn[:ve_ch]) * value_embed[tok]
       float dot = 0.f;
-      if (lane < A.ve_ch) dot = elem<DT>::ld(A.xn, r * A.d + lane) * A.ve_gate[kh * A.ve_ch + lane];
-      dot = round_t<DT>(wave_sum(dot));
+      if (A.ext) dot = elem<DT>::ld(A.qkv, base + W + A.H + kh);
+      else {
+        if (lane < A.ve_ch) dot = elem<DT>::ld(A.xn, r * A.d + lane) * A.ve_gate[kh * A.ve_ch + lane];
+        dot = round_t<DT>(wave_sum(dot));
+      }
       const float g = round_t<DT>(2.0f * round_t<DT>(1.0f / (1.0f + __expf(-dot))));
       int64_t t = A.tok[r];
       if (t < 0) t = 0;
@@ -447,10 +453,15 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   UVMI_REQUIRE(a->n >= 0 && a->H > 0 && a->KH > 0 && a->H % a->KH == 0, UVMI_EINVAL, "uvmi_qkv_post: bad sizes");
   UVMI_REQUIRE(!a->rope || (a->inv_freq && a->n_pairs >= 8 && a->n_pairs <= 32 && (a->n_pairs & (a->n_pairs - 1)) == 0), UVMI_EUNSUPPORTED,
                "uvmi_qkv_post: rope needs inv_freq and 8, 16 or 32 rotated pairs");
-  UVMI_REQUIRE(!a->gate_out || (a->gate_w && a->xn && a->gate_ch > 0 && a->gate_ch % 8 == 0 && a->gate_ch <= a->d), UVMI_EINVAL,
-               "uvmi_qkv_post: gate_out needs gate_w, xn and a gate_ch that is a multiple of 8");
+  UVMI_REQUIRE(!a->gate_out || a->ext_logits || (a->gate_w && a->xn && a->gate_ch > 0 && a->gate_ch % 8 == 0 && a->gate_ch <= a->d), UVMI_EINVAL,
+               "uvmi_qkv_post: gate_out needs gate_w, xn and a gate_ch that is a multiple of 8 (or ext_logits)");
+  const int64_t qkv_w = (int64_t)(a->H + 2 * a->KH) * a->hd;
+  UVMI_REQUIRE(a->qkv_ld == 0 || a->qkv_ld >= qkv_w, UVMI_EINVAL, "uvmi_qkv_post: qkv_ld below the row width");
+  UVMI_REQUIRE(a->qkv_ld % 8 == 0, UVMI_EUNSUPPORTED, "uvmi_qkv_post: qkv_ld must be a multiple of 8 (16-byte rows)");
+  UVMI_REQUIRE(!a->ext_logits || a->qkv_ld >= qkv_w + a->H + a->KH, UVMI_EINVAL,
+               "uvmi_qkv_post: ext_logits needs a row pitch that holds the H + KH logits behind q, k, v");
   UVMI_REQUIRE(((uintptr_t)a->qkv % 16) == 0 && ((uintptr_t)a->q_out % 16) == 0, UVMI_EUNSUPPORTED, "uvmi_qkv_post: qkv and q_out must be 16-byte aligned");
-  UVMI_REQUIRE(!a->has_ve || (a->xn && a->ve_table && a->ve_gate && a->tok && a->ve_ch > 0 && a->ve_ch <= 64 && a->vocab > 0), UVMI_EINVAL,
+  UVMI_REQUIRE(!a->has_ve || (a->ve_table && a->tok && a->vocab > 0 && (a->ext_logits || (a->xn && a->ve_gate && a->ve_ch > 0 && a->ve_ch <= 64))), UVMI_EINVAL,
                "uvmi_qkv_post: value-embedding inputs missing");
   UVMI_REQUIRE(!a->k_cache || (a->v_cache && a->k_scale && a->v_scale && a->S > 0), UVMI_EINVAL, "uvmi_qkv_post: incomplete cache arguments");
   if (a->n == 0) return UVMI_OK;
@@ -464,6 +475,8 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   A.gate_w = a->gate_w; A.gate_out = a->gate_out; A.vhat_out = a->vhat_out; A.gate_ch = a->gate_ch; A.xsa_eps = a->xsa_eps;
   A.rope_tab = a->rope && a->rope_positions > 0 ? a->rope_table : nullptr;
   A.rope_n = a->rope_positions;
+  A.ld = a->qkv_ld ? a->qkv_ld : qkv_w;
+  A.ext = a->ext_logits != 0;
   const dim3 grid((unsigned)((a->n + 3) / 4)), blk(256);
   dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
   UVMI_CHECK_LAUNCH("uvmi_qkv_post");

@@ -146,11 +146,15 @@ class UVEngine:
         L.check(rc, "uvmi_add_norm")
 
     def _qkv_post(self, l: int, tok: Tensor, pos: Tensor, rows: Tensor | None, last_pos: Tensor | None, st: KVState | None,
-                  n: int, write_cache: bool = True):
+                  n: int, write_cache: bool = True, ext: bool = False):
+        """ext: the rows come from the extended projection (buf qkvx), whose last columns are the gates' logits: the
+        normalised block input is then not read."""
         cfg, b, W = self.cfg, self.buf, self.w.layers[l]
         glob = cfg.is_global(l)
         a = L.QkvPostArgs()
-        a.qkv, a.dtype, a.xn = b["qkv"].data_ptr(), self.dt_code, b["xn"].data_ptr()
+        a.qkv, a.dtype, a.xn = b["qkvx" if ext else "qkv"].data_ptr(), self.dt_code, b["xn"].data_ptr()
+        if ext:
+            a.qkv_ld, a.ext_logits = b["qkvx"].stride(0), 1
         has_ve = cfg.has_ve(l)
         if has_ve:
             a.ve_table, a.ve_gate, a.tok = self.w.value_embed.data_ptr(), W["ve_gate"].data_ptr(), tok.data_ptr()
@@ -344,6 +348,10 @@ class UVEngine:
                and cfg.d_model % 8 == 0)
         if own:
             mm = lambda a, w, out: gemm_tn(a, w, out, config=self.gemm_config)
+        # ... and with the extended projection (q, k, v and the gates' logits) the block's pre-norm rides on the QKV GEMM as a
+        # row scale and the post-processing reads the logits from the projection: the normalised hidden is not written between
+        # blocks (it is formed on demand for a layer whose attention leaves its epilogue to _attn_post)
+        own_ext = own and self.fuse_qkv and fused_attn is None and all("wqkv_ext" in W for W in self.w.layers)
         x_is_normed = True   # buf xn holds rmsnorm(x)
         for l, W in enumerate(self.w.layers):
             if fused_attn is not None and self.fused_layer_ok(l, st):
@@ -356,6 +364,18 @@ class UVEngine:
                 if self.qkvx_keep is not None:   # a benchmark re-issues this layer's launch later on the same projection
                     self.qkvx_keep[l][:n].copy_(b["qkvx"][:n])
                 fused_attn(l)
+            elif own_ext:
+                if x_is_normed:
+                    gemm_tn(xn, W["wqkv_ext"], b["qkvx"][:n], config=self.gemm_config)
+                else:
+                    gemm_tn(x, W["wqkv_ext"], b["qkvx"][:n], norm_eps=self.eps, config=self.gemm_config)
+                self._qkv_post(l, tok, pos, rows, last_pos, st, n, ext=True)
+                z = attn(l, b["q"][:n])
+                if z is not None:
+                    if not x_is_normed:
+                        self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
+                        x_is_normed = True
+                    self._attn_post(l, z, n)
             else:
                 mm(xn, W["wqkv"], b["qkv"][:n])
                 self._qkv_post(l, tok, pos, rows, last_pos, st, n)
@@ -385,7 +405,10 @@ class UVEngine:
                     gemm_tn(b["act"][:n], W["down"], x, epilogue=RESID, resid=x, ca=W["resid_mlp"], cb=W["post_mlp"], config=self.gemm_config)
                 else:
                     torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
-                self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
+                if own_ext:
+                    x_is_normed = False
+                else:
+                    self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])
                 continue
             else:
                 mm(b["zg"][:n], W["wo"], b["a"][:n])
