@@ -97,9 +97,9 @@ class UVEngine:
         projection (with the residual update) and the gate-up projection (with the pre-norm and the SwiGLU) run on this
         library's GEMM kernels instead of the vendor library's (see _trunk_folded); lean / fold: the launch plans that drop
         the residual-add and norm launches (off: the general path); gemm_config: form of the hand-written GEMM (0: its own
-        choice by size; tests force the tiled forms at a few rows); big_rows: passes of at least this many rows (a packed
-        prefill, a mixed pass) run all four projections of a block on this library's GEMM, whose 256 x 256 tile form is
-        faster than the vendor library there, with the residual updates in the epilogues.  The defaults are the measured
+        choice by size; tests force the tiled forms at a few rows); big_rows: passes of the general path with at least this
+        many rows (a packed prefill, a mixed pass) run the down projection too on this library's GEMM, whose 256 x 256 tile
+        form is faster than the vendor library there (the other three projections run on it from 448 rows).  The defaults are the measured
         optimum on UV-50M."""
         self.w, self.cfg = weights, weights.cfg
         cfg, dt, dev = self.cfg, weights.dtype, weights.device
@@ -343,9 +343,11 @@ class UVEngine:
         fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and self.fold
         tiled_gu = (fold_mlp and self.tiled_prefill and n >= 448 and cfg.d_model % 64 == 0
                     and all("gu_il" in W for W in self.w.layers))
-        # the largest passes: every projection on this library's GEMM (its 256 x 256 tile form), residual updates in place
-        own = (fold_mlp and tiled_gu and n >= self.big_rows and (cfg.n_heads * cfg.head_dim) % 64 == 0 and cfg.d_ff % 64 == 0
-               and cfg.d_model % 8 == 0)
+        # Passes of the general path with many rows (a packed prefill, a mixed step): the QKV and output projections run on this
+        # library's GEMM (64 x 64 / 128 x 128 tiles, 256 x 256 from big_rows rows on - faster than the vendor library's at these
+        # shapes), the output projection with the residual update in place; from big_rows rows on the down projection too.
+        own = (fold_mlp and tiled_gu and (cfg.n_heads * cfg.head_dim) % 64 == 0 and cfg.d_ff % 64 == 0 and cfg.d_model % 8 == 0)
+        own_down = own and n >= self.big_rows
         if own:
             mm = lambda a, w, out: gemm_tn(a, w, out, config=self.gemm_config)
         # ... and with the extended projection (q, k, v and the gates' logits) the block's pre-norm rides on the QKV GEMM as a
@@ -401,7 +403,7 @@ class UVEngine:
                 else:
                     torch.mm(x, W["gu"].t(), out=b["gu"][:n])
                     self._swiglu_norm(x, n)
-                if own:
+                if own_down:
                     gemm_tn(b["act"][:n], W["down"], x, epilogue=RESID, resid=x, ca=W["resid_mlp"], cb=W["post_mlp"], config=self.gemm_config)
                 else:
                     torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
