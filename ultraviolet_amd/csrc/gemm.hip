@@ -375,8 +375,11 @@ void gemm_tile_launch(const uvmi_gemm_args* a, bool big, hipStream_t st);  // ge
 void gemm_big_launch(const uvmi_gemm_args* a, int tile, hipStream_t st);   // gemm_big.hip
 }
 
-// Rows from which the tiled kernel takes over from the skinny forms when config == 0 (measured on UV-50M's projections).
-constexpr int64_t TILE_MIN_ROWS = 448;
+// Rows from which the tiled kernel takes over from the skinny forms when config == 0 (measured on UV-50M's projections):
+// 448 for the narrow projections (N ~ 640: fewer rows give the 64 x 64 grid too few tiles); the wide gate-up projection with
+// its SwiGLU epilogue already from 128 rows (2 x 52 tiles: 6.8 us at 128 - 256 rows and 9.0 us at 384, where the 64-row
+// skinny form takes 7.6 - 10.5 and 15.4 us).
+constexpr int64_t TILE_MIN_ROWS = 448, TILE_MIN_ROWS_SWIGLU = 128;
 // Rows from which the 256 x 256 tile of gemm_big.hip takes over (one workgroup per compute unit: it needs several rounds of
 // tiles to pay; measured on UV-50M's projections at 2 k - 33 k rows: from ~12 k rows it is the fastest form for every
 // projection, for the wide gate-up projection with its SwiGLU epilogue already from 4 k).
@@ -455,7 +458,8 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
     UVMI_CHECK_LAUNCH("uvmi_gemm_tn(128 x 128, direct)");
     return UVMI_OK;
   }
-  if (a->config >= 3 || (a->config == 0 && (BN == 0 || a->M >= TILE_MIN_ROWS))) {
+  const int64_t tile_min_rows = a->epilogue == UVMI_GEMM_SWIGLU && a->N >= 2048 ? TILE_MIN_ROWS_SWIGLU : TILE_MIN_ROWS;
+  if (a->config >= 3 || (a->config == 0 && (BN == 0 || a->M >= tile_min_rows))) {
     // tiled kernel: 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64
     int cus = uvmi_device_cus();
     if (cus <= 0) cus = 256;
