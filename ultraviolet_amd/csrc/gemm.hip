@@ -460,11 +460,11 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
   }
   const int64_t tile_min_rows = a->epilogue == UVMI_GEMM_SWIGLU && a->N >= 2048 ? TILE_MIN_ROWS_SWIGLU : TILE_MIN_ROWS;
   if (a->config >= 3 || (a->config == 0 && (BN == 0 || a->M >= tile_min_rows))) {
-    // tiled kernel: 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64
+    // tiled kernel: 128 x 128 tiles when there are enough of them for 3/5 of the compute units, else 64 x 64
     int cus = uvmi_device_cus();
     if (cus <= 0) cus = 256;
     const int64_t t128 = ((a->M + 127) / 128) * ((a->N + 127) / 128);
-    const bool big = a->config == 3 || (a->config == 0 && 4 * t128 >= 3 * cus);
+    const bool big = a->config == 3 || (a->config == 0 && 5 * t128 >= 3 * cus);   // (measured crossover: gate-up at ~640 rows)
     if (big && a->config == 0 && big_ok(a)) {   // the 128 x 128 tile in its direct-to-LDS form (gemm_big.hip): faster wherever it applies
       gemm_big_launch(a, 128, (hipStream_t)stream);
       UVMI_CHECK_LAUNCH("uvmi_gemm_tn(128 x 128, direct)");
