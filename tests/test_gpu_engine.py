@@ -118,12 +118,15 @@ def test_greedy_64_tokens_identical_fp32(name, over):
 # the decode pass's launch plans by row count, forced here at a few rows:
 # (skinny_rows, fold_qkv_rows, fold_o_rows, fold_gu_rows, form of the hand-written GEMM)
 _TRUNK_PLANS = {"small": None, "large-skinny-attn-block": (0, 1 << 30, 1 << 30, 0, 0), "large-library": (0, 0, 0, 0, 0),
-                "large-tiled-64": (0, 1 << 30, 1 << 30, 1 << 30, 4), "large-tiled-128": (0, 1 << 30, 1 << 30, 1 << 30, 3)}
+                "large-tiled-64": (0, 1 << 30, 1 << 30, 1 << 30, 4), "large-tiled-128": (0, 1 << 30, 1 << 30, 1 << 30, 3),
+                "large-tiled-64-own-down": (0, 1 << 30, 1 << 30, 1 << 30, 4, (0, 1 << 30))}
 
 
 def _force_plan(eng, plan):
     if _TRUNK_PLANS[plan] is not None:
-        eng.skinny_rows, eng.fold_qkv_rows, eng.fold_o_rows, eng.fold_gu_rows, eng.gemm_config = _TRUNK_PLANS[plan]
+        eng.skinny_rows, eng.fold_qkv_rows, eng.fold_o_rows, eng.fold_gu_rows, eng.gemm_config = _TRUNK_PLANS[plan][:5]
+        if len(_TRUNK_PLANS[plan]) > 5:   # the down projection on this library's tiled GEMM too
+            eng.fold_down_rows = _TRUNK_PLANS[plan][5]
 
 
 @pytest.mark.parametrize("dtype,max_bar,mean_bar", [(torch.bfloat16, 0.15, 0.02), (torch.float16, 0.04, 0.005)])
@@ -380,7 +383,7 @@ def test_fused_qkv_decode_matches_unfused(dtype, name, over):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("plan", ["large-skinny-attn-block", "large-library", "large-tiled-64", "large-tiled-128"])
+@pytest.mark.parametrize("plan", ["large-skinny-attn-block", "large-library", "large-tiled-64", "large-tiled-128", "large-tiled-64-own-down"])
 def test_large_pass_plans_match_unfused(dtype, plan):
     """The launch plans of passes with many rows (forced here at 6 rows) against the unfused general path, to the same
     bounds as the small-pass plan above."""

@@ -90,7 +90,7 @@ def rms_norm_eps(dtype: torch.dtype) -> float:
 class UVEngine:
     def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 1 << 30, fold_o_rows: int = 1 << 30,
                  fold_gu_rows: int = 1 << 30, lean: bool = True, fold: bool = True, gemm_config: int = 0,
-                 tiled_prefill: bool = True, big_rows: int = 12288):
+                 tiled_prefill: bool = True, big_rows: int = 12288, fold_down_rows: tuple = (800, 1632)):
         """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens).
         skinny_rows: passes of at most this many rows run every projection on the skinny GEMM; fold_qkv_rows, fold_o_rows,
         fold_gu_rows: above skinny_rows, row counts up to which the QKV projection (with the pre-norm), the output
@@ -99,7 +99,8 @@ class UVEngine:
         the residual-add and norm launches (off: the general path); gemm_config: form of the hand-written GEMM (0: its own
         choice by size; tests force the tiled forms at a few rows); big_rows: passes of the general path with at least this
         many rows (a packed prefill, a mixed pass) run the down projection too on this library's GEMM, whose 256 x 256 tile
-        form is faster than the vendor library there (the other three projections run on it from 448 rows).  The defaults are the measured
+        form is faster than the vendor library there (the other three projections run on it from 448 rows); fold_down_rows:
+        (first, last) row count of decode passes whose down projection runs on this library's tiled GEMM.  The defaults are the measured
         optimum on UV-50M."""
         self.w, self.cfg = weights, weights.cfg
         cfg, dt, dev = self.cfg, weights.dtype, weights.device
@@ -128,6 +129,9 @@ class UVEngine:
         self.lean, self.fold, self.gemm_config = bool(lean), bool(fold), int(gemm_config)
         self.tiled_prefill = bool(tiled_prefill)
         self.big_rows = int(big_rows)
+        # the folded plan's down projection runs on this library's tiled GEMM between these row counts (measured inside the
+        # decode step: 4 - 11 us per step faster than the vendor library's there, slower below and above)
+        self.fold_down_rows = (int(fold_down_rows[0]), int(fold_down_rows[1]))
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -464,7 +468,10 @@ class UVEngine:
                 torch.mm(x, W["gu"].t(), out=b["gu"][:n])
                 self._swiglu_norm(x, n)
             # x <- resid_mlp * x + post_mlp * (act @ down.T)
-            torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
+            if sk_ok and self.fold_down_rows[0] <= n <= self.fold_down_rows[1] and cfg.d_ff % 64 == 0:
+                gemm_tn(b["act"][:n], W["down"], x, epilogue=RESID, resid=x, ca=W["resid_mlp"], cb=W["post_mlp"], config=gc)
+            else:
+                torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
         self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
         return xn
 
