@@ -125,6 +125,7 @@ _TRUNK_PLANS = {"small": None, "large-skinny-attn-block": (0, 1 << 30, 1 << 30, 
 def _force_plan(eng, plan):
     if _TRUNK_PLANS[plan] is not None:
         eng.skinny_rows, eng.fold_qkv_rows, eng.fold_o_rows, eng.fold_gu_rows, eng.gemm_config = _TRUNK_PLANS[plan][:5]
+        eng.general_skinny_rows = eng.skinny_rows   # the unfused path the plans are compared with runs the library's GEMMs too
         if len(_TRUNK_PLANS[plan]) > 5:   # the down projection on this library's tiled GEMM too
             eng.fold_down_rows = _TRUNK_PLANS[plan][5]
 

@@ -88,11 +88,12 @@ def rms_norm_eps(dtype: torch.dtype) -> float:
 
 
 class UVEngine:
-    def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 384, fold_qkv_rows: int = 1 << 30, fold_o_rows: int = 1 << 30,
+    def __init__(self, weights: UVWeights, max_tokens: int, skinny_rows: int = 192, fold_qkv_rows: int = 1 << 30, fold_o_rows: int = 1 << 30,
                  fold_gu_rows: int = 1 << 30, lean: bool = True, fold: bool = True, gemm_config: int = 0,
-                 tiled_prefill: bool = True, big_rows: int = 12288, fold_down_rows: tuple = (800, 1632)):
+                 tiled_prefill: bool = True, big_rows: int = 12288, fold_down_rows: tuple = (800, 1632), general_skinny_rows: int = 384):
         """max_tokens: largest number of token rows one forward call processes (decode rows + packed prefill tokens).
-        skinny_rows: passes of at most this many rows run every projection on the skinny GEMM; fold_qkv_rows, fold_o_rows,
+        skinny_rows: decode passes of at most this many rows run every projection on the skinny GEMM (general_skinny_rows:
+        the same for passes of the general path); fold_qkv_rows, fold_o_rows,
         fold_gu_rows: above skinny_rows, row counts up to which the QKV projection (with the pre-norm), the output
         projection (with the residual update) and the gate-up projection (with the pre-norm and the SwiGLU) run on this
         library's GEMM kernels instead of the vendor library's (see _trunk_folded); lean / fold: the launch plans that drop
@@ -118,10 +119,14 @@ class UVEngine:
         # post-processing to the attention kernel (one launch less per layer)
         self.fuse_qkv = dt in (torch.bfloat16, torch.float16) and cfg.n_heads // cfg.n_kv_heads <= 8 and cfg.n_pairs in (0, 16)
         self.qkvx_keep = None
-        # Passes of at most this many rows run their K = d_model projections on the skinny GEMM (the MLP's SwiGLU in its
-        # epilogue); above it, and for the down projection, the library GEMM is faster.  Measured on UV-50M decode steps:
-        # 0.544 -> 0.476 ms at 128 rows, 0.551 -> 0.523 at 256, 0.606 -> 0.589 at 384, slower from 512 on.
+        # Passes of at most this many rows run every projection on the skinny GEMM (the down projection with the block's
+        # second residual update in its epilogue); above it the folded plan (tiled GEMMs, the vendor library for the down
+        # projection).  Measured on UV-50M decode steps inside a rollout: 0.369 against 0.388 ms at 192 rows, 0.424 against
+        # 0.415 at 256, 0.466 against 0.460 at 320, equal at 384.
         self.skinny_rows = int(skinny_rows) if dt in (torch.bfloat16, torch.float16) else 0
+        # passes of the general path (prefill, mixed steps, layers without the fused attention) keep the skinny GEMM up to
+        # this many rows: their alternative below 448 rows is the vendor library with separate SwiGLU and norm launches
+        self.general_skinny_rows = int(general_skinny_rows) if dt in (torch.bfloat16, torch.float16) else 0
         # above skinny_rows the skinny kernel still carries the QKV projection (with the pre-norm) and the output projection
         # (with the residual update) up to these many rows
         self.fold_qkv_rows = int(fold_qkv_rows)
@@ -328,7 +333,8 @@ class UVEngine:
         assert n <= self.max_tokens
         self._embed_norm(tok, n)
         x, xn = b["x"][:n], b["xn"][:n]
-        skinny = n <= self.skinny_rows and cfg.d_model % 64 == 0 and cfg.d_model <= 960 and (cfg.n_heads * cfg.head_dim) % 64 == 0
+        skinny_rows = self.skinny_rows if fused_attn is not None else max(self.skinny_rows, self.general_skinny_rows)
+        skinny = n <= skinny_rows and cfg.d_model % 64 == 0 and cfg.d_model <= 960 and (cfg.n_heads * cfg.head_dim) % 64 == 0
         mm = (lambda a, w, out: gemm_tn(a, w, out)) if skinny else (lambda a, w, out: torch.mm(a, w.t(), out=out))
         # Small passes whose every layer takes the fused attention never need the normalised hidden in memory: the block's
         # second residual update then rides on the down projection and the next block's pre-norm on its QKV projection (a row
