@@ -53,6 +53,31 @@ def test_argument_errors_are_reported_not_thrown():
     assert lib.uvmi_decode_attn(None, None) == -1
 
 
+def test_gemm_capability_predicate_and_argument_checks():
+    """uvmi_gemm_tn_supported is host logic: 16-bit types, K in slabs of 64 up to 8192, N in fragments of 16 (32 for the
+    interleaved SwiGLU layout), pitches that keep 16-byte rows, 32-bit operand offsets.  The entry point refuses bad
+    arguments before it touches the device."""
+    from ultraviolet_amd import _lib
+    lib = _lib.lib()
+    F16, BF16, F32 = 0, 1, 2
+    ok = lambda *a: bool(lib.uvmi_gemm_tn_supported(*a))
+    assert ok(BF16, 2048, 656, 640, 640, 640, 656, 0) and ok(F16, 1, 16, 64, 64, 64, 16, 0)
+    assert ok(BF16, 33216, 3328, 640, 640, 640, 1664, 1)             # SWIGLU writes N / 2 columns
+    assert not ok(F32, 64, 64, 64, 64, 64, 64, 0)                    # 16-bit only
+    assert not ok(BF16, 64, 64, 96, 96, 96, 64, 0)                   # K % 64
+    assert not ok(BF16, 64, 64, 8256, 8256, 8256, 64, 0)             # K > 8192
+    assert not ok(BF16, 64, 24, 64, 64, 64, 24, 0)                   # N % 16
+    assert not ok(BF16, 64, 48, 64, 64, 64, 24, 1)                   # SWIGLU needs N % 32
+    assert not ok(BF16, 64, 64, 64, 60, 64, 64, 0)                   # lda < K
+    assert not ok(BF16, 64, 64, 64, 68, 64, 64, 0)                   # lda % 8
+    assert not ok(BF16, 64, 64, 64, 64, 64, 48, 0)                   # ldc < N
+    assert not ok(BF16, 65536, 64, 8192, 8192, 8192, 64, 0)          # operand offsets past 2^30 bytes
+    assert not ok(BF16, 64, 64, 64, 64, 64, 64, 3)                   # unknown epilogue
+    g = _lib.GemmArgs()
+    assert lib.uvmi_gemm_tn_ex(C.byref(g), None) == -1               # null pointers
+    assert lib.uvmi_gemm_tn_ex(None, None) == -1
+
+
 def test_no_cpu_fallback():
     import torch
     from ultraviolet_amd import _lib
