@@ -453,8 +453,12 @@ class UVEngine:
         sk_ok = cfg.d_model % 64 == 0 and (cfg.n_heads * cfg.head_dim) % 64 == 0
         sk_qkv, sk_o = sk_ok and n <= self.fold_qkv_rows, sk_ok and n <= self.fold_o_rows
         for l, W in enumerate(self.w.layers):
-            if l == 0:      # (the embedding's norm exists already: the same product as on the general path, bit for bit)
-                torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
+            if l == 0:      # (the embedding's norm exists already: the same product as on the general path, bit for bit -
+                            # the tiled GEMM of this library from 448 rows, where the general path takes it too)
+                if sk_qkv and n >= 448:
+                    gemm_tn(xn, W["wqkv_ext"], b["qkvx"][:n], config=gc)
+                else:
+                    torch.mm(xn, W["wqkv_ext"].t(), out=b["qkvx"][:n])
             elif sk_qkv:
                 gemm_tn(x, W["wqkv_ext"], b["qkvx"][:n], norm_eps=self.eps, config=gc)
             else:
