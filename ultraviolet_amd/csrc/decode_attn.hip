@@ -1125,6 +1125,8 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     // Waves per work item.  Long rows are streamed by all 4 waves of a workgroup, short ones by 2 or 1; and when 4 waves
     // per item would need more wave slots than the device has at this kernel's occupancy (4 per SIMD), 2 per item keep
     // the whole launch resident in one round instead of two (measured: 2000 rows x ~230 keys, 15.6 us against 18.9 us).
+    // Already from 4/5 of the slots on, 2 waves per item are the faster form (measured inside a 2048-sequence rollout, whose
+    // contexts are 800 - 1100 keys by then: steps of 832 - 1024 rows 0.589 - 0.607 ms against 0.609 - 0.621).
     const int ctx = a->window > 0 && a->window < a->S ? a->window : a->S;
     int wpr = ctx >= 256 ? 4 : (ctx >= 128 ? 2 : 1);
     {
@@ -1132,6 +1134,7 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
       if (cus <= 0) cus = 256;
       const int64_t slots = (int64_t)cus * 16;
       while (wpr > 1 && P.n_items * wpr > slots && P.n_items * (wpr / 2) <= slots) wpr /= 2;
+      if (wpr == 4 && P.n_items * 5 > slots) wpr = 2;
     }
     P.gran = 32 * wpr;
     if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
