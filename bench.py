@@ -41,23 +41,13 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from ultraviolet_amd.engine.workloads import c3_rollout, c5_requests as _c5_requests, fill_cache as _fill_cache  # noqa: E402
+
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch / algorithmic bytes per launch of the decode-attention kernel, from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/c5_attention_hbm_counters.md (FETCH_SIZE scaled x2.000 and WRITE_SIZE
 # x1.000 by what they read for a 1 GiB device copy).
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.10
-
-
-def _c5_requests(cfg, n_prompts=256, group=8, seed=0):
-    rng = np.random.default_rng(seed)
-    prompts, limits = [], []
-    for _ in range(n_prompts):
-        n = int(rng.integers(64, 257))
-        p = rng.integers(1, cfg.vocab_size, size=n).tolist()
-        for _ in range(group):
-            prompts.append(p)
-            limits.append(int(min(rng.geometric(1.0 / 600.0), 2048)))
-    return prompts, limits
 
 
 def _attn_bytes(pos, starts, window, B, H=8, hd=64):
@@ -331,16 +321,6 @@ def bench_c2(args):
                                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}))
 
 
-def _fill_cache(st, rows, ctx, gen):
-    """Materialise contexts without running a prefill: random int8 K/V and fp16 scales in every cache row, pos = ctx."""
-    for l in range(len(st.k)):
-        for c, sc in ((st.k[l], st.k_scale[l]), (st.v[l], st.v_scale[l])):
-            c.copy_(torch.randint(-127, 128, c.shape, device=c.device, dtype=torch.int8, generator=gen))
-            sc.copy_((torch.rand(sc.shape, device=c.device, generator=gen) * 0.02 + 0.005).half())
-    st.pos[rows] = ctx
-    st.starts[rows] = 0
-
-
 def bench_c4(args):
     """BASELINE configs[3]: mixed batch, 64 prompt chunks x 512 tokens + 448 decode rows, one forward pass per iteration."""
     from ultraviolet_amd.engine import KVState, UVEngine, UVWeights, make_config
@@ -413,30 +393,6 @@ def bench_c4(args):
                                  "prefill_attn_local_TFLOPs": round(fl_l / phases["prefill_attn_local_us"] / 1e6, 1),
                                  "prefill_attn_bwd_global_TFLOPs": round(2.5 * fl_g / phases["prefill_attn_bwd_global_us"] / 1e6, 1),
                                  "prefill_attn_bwd_local_TFLOPs": round(2.5 * fl_l / phases["prefill_attn_bwd_local_us"] / 1e6, 1)}}))
-
-
-def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0):
-    """The C3 workload as a Rollout ready to step: B running slots whose contexts U{128..2048} are materialised in the cache
-    (request ids 0..B-1, one token generated so far), Bernoulli(0.01) retirement per slot and step on the device, and a
-    queue of 64-token prompts (ids B, B + 1, ..) long enough for n_steps steps, admitted inside decode passes."""
-    from ultraviolet_amd.engine.rollout import Rollout
-    dev = eng.device
-    rng = np.random.default_rng(seed)
-    gen = torch.Generator(device=dev).manual_seed(seed)
-    g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + n_steps + 64, temperature=1.0, seed=seed, eos_id=None, check_every=4, bucket=128,
-                retire_p=0.01, mixed=True, admit_cap=24, overlap_harvest=True, use_graph=use_graph)
-    rows = torch.arange(B, device=dev)
-    _fill_cache(g.st, rows, torch.from_numpy(rng.integers(128, 2049, size=B)).to(dev), gen)
-    g.slot_req.copy_(rows)
-    g.slot_cnt.fill_(1)
-    g.slot_limit.fill_(g.max_new)
-    g.slot_tok.copy_(torch.from_numpy(rng.integers(1, cfg.vocab_size, size=B)).to(dev))
-    g.free, g.next_req, g.n_active_host = [], B, B
-    for r in range(B):
-        g.meta[r] = (r, 0)
-    for i in range(int(n_steps * B * 0.01 * 2) + 64):
-        g.add(rng.integers(1, cfg.vocab_size, size=64).tolist(), B + i)
-    return g
 
 
 def bench_c3(args):

@@ -6,7 +6,13 @@
  * allocates device memory, synchronises the device or throws: the return value is 0 on success or a negative
  * UVMI_E* code, and uvmi_last_error() returns a thread-local message for the last failure on this thread.
  * All launches go to the device that is current on the calling thread, so callers running a second Python
- * thread under another device (reference: scripts/rl_grpo.py:519-521) are served without global state.
+ * thread under another device (reference: scripts/rl_grpo.py:519-521) are served.  The library keeps no state
+ * between calls, with two stated exceptions: a per-thread cached compute-unit count, and uvmi_decode_attn_noalloc,
+ * which keeps a process-wide table of one device address per GPU (filled under a mutex on the first call on each
+ * device) and a scratch array in device memory that all its calls on one GPU share (see its declaration).
+ *
+ * uvmi_version() is the revision of this header's argument structs: it moves whenever a struct gains a field, so a
+ * caller built against an older header can tell that the layout it passes is no longer the one the library reads.
  *
  * Each declaration cites the reference interface it replaces (paths relative to the reference checkout).
  */
@@ -34,6 +40,8 @@ extern "C" {
 #define UVMI_I32 4
 #define UVMI_I64 5
 
+/* Revision of the argument structs below (uvmi_version() returns the value the library was built with). */
+#define UVMI_ABI_VERSION 3
 int uvmi_version(void);
 const char* uvmi_last_error(void);
 /* Number of compute units of the current device (used by the split heuristics); <0 on error. */

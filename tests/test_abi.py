@@ -23,7 +23,9 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/uvmi.h but not exported"
     assert set(_lib.EXPORTS) <= set(names)
-    assert lib.uvmi_version() >= 1
+    assert lib.uvmi_version() == _lib.ABI_VERSION
+    hdr = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "uvmi.h")).read()
+    assert int(re.search(r"#define UVMI_ABI_VERSION (\d+)", hdr).group(1)) == _lib.ABI_VERSION
 
 
 def test_host_only_entry_points():
@@ -238,3 +240,42 @@ def test_integration_doc_stub_matches_the_binding():
                     torch.zeros(2, 1, 32, dtype=torch.float16), torch.zeros(2, 1, 32, dtype=torch.float16), 1, torch.zeros(2, 8, 64), None)
     assert (a.B, a.H, a.KH, a.S, a.hd, a.q_dtype, a.kv_dtype, a.out_dtype, a.idx_dtype) == (2, 8, 1, 32, 64, 1, 3, 2, 5)
     assert _lib.lib().uvmi_decode_attn_path(C.byref(a)) == 1    # CPU pointers are never dereferenced by the path predicate
+
+
+def test_weight_stamp_is_stable_on_a_real_module():
+    """The stamp a patched model's methods compare must not move unless a parameter was written: nn.Module.state_dict()
+    returns fresh detached tensors on every call, so the stamp keys on the live parameters (address + version counter)."""
+    import torch
+    from ultraviolet_amd.kernels import fast_decode as fd
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Linear(4, 3)
+            self.register_buffer("b", torch.zeros(2))
+
+    m = Net()
+    assert [id(t) for t in m.state_dict().values()] != [id(t) for t in m.state_dict().values()]   # why ids cannot be used
+    s0 = fd._weights_stamp(m)
+    assert fd._weights_stamp(m) == s0 and fd._weights_stamp(m) == s0
+    fd._remember_stamp(m)
+    assert fd._quick_stamp(m) == m.__dict__["_uvmi_quick"]
+    with torch.no_grad():
+        m.a.weight.mul_(1.5)                      # an optimizer step
+    assert fd._weights_stamp(m) != s0 and fd._quick_stamp(m) != m.__dict__["_uvmi_quick"]
+    s1 = fd._weights_stamp(m)
+    assert fd._weights_stamp(m) == s1
+    with torch.no_grad():
+        m.b.add_(1.0)                             # buffers count too
+    assert fd._weights_stamp(m) != s1
+    # an object that only offers state_dict() without arguments (a dict of tensors) is stamped on its own tensors
+    class Plain:
+        def __init__(self):
+            self._sd = {"w": torch.zeros(3)}
+        def state_dict(self):
+            return self._sd
+    p = Plain()
+    s2 = fd._weights_stamp(p)
+    assert fd._weights_stamp(p) == s2
+    p._sd["w"].add_(1)
+    assert fd._weights_stamp(p) != s2

@@ -548,18 +548,24 @@ def test_streamgen_adapter_runs_the_reference_loop():
     for i, p in enumerate(prompts):
         g.add(p, i)
     res = []
+    raw = _StubModel(cfg, params)                              # the trainer's policy
     for it in range(200):
         if g.n_outstanding() == 0:
             break
         res += g.chunk()
-        if it == 1:
-            model._sd["blocks.0.attn.wq"].mul_(1.01)
+        if it == 1:                                            # an optimizer step, then the reference's two lines (rl_grpo.py:1308-1309)
+            raw._sd["blocks.0.attn.wq"].mul_(1.01)
+            perf.sync_weights_inplace(model, raw)
+            g.version += 1
+        if it == 3:                                            # a write straight into the generation model: picked up, not counted
+            model._sd["blocks.0.attn.wk"].mul_(1.01)
     res += g.harvest_end() if g.harvest_pending else []
     assert sorted(m for m, *_ in res) == list(range(len(prompts)))
     for meta, row, lp, v0 in res:
         assert len(row) == len(lp) and (row[-1] == 0 or len(row) == 12) and 0 not in row[:-1]
         assert np.isfinite(lp).all() and (lp <= 1e-6).all() and v0 in (0, 1)
     assert g.version == 1
+    torch.testing.assert_close(model._sd["blocks.0.attn.wq"], raw._sd["blocks.0.attn.wq"])
 
 
 def test_reference_op_name_runs_the_hip_kernels():

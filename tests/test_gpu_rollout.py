@@ -270,9 +270,10 @@ def test_rollout_mixed_sampled_with_random_retirement():
         assert same >= 38, (a, b_, same)
 
 
-def test_sync_weights_inplace_keeps_graphs_and_bumps_version():
+def test_sync_weights_inplace_keeps_graphs_and_version_is_the_callers():
     """New weights between chunks (scripts/rl_stream.py:22-36): tensors are overwritten in place so captured step graphs
-    keep working and pick the new weights up; requests admitted afterwards carry the new start version."""
+    keep working and pick the new weights up; the version counter is advanced by the caller, as the reference's loop does
+    (scripts/rl_grpo.py:1308-1309), and requests admitted afterwards carry the new start version."""
     from ultraviolet_amd.engine import random_params
     from ultraviolet_amd.engine.rollout import Rollout
     cfg, eng = _engine(torch.float32, window=32)
@@ -289,7 +290,9 @@ def test_sync_weights_inplace_keeps_graphs_and_bumps_version():
         if k.endswith(".wq") or k.endswith("w_up"):
             p2[k] = p2[k] * 1.05
     g.sync_weights_inplace(p2)
-    assert g.version == 1 and len(g.graphs) == n_graphs          # no residual scalar changed: graphs kept
+    assert g.version == 0                                        # the sync itself never counts
+    g.version += 1
+    assert len(g.graphs) == n_graphs                             # no residual scalar changed: graphs kept
     for i, p in enumerate(prompts[4:]):
         g.add(p, 4 + i)
     res = first + g.run(max_chunks=200)
@@ -305,7 +308,7 @@ def test_sync_weights_inplace_keeps_graphs_and_bumps_version():
     p3 = dict(p2)
     p3["blocks.0.resid_attn"] = np.float32(0.9)
     g.sync_weights_inplace(p3)
-    assert g.version == 2 and len(g.graphs) == 0                 # a launch-argument scalar changed: recapture
+    assert g.version == 1 and len(g.graphs) == 0                 # a launch-argument scalar changed: recapture
 
 
 def test_prompt_table_expansion_bit_exact():

@@ -21,8 +21,8 @@ def _uv50m(max_tokens):
 
 
 def _run_c3(eng, cfg, n_steps, use_graph):
-    import bench
-    g = bench.c3_rollout(eng, cfg, 512, n_steps, use_graph=use_graph)
+    from ultraviolet_amd.engine import workloads
+    g = workloads.c3_rollout(eng, cfg, 512, n_steps, use_graph=use_graph)
     ctx0 = g.st.pos.cpu().numpy().copy()
     if use_graph:
         g.precapture()
@@ -72,7 +72,7 @@ def test_c4_full_size_mixed_pass_equals_its_halves():
     prefill-only pass (the reference runs exactly those two passes, model.py:1296-1313, 1321-1330): final hidden states to a
     few units in the last place (the GEMMs run other tile shapes at other row counts), the same argmax, and identical int8
     bytes in layer 0, which sees no attention output."""
-    import bench
+    from ultraviolet_amd.engine import workloads
     from ultraviolet_amd.engine import KVState
     cfg, params, eng = _uv50m(64 * 512 + 512)
     rng = np.random.default_rng(0)
@@ -85,7 +85,7 @@ def test_c4_full_size_mixed_pass_equals_its_halves():
 
     def state():
         st = KVState(cfg, 512, 2048 + 64, DEV)
-        bench._fill_cache(st, rows_d, ctx, torch.Generator(device=DEV).manual_seed(0))
+        workloads.fill_cache(st, rows_d, ctx, torch.Generator(device=DEV).manual_seed(0))
         return st
 
     st_m, st_p, st_d = state(), state(), state()
@@ -120,11 +120,11 @@ def test_c5_long_rollout_sixteen_sequences_teacher_forced_through_the_oracle():
     groups that run longest the recorded tokens are fed through OracleModel(bf16) on the CPU - the reference's decode step
     restated, same int8 cache, same rounding points - and the behaviour log-probs the rollout recorded must match the
     oracle's log softmax(logits / T) of the same tokens (reference: tests/test_rl_stream.py:96-120)."""
-    import bench
+    from ultraviolet_amd.engine import workloads
     from oracle.model import OracleModel, OracleState
     from ultraviolet_amd.engine.rollout import Rollout
     cfg, params, eng = _uv50m(16384)
-    prompts, limits = bench._c5_requests(cfg)
+    prompts, limits = workloads.c5_requests(cfg)
     MAXN = 640
     limits = [min(l, MAXN) for l in limits]
     g = Rollout(eng, slots=2048, max_prompt=256, max_new=MAXN, temperature=1.0, seed=0, eos_id=None, check_every=16, bucket=128,

@@ -37,14 +37,22 @@ def _both(c, splits, out_dtype=torch.float32):
         a, keep = build_attn_args(c["q"], c["kq"], c["vq"], c["pos"], c["starts"], 0.14125, 0, False, c["ks"], c["vs"], splits, out)
         if entry.endswith("noalloc"):
             a.workspace, a.workspace_bytes = None, 0          # the entry point must not need it
-        before = torch.cuda.memory_allocated()
+        torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         rc = getattr(L.lib(), entry)(C.byref(a), L.stream_ptr(out))
         L.check(rc, entry)
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.memory_allocated() == before        # nothing through torch's allocator
         torch.cuda.synchronize()
+        if entry.endswith("noalloc") and _both.calls > 0:      # and nothing through hipMalloc either (the driver's free bytes;
+            assert torch.cuda.mem_get_info()[0] == free_before  # the first call on a device may look the scratch symbol up)
+        if entry.endswith("noalloc"):
+            _both.calls += 1
         outs.append(out.cpu())
         del keep
     return outs
+
+
+_both.calls = 0
 
 
 def test_noalloc_entry_matches_workspace_entry_twice_and_smaller():

@@ -119,6 +119,7 @@ class SampleCommit(C.Structure):
 
 
 _lib = None
+ABI_VERSION = 3   # UVMI_ABI_VERSION of include/uvmi.h
 
 
 def lib() -> C.CDLL:
@@ -129,6 +130,9 @@ def lib() -> C.CDLL:
         if not os.path.exists(LIB_PATH):
             raise UvmiError(f"{LIB_PATH} not found: run `python -m ultraviolet_amd.csrc.build` (no CPU fallback)")
         L = C.CDLL(LIB_PATH)
+        if L.uvmi_version() != ABI_VERSION:   # the ctypes structs below mirror one revision of include/uvmi.h
+            raise UvmiError(f"{LIB_PATH} was built for revision {L.uvmi_version()} of include/uvmi.h, these bindings are for "
+                            f"{ABI_VERSION}: rebuild it with `python -m ultraviolet_amd.csrc.build`")
         L.uvmi_last_error.restype = C.c_char_p
         L.uvmi_decode_attn_workspace_bytes.restype = C.c_size_t
         L.uvmi_decode_attn_workspace_bytes.argtypes = [C.c_int] * 5

@@ -13,7 +13,7 @@ void set_error(const char* fmt, ...) {
 }
 }  // namespace uvmi
 
-extern "C" int uvmi_version(void) { return 1; }
+extern "C" int uvmi_version(void) { return UVMI_ABI_VERSION; }
 extern "C" const char* uvmi_last_error(void) { return uvmi::g_err; }
 
 extern "C" int uvmi_device_cus(void) {

@@ -104,7 +104,8 @@ class Rollout:
         self.n_active_host = 0                    # upper bound on active slots (exact after each poll / admit)
         self.done_seen = 0
         self._dense_n = None                      # bucket the dense step arrays are valid for (None: stale, compact first)
-        self.version = 0
+        self.version = 0                          # advanced by the caller after each weight update (scripts/rl_grpo.py:1309)
+        self._scalar_epoch = getattr(self.e.w, "scalar_epoch", 0)
         self.n_decode_steps = 0
         self.n_tokens = 0
         self.n_prefill_tokens = 0                 # prompt tokens that went through a prefill pass of _admit (shared prompts once)
@@ -129,15 +130,23 @@ class Rollout:
 
     @torch.no_grad()
     def sync_weights_inplace(self, params: dict):
-        """New policy weights for the following steps (reference: sync_weights_inplace + the version counter of
-        StreamGen, scripts/rl_stream.py:22-36, 152-154): the fused tensors are overwritten in place, so captured step
-        graphs stay valid; they are only dropped when a residual scalar (a launch argument) changed.  Requests admitted
-        from now on carry the new version as their start_version."""
-        if self.e.w.load_(params):
+        """New policy weights for the following steps (reference: sync_weights_inplace, scripts/rl_stream.py:22-36): the
+        fused tensors are overwritten in place, so captured step graphs stay valid; they are only dropped when a residual
+        scalar (a launch argument) changed.  `version` is the caller's to advance, as in the reference's loop
+        (scripts/rl_grpo.py:1308-1309: sync_weights_inplace(gen_m, raw); gen.version += 1); requests admitted after that
+        carry the new value as their start_version."""
+        self.e.w.load_(params)
+        self._check_weight_epoch()
+        torch.cuda.synchronize(self.dev)
+
+    def _check_weight_epoch(self):
+        """Drop the captured graphs when the engine's weights were reloaded with different launch-argument scalars since the
+        graphs were captured - whoever reloaded them (this object, a patched model's refresh, perf.sync_weights_inplace)."""
+        ep = getattr(self.e.w, "scalar_epoch", 0)
+        if ep != self._scalar_epoch:
+            self._scalar_epoch = ep
             self.graphs.clear()
             self.mixed_graphs.clear()
-        torch.cuda.synchronize(self.dev)
-        self.version += 1
 
     # ------------------------------------------------------------------------------------------------ admission
     @torch.no_grad()

@@ -137,6 +137,7 @@ class UVWeights:
         if self.value_embed is not None:
             self.value_embed.copy_(value_embed)
         scalars_changed = False
+        self.epoch = getattr(self, "epoch", 0) + 1
         for old, new in zip(self.layers, layers):
             for k, v in new.items():
                 if isinstance(v, torch.Tensor):
@@ -144,6 +145,8 @@ class UVWeights:
                 elif v is not None and old[k] != v:
                     old[k] = v
                     scalars_changed = True
+        if scalars_changed:
+            self.scalar_epoch = getattr(self, "scalar_epoch", 0) + 1
         return scalars_changed
 
     @classmethod

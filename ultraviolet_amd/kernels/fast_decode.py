@@ -73,21 +73,50 @@ def kv_bytes_per_seq(cfg, ctx: int, kv_dtype: str = "int8") -> int:
     return sum(2 * c.n_kv_heads * 2 * c.head_dim * (ctx if c.is_global(l) else min(ctx, c.window)) for l in range(c.n_layers))
 
 
+def _live_tensors(model) -> dict:
+    """The model's parameters and buffers as the objects the model itself holds.  nn.Module.state_dict() hands out fresh
+    detached tensors on every call (their ids never repeat); keep_vars=True returns the live ones, whose storage address and
+    version counter identify the weights.  Objects whose state_dict takes no such argument (a plain dict of tensors behind a
+    state_dict() method) hold their tensors directly."""
+    try:
+        return dict(model.state_dict(keep_vars=True))
+    except TypeError:
+        return dict(model.state_dict())
+
+
 def _weights_stamp(model) -> tuple:
-    """Changes whenever a parameter of the model was written in place or replaced (torch bumps a tensor's version counter
-    on every in-place write - optimizer steps, copy_, sync_weights_inplace of scripts/rl_stream.py:22-36)."""
-    return tuple((id(t), t._version) for t in model.state_dict().values())
+    """Changes whenever a parameter of the model was written in place or replaced: (name, storage address, version counter)
+    of every live tensor (torch bumps the counter on every in-place write - optimizer steps, copy_, the parameter copy of
+    scripts/rl_stream.py:22-36).  Stable across calls when nothing was written."""
+    return tuple((k, t.data_ptr(), t._version) for k, t in _live_tensors(model).items())
 
 
-def _engine(model) -> UVEngine:
+def _quick_stamp(model) -> tuple:
+    """The version counters of the tensors seen by the last full stamp: what a decode step checks (a few dozen attribute
+    reads, no state_dict walk).  Replaced parameter objects are caught by the full stamp of the next prefill / chunk."""
+    return tuple(t._version for t in model.__dict__.get("_uvmi_live", ()))
+
+
+def _remember_stamp(model) -> None:
+    live = _live_tensors(model)
+    model.__dict__["_uvmi_live"] = tuple(live.values())
+    model.__dict__["_uvmi_stamp"] = tuple((k, t.data_ptr(), t._version) for k, t in live.items())
+    model.__dict__["_uvmi_quick"] = tuple(t._version for t in live.values())
+
+
+def _engine(model, full_check: bool = True) -> UVEngine:
     """The engine bound to a patched model, with its fused device weights brought up to date first: the reference's patched
     methods read the model's live fused weights (fast_decode.py:296-311), so a caller that updates the parameters in place
-    expects the next prefill / decode step to use them."""
+    expects the next prefill / decode step to use them.  full_check: walk state_dict (prefill, a generator's chunk);
+    otherwise only the version counters of the tensors seen by the last walk are compared (every decode step)."""
     eng = model.__dict__.get("_uvmi_engine")
     if eng is None:
         raise L.UvmiError("model has not been patched: call patch_model(model) first")
-    stamp = _weights_stamp(model)
-    if stamp != model.__dict__.get("_uvmi_stamp"):
+    if full_check:
+        stale = _weights_stamp(model) != model.__dict__.get("_uvmi_stamp")
+    else:
+        stale = _quick_stamp(model) != model.__dict__.get("_uvmi_quick")
+    if stale:
         sync_patched_weights(model)
     return eng
 
@@ -139,7 +168,7 @@ def decode_step_fast(self, tok: Tensor, st: KVState, g_len: int = 0, skip_attn: 
     return_hidden (the caller then runs the head GEMM and the fused sampler)."""
     assert not skip_attn, "skip_attn is a profiling switch of the reference and is not supported"
     assert backend in ("auto", "hip"), f"backend {backend!r}: this library has one backend"
-    eng = _engine(self)
+    eng = _engine(self, full_check=False)
     h = eng.decode_step(tok, st, num_splits)
     if hasattr(st, "host_pos"):
         st.host_pos += 1
@@ -177,7 +206,7 @@ def patch_model(model, kv_dtype: str | None = "fp16", num_splits: dict | None = 
         return decode_step_fast(self, tok, st, g_len, skip_attn, num_splits, backend)
 
     model.__dict__["_uvmi_engine"] = eng
-    model.__dict__["_uvmi_stamp"] = _weights_stamp(model)
+    _remember_stamp(model)
     model.__dict__["new_state"] = types.MethodType(new_state, model)
     model.__dict__["prefill"] = types.MethodType(prefill_fast, model)
     model.__dict__["decode_step"] = types.MethodType(decode_step, model)
@@ -185,7 +214,7 @@ def patch_model(model, kv_dtype: str | None = "fp16", num_splits: dict | None = 
 
 
 def unpatch_model(model):
-    for n in ("new_state", "prefill", "decode_step", "_uvmi_engine", "_uvmi_stamp"):
+    for n in ("new_state", "prefill", "decode_step", "_uvmi_engine", "_uvmi_stamp", "_uvmi_quick", "_uvmi_live"):
         model.__dict__.pop(n, None)
     return model
 
@@ -198,5 +227,5 @@ def sync_patched_weights(model) -> None:
     eng = model.__dict__.get("_uvmi_engine")
     if eng is None:
         raise L.UvmiError("model has not been patched: call patch_model(model) first")
-    eng.w.load_(model.state_dict())
-    model.__dict__["_uvmi_stamp"] = _weights_stamp(model)
+    eng.w.load_(_live_tensors(model))
+    _remember_stamp(model)

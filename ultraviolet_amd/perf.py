@@ -12,7 +12,7 @@ import torch
 
 from . import _lib as L
 from .engine.rollout import Rollout
-from .kernels.fast_decode import _engine, _weights_stamp, patch_model
+from .kernels.fast_decode import _engine, _weights_stamp, patch_model, sync_patched_weights
 from .kernels.fused_sample import fused_sample_ok
 
 PERF_FLAGS = {"lp", "hv", "rfh", "fz", "acc16", "pack", "head16", "pf", "pfc", "pkv"}
@@ -35,10 +35,13 @@ class StreamGen(Rollout):
                          check_every=check_every, bucket=min(row_bucket, slots), use_graph=use_graph, left_pad=True)
 
     def chunk(self):
-        stamp = _weights_stamp(self.m)   # parameters the trainer has written in place since the last chunk
-        if stamp != self.m.__dict__.get("_uvmi_stamp"):
-            self.sync_weights_inplace(self.m.state_dict())
-            self.m.__dict__["_uvmi_stamp"] = stamp
+        """StreamGen.chunk of the reference.  Parameters the trainer has written in place since the last chunk are brought
+        into the engine first (the reference's graphs read the live fused weights); `version` is left alone - it is the
+        caller's counter (scripts/rl_grpo.py:1309)."""
+        if _weights_stamp(self.m) != self.m.__dict__.get("_uvmi_stamp"):
+            sync_patched_weights(self.m)
+            torch.cuda.synchronize(self.dev)
+        self._check_weight_epoch()
         return super().chunk()
 
 
@@ -64,7 +67,24 @@ def install_fz(runner) -> bool:
 
 
 @torch.no_grad()
-def sync_weights_inplace(gen, raw) -> None:
-    """scripts/rl_stream.py:22-36: the policy `raw` (an object with state_dict() under the reference's parameter names)
-    becomes the generator's weights, in place, so captured step graphs keep reading the same tensors."""
-    gen.sync_weights_inplace(raw.state_dict())
+def sync_weights_inplace(gen_m, raw) -> None:
+    """sync_weights_inplace(gen_m, raw) of the reference (scripts/rl_stream.py:22-36): the policy `raw` becomes the weights
+    of the generation model `gen_m` - a model patch_model has bound - in place: its parameters are overwritten, and the
+    engine's fused device tensors are refreshed at their addresses, so captured step graphs keep reading the same tensors.
+    A StreamGen / Rollout is accepted in place of the model (its engine's weights are refreshed from raw.state_dict()).
+    As in the reference, the generator's `version` is not touched: the caller advances it (scripts/rl_grpo.py:1308-1309)."""
+    if isinstance(gen_m, Rollout):
+        gen_m.sync_weights_inplace(raw.state_dict())
+        return
+    if gen_m.__dict__.get("_uvmi_engine") is None:
+        raise L.UvmiError("sync_weights_inplace: the generation model has not been patched (patch_model) and is not a StreamGen")
+    if gen_m is not raw:
+        if hasattr(gen_m, "parameters") and hasattr(raw, "parameters"):
+            for pg, pt in zip(gen_m.parameters(), raw.parameters()):
+                pg.copy_(pt)
+        else:
+            src = raw.state_dict()
+            for k, t in gen_m.state_dict().items():
+                t.copy_(src[k])
+    sync_patched_weights(gen_m)
+    torch.cuda.synchronize(next(iter(gen_m.__dict__["_uvmi_live"])).device)
