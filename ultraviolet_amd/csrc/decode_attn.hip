@@ -73,7 +73,7 @@ __device__ __forceinline__ int load_idx32(const void* p, int is64, int64_t i) {
 }
 // own_key_apart: the key at the row's own position is not in the cache yet (the kernel forms it itself), so the streamed
 // range ends one position earlier.
-__device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b, bool own_key_apart = false) {
+__device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b, bool own_key_apart = false, bool uncut = false) {
   RowPlan r;
   const int pv = load_idx32(P.pos, P.idx64, b);
   const int st = load_idx32(P.starts, P.idx64, b);
@@ -90,6 +90,11 @@ __device__ __forceinline__ RowPlan plan_row(const AttnParams& P, int b, bool own
   r.a0 = lo & ~31;
   int span = p + 1 - r.a0;
   if (span < 0) span = 0;
+  if (uncut) {  // (known at compile time where it is set: the whole row is one chunk)
+    r.chunk = 0x3fffffff;
+    r.nsplit = 1;
+    return r;
+  }
   // (integer divisions by run-time values cost a few dozen instructions each, here on the way to the row's first tile
   // request: the granule is a power of two, and an uncut row - every decode step of the engine - divides by nothing)
   const int gr = P.gran;  // 32, 64 or 128
@@ -150,7 +155,8 @@ __device__ __forceinline__ f4 mfma_kv(const h8& a, const h8& b, f4 acc) {
 
 struct AttnState {
   f4 O[4];                // O''^T tiles: 2^-24 * sum (v + 128) P'
-  float mrun, lrun, psum; // running max (score units before scale), sum p, sum of the fp16-rounded P'
+  float mrun, lrun, psum; // reference point of the exponentials (score units before scale), sum p, sum of the fp16-rounded P'
+  float mthr;             // mrun + the slack a score may exceed it by before the reference point moves
 };
 
 // WPR waves of a workgroup share one work item (row, kv head, split): wave w takes super-tiles w, w + WPR, ... of the
@@ -166,11 +172,15 @@ struct AttnState {
 // KV16: the cache holds K / V unquantized in the q dtype (no scales): the same work split, plan, online softmax, merge and
 // epilogue around tiles that go into the MFMAs as they are loaded - no conversion, no bias terms, probabilities rounded to
 // the cache type (a tile is 32 dwords per lane, still 4 waves per SIMD).  Not combined with FUSE.
-template <int QDT, int ODT, int WPR, bool FUSE, bool KV16 = false>
+// FAST: the shape of the engine's decode step as compile-time constants - one kv head, 8 query heads, uncut rows, 64-bit
+// indices - so that the item arithmetic, the head masks, the split bookkeeping and the partial-result path fold away
+// (the fixed part of a wave's life is as long as its streaming loop on rows of a few hundred keys).
+template <int QDT, int ODT, int WPR, bool FUSE, bool KV16 = false, bool FAST = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_rows, const void* a_q, int64_t a_items, int a_idx64,
                        int a_splits, int a_kh, AttnParams P) {
   P.pos = a_pos; P.starts = a_starts; P.rows = a_rows; P.n_items = a_items; P.idx64 = a_idx64; P.splits = a_splits; P.KH = a_kh;
+  if constexpr (FAST) { P.idx64 = 1; P.splits = 1; P.KH = 1; P.G = 8; P.H = 8; P.hd = 64; P.chunk_keys = 0; }
   if (FUSE) P.f_qkv = a_q; else P.q = a_q;
   constexpr int IPB = 4 / WPR;  // items per block
   __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
@@ -235,7 +245,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   const float* pg_src = !FUSE && has_post && P.post_gate ? P.post_gate + (int64_t)b * P.H + hsafe : anyf;
   const float* px_src = has_post && P.post_xsa ? P.post_xsa + hsafe : anyf;
   const float pv_val = *pv_src, pg_val = *pg_src, px_val = *px_src;
-  const RowPlan rp = plan_row(P, b, FUSE);
+  const RowPlan rp = plan_row(P, b, FUSE, FAST);
   // FUSE: the row of the rotation table (cos / sin of the row's position per frequency, already rounded to the activation
   // type): prep_q reads its 32 values as scalars, the lane that owns dim d of the own key reads its own pair
   const int rope_row = rp.pc < 0 ? 0 : (rp.pc < P.f_rope_n ? rp.pc : P.f_rope_n - 1);
@@ -395,8 +405,11 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
 #pragma unroll
   for (int t = 0; t < 4; t++) st.O[t] = f4{0.f, 0.f, 0.f, 0.f};
   st.mrun = -INFINITY;
+  st.mthr = -INFINITY;
   st.lrun = 0.f;
   st.psum = 0.f;
+  constexpr float LAZY = 4.0f;           // log2 of the largest probability relative to the reference point
+  const float lazy_pre = LAZY / c;       // in score units before the softmax scale (c > 0, host-checked)
 
   // ---- addressing: wave-uniform row base + wave-uniform tile offset (scalar) + lane-invariant 32-bit offsets
   const int64_t cb = rp.cb;
@@ -523,9 +536,12 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       for (int i = 0; i < 4; i++)
         if (t0 + i < lo_eff || t0 + i >= s1) { t[i] = -INFINITY; vsf[i] = 0.f; }
     }
+    // The reference point of a column's exponentials only has to stay within 2^LAZY of its true maximum (probabilities up
+    // to 2^LAZY are as exact in fp16 / fp32 as those below 1), so the common tile compares each lane's own scores with
+    // the column's threshold and skips both the cross-lane maximum and the rescale.
     float mx = fmaxf(fmaxf(t[0], t[1]), fmaxf(t[2], t[3]));
-    mx = xmax32(xmax16(mx));
-    if (__builtin_amdgcn_ballot_w64(mx > st.mrun) != 0) {  // some column's maximum grew: rescale (alpha = 1 elsewhere)
+    if (__builtin_amdgcn_ballot_w64(mx > st.mthr) != 0) {  // some column outgrew its reference point: move it (alpha = 1 elsewhere)
+      mx = xmax32(xmax16(mx));
       const float mnew = fmaxf(st.mrun, mx);
       const float alpha = mnew == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((st.mrun - mnew) * c);
 #pragma unroll
@@ -533,6 +549,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       st.lrun *= alpha;
       st.psum *= alpha;
       st.mrun = mnew;
+      st.mthr = mnew + lazy_pre;   // (-inf stays -inf)
     }
     const float mc = st.mrun == -INFINITY ? 0.f : st.mrun * c;
     float p[4];
@@ -731,7 +748,7 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     }
   }
   if (strm == 0 && head < G) {
-    if (rp.nsplit == 1) {
+    if (FAST || rp.nsplit == 1) {
       if constexpr (FUSE) {
         if (rp.pc >= 0) {  // the own key joins the softmax after the streamed range
           const float s2 = sh_cur[wave][head] * c;
@@ -1149,9 +1166,18 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
   } while (0)
 #define UVMI_LF(QD)                                                                                   \
   do {                                                                                                \
-    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true>), grid, blk, 0, st, UVMI_LEAD, P);       \
+    if (fast && wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true, false, true>), grid, blk, 0, st, UVMI_LEAD, P);       \
+    else if (fast && wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true, false, true>), grid, blk, 0, st, UVMI_LEAD, P);  \
+    else if (fast) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true, false, true>), grid, blk, 0, st, UVMI_LEAD, P);              \
+    else if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true>), grid, blk, 0, st, UVMI_LEAD, P);  \
     else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true>), grid, blk, 0, st, UVMI_LEAD, P);  \
     else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true>), grid, blk, 0, st, UVMI_LEAD, P);                \
+  } while (0)
+#define UVMI_LFAST(QD)                                                                                \
+  do {                                                                                                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, false, false, true>), grid, blk, 0, st, UVMI_LEAD, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, false, false, true>), grid, blk, 0, st, UVMI_LEAD, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, false, false, true>), grid, blk, 0, st, UVMI_LEAD, P);               \
   } while (0)
 #define UVMI_L16(QD, OD)                                                                              \
   do {                                                                                                \
@@ -1160,6 +1186,8 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1, false, true>), grid, blk, 0, st, UVMI_LEAD, P);               \
   } while (0)
     const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
+    // the engine's decode-step shape has an instantiation of its own (see FAST)
+    const bool fast = !kv16 && a->num_splits == 1 && a->KH == 1 && a->H == 8 && a->idx_dtype == UVMI_I64;
     if (kv16) {
       if (a->q_dtype == UVMI_F16) {
         if (od == UVMI_F16) UVMI_L16(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L16(UVMI_F16, UVMI_BF16); else UVMI_L16(UVMI_F16, UVMI_F32);
@@ -1168,6 +1196,8 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
       }
     } else if (a->fuse) {
       if (a->q_dtype == UVMI_F16) UVMI_LF(UVMI_F16); else UVMI_LF(UVMI_BF16);
+    } else if (fast && od == a->q_dtype) {
+      if (a->q_dtype == UVMI_F16) UVMI_LFAST(UVMI_F16); else UVMI_LFAST(UVMI_BF16);
     } else if (a->q_dtype == UVMI_F16) {
       if (od == UVMI_F16) UVMI_L(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(UVMI_F16, UVMI_BF16); else UVMI_L(UVMI_F16, UVMI_F32);
     } else {
@@ -1175,6 +1205,7 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     }
 #undef UVMI_L
 #undef UVMI_LF
+#undef UVMI_LFAST
 #undef UVMI_L16
 #undef UVMI_LEAD
   } else {
