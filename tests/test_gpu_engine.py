@@ -318,6 +318,7 @@ def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 2
     step the fused state's caches are overwritten with the unfused ones so that differences do not accumulate.  Returns
     per-step hidden differences, argmax agreement of the logits and per-layer cache statistics."""
     from ultraviolet_amd.engine import KVState
+    _fused_vs_unfused.gaps = []
     prompts = _prompts(cfg, lens, seed=11)
     B = len(prompts)
     cont = np.random.default_rng(12).integers(1, cfg.vocab_size, size=(B, steps))
@@ -331,7 +332,12 @@ def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 2
         h1 = eng.decode_step(tok, sts[1], fuse=True).clone()
         assert torch.isfinite(h1.float()).all()
         hdiff.append(float((h0.float() - h1.float()).abs().max()))
-        agree.append(float((eng.logits(h0).argmax(-1) == eng.logits(h1).argmax(-1)).float().mean()))
+        lg0, lg1 = eng.logits(h0), eng.logits(h1)
+        same = lg0.argmax(-1) == lg1.argmax(-1)
+        agree.append(float(same.float().mean()))
+        if not bool(same.all()):   # where the two paths pick different tokens, the unfused path's own top-2 gap (a near-tie, or a bug)
+            top2 = lg0.topk(2, dim=-1).values
+            _fused_vs_unfused.gaps.append(float((top2[:, 0] - top2[:, 1])[~same].max()))
         for l in range(cfg.n_layers):
             for a, b_, sa, sb in ((sts[0].k[l], sts[1].k[l], sts[0].k_scale[l], sts[1].k_scale[l]),
                                   (sts[0].v[l], sts[1].v[l], sts[0].v_scale[l], sts[1].v_scale[l])):
@@ -344,6 +350,20 @@ def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 2
                     sb.copy_(sa)
     assert sts[0].pos.tolist() == sts[1].pos.tolist()
     return hdiff, agree, cmax, cfrac, sfrac
+
+
+_fused_vs_unfused.gaps = []
+
+
+def _check_agreement(agree, dtype):
+    """The two paths' hidden states differ by units in the last place, so their argmax differs wherever the model's own top
+    two logits are closer than that noise - often, on a randomly initialised model with 32 768 softcapped logits.  What must
+    hold: every disagreement sits at such a near-tie (the reference path's top-2 gap is of the size of the last-place noise
+    of a logit, not larger), and near-ties are a minority."""
+    gaps, _fused_vs_unfused.gaps = _fused_vs_unfused.gaps, []
+    noise = 0.08 if dtype == torch.bfloat16 else 0.02      # logits live in (0, 23): a few units in the last place of the hidden, through the head
+    assert all(g < noise for g in gaps), (max(gaps), noise)
+    assert np.mean(agree) > 0.8, np.mean(agree)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -380,7 +400,7 @@ def test_fused_qkv_decode_matches_unfused(dtype, name, over):
     assert (cmax <= 3 + np.arange(cfg.n_layers)).all(), cmax
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
-    assert np.mean(agree) > 0.9, np.mean(agree)
+    _check_agreement(agree, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -395,7 +415,7 @@ def test_large_pass_plans_match_unfused(dtype, plan):
     assert (cmax <= 3 + np.arange(cfg.n_layers)).all(), cmax
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
-    assert np.mean(agree) > 0.9, np.mean(agree)
+    _check_agreement(agree, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

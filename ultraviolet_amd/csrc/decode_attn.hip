@@ -183,8 +183,8 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   if constexpr (FAST) { P.idx64 = 1; P.splits = 1; P.KH = 1; P.G = 8; P.H = 8; P.hd = 64; P.chunk_keys = 0; }
   if (FUSE) P.f_qkv = a_q; else P.q = a_q;
   constexpr int IPB = 4 / WPR;  // items per block
-  __shared__ float sh_o[WPR > 1 ? 4 : 1][8][64];
-  __shared__ float sh_ml[WPR > 1 ? 4 : 1][8][2];
+  __shared__ __attribute__((aligned(16))) float sh_o[4][16][68];
+  __shared__ __attribute__((aligned(16))) float sh_ml[4][16][4];
   __shared__ float sh_post[4][80];  // epilogue operands of the item whose first wave this is: v_hat[64], gate[8], xsa[8]
   __shared__ float sh_cur[FUSE ? 4 : 1][72];  // own key of that item: score per head [8], dequantised v [64]
   __shared__ __attribute__((aligned(16))) uint16_t sh_q[FUSE ? 4 : 1][8][64];  // the item's q as fp16 operand words
@@ -696,134 +696,60 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       step(TT, tb, true);
     }
   }
-  // ---- reduce l and sum P' over the 4 lane groups, merge stream B into stream A (lanes n and n^8), undo the bias
-  float lsum = xsum32(xsum16(st.lrun)), ps = xsum32(xsum16(st.psum));
+  // ---- reduce l and sum P' over the 4 lane groups of a column
+  const float lsum = xsum32(xsum16(st.lrun)), ps = xsum32(xsum16(st.psum));
   const float m2 = st.mrun == -INFINITY ? -INFINITY : st.mrun * c;  // exp2 domain
-  // (lane ^ 8 is a rotation by 8 inside a row of 16 lanes: a DPP move on the vector ALU, where __shfl_xor would go through the LDS crossbar)
-  const float m_o = dpp_mov<0x128>(m2), l_o = dpp_mov<0x128>(lsum), ps_o = dpp_mov<0x128>(ps);
-  const float mm = fmaxf(m2, m_o);
-  const float ms = mm == -INFINITY ? 0.f : mm;
-  const float w_s = __builtin_amdgcn_exp2f(m2 - ms), w_o = __builtin_amdgcn_exp2f(m_o - ms);
-  const float lm = lsum * w_s + l_o * w_o;
-  const float pm = KV16 ? 0.f : 128.0f * (ps * w_s + ps_o * w_o);
-  const float w_s24 = KV16 ? w_s : w_s * 16777216.0f, w_o24 = KV16 ? w_o : w_o * 16777216.0f;
-  float o[16];  // head dims 16g .. 16g+15: O[t][i] is dim 16g + 4i + t
+  if (!FAST && rp.nsplit > 1) {
+    // ---- a chunk of a cut row: stream B is merged into stream A (lanes n and n ^ 8: a rotation by 8 inside a row of 16
+    // lanes, a DPP move), the WPR waves of the item through LDS, and the item's first wave writes the partial state
+    const float m_o = dpp_mov<0x128>(m2), l_o = dpp_mov<0x128>(lsum), ps_o = dpp_mov<0x128>(ps);
+    const float mm = fmaxf(m2, m_o);
+    const float ms = mm == -INFINITY ? 0.f : mm;
+    const float w_s = __builtin_amdgcn_exp2f(m2 - ms), w_o = __builtin_amdgcn_exp2f(m_o - ms);
+    const float lm = lsum * w_s + l_o * w_o;
+    const float pm = KV16 ? 0.f : 128.0f * (ps * w_s + ps_o * w_o);
+    const float w_s24 = KV16 ? w_s : w_s * 16777216.0f, w_o24 = KV16 ? w_o : w_o * 16777216.0f;
+    float o[16];  // head dims 16g .. 16g+15: O[t][i] is dim 16g + 4i + t
 #pragma unroll
-  for (int t = 0; t < 4; t++)
+    for (int t = 0; t < 4; t++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const float mine = st.O[t][i];
-      const float oth = dpp_mov<0x128>(mine);
-      o[4 * i + t] = (mine * w_s24 + oth * w_o24) - pm;
-    }
-  float mfin = mm, lfin = lm;
-  if (WPR > 1) {  // merge the WPR waves of this item through LDS; its first wave writes the result
-    if (strm == 0) {
-#pragma unroll
-      for (int i = 0; i < 4; i++) *(float4*)&sh_o[wave][head][16 * g + 4 * i] = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
-      if (g == 0) { sh_ml[wave][head][0] = mm; sh_ml[wave][head][1] = lm; }
-    }
-    __syncthreads();
-    if (wsub != 0 || !live) return;
-    if (strm == 0) {
-      float mw[WPR];
-      float mall = -INFINITY;
-#pragma unroll
-      for (int w = 0; w < WPR; w++) { mw[w] = sh_ml[wave + w][head][0]; mall = fmaxf(mall, mw[w]); }
-      const float msf = mall == -INFINITY ? 0.f : mall;
-      lfin = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; i++) o[i] = 0.f;
-#pragma unroll
-      for (int w = 0; w < WPR; w++) {
-        const float ww = __builtin_amdgcn_exp2f(mw[w] - msf);
-        lfin += ww * sh_ml[wave + w][head][1];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const float4 x = *(const float4*)&sh_o[wave + w][head][16 * g + 4 * i];
-          o[4 * i] += ww * x.x; o[4 * i + 1] += ww * x.y; o[4 * i + 2] += ww * x.z; o[4 * i + 3] += ww * x.w;
-        }
+      for (int i = 0; i < 4; i++) {
+        const float mine = st.O[t][i];
+        const float oth = dpp_mov<0x128>(mine);
+        o[4 * i + t] = (mine * w_s24 + oth * w_o24) - pm;
       }
-      mfin = mall;
-    }
-  }
-  if (strm == 0 && head < G) {
-    if (FAST || rp.nsplit == 1) {
-      if constexpr (FUSE) {
-        if (rp.pc >= 0) {  // the own key joins the softmax after the streamed range
-          const float s2 = sh_cur[wave][head] * c;
-          const float mnew = fmaxf(mfin, s2);
-          const float wa = mfin == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mfin - mnew), wb = __builtin_amdgcn_exp2f(s2 - mnew);
-          lfin = lfin * wa + wb;
+    float mfin = mm, lfin = lm;
+    if (WPR > 1) {
+      if (strm == 0) {
 #pragma unroll
-          for (int i = 0; i < 16; i++) o[i] = o[i] * wa + wb * sh_cur[wave][8 + 16 * g + i];
-          mfin = mnew;
-        }
+        for (int i = 0; i < 4; i++) *(float4*)&sh_o[wave][head][16 * g + 4 * i] = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+        if (g == 0) { sh_ml[wave][head][0] = mm; sh_ml[wave][head][1] = lm; }
       }
-      const float inv = lfin > 0.f ? 1.0f / lfin : 0.f;
-      const int64_t off = (int64_t)b * P.sob + (int64_t)(h * G + head) * P.soh + 16 * g;
-      if (has_post) {
-        // z (rounded to the q dtype, as the attention output tensor would be) -> XSA -> gate, written in the output type.
-        // All lanes of a head column (n, g = 0..3) are active here, so the cross-group swaps are well defined.
-        auto rnd = [&](float x, int dt) -> float {
-          return dt == UVMI_F32 ? x : (dt == UVMI_BF16 ? bf16_to_float(float_to_bf16(x)) : (float)(half_t)x);
-        };
-        const bool dead = FUSE && rp.pc < 0;  // padding row of the fused path: nothing was parked for it, the output is zero
-        float vv[16];
+      __syncthreads();
+      if (wsub != 0 || !live) return;
+      if (strm == 0) {
+        float mw[WPR];
+        float mall = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const float4 x = *(const float4*)&sh_post[wave][16 * g + 4 * i];
-          vv[4 * i] = dead ? 0.f : x.x; vv[4 * i + 1] = dead ? 0.f : x.y; vv[4 * i + 2] = dead ? 0.f : x.z; vv[4 * i + 3] = dead ? 0.f : x.w;
-        }
-        const float gate = dead ? 0.f : (FUSE || P.post_gate ? sh_post[wave][64 + head] : 1.0f);
-        float proj = 0.f;
+        for (int w = 0; w < WPR; w++) { mw[w] = sh_ml[wave + w][head][0]; mall = fmaxf(mall, mw[w]); }
+        const float msf = mall == -INFINITY ? 0.f : mall;
+        lfin = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          o[i] = rnd(o[i] * inv, QDT);
-          proj += o[i] * vv[i];
-        }
-        if (P.post_xsa) {
-          proj = xsum32(xsum16(proj));
-          const float ah = dead ? 0.f : sh_post[wave][72 + head] * proj;
+        for (int i = 0; i < 16; i++) o[i] = 0.f;
 #pragma unroll
-          for (int i = 0; i < 16; i++) o[i] = rnd(o[i] - ah * vv[i], QDT);
-        }
+        for (int w = 0; w < WPR; w++) {
+          const float ww = __builtin_amdgcn_exp2f(mw[w] - msf);
+          lfin += ww * sh_ml[wave + w][head][1];
 #pragma unroll
-        for (int i = 0; i < 16; i++) o[i] *= gate;
-        if (ODT == UVMI_F32) {
-          float* op = (float*)P.out + off;
-#pragma unroll
-          for (int i = 0; i < 4; i++) *(float4*)(op + 4 * i) = float4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
-        } else {
-          uint32_t w[8];
-#pragma unroll
-          for (int i = 0; i < 8; i++) {
-            const uint32_t l16 = ODT == UVMI_BF16 ? float_to_bf16(o[2 * i]) : float_to_half_bits(o[2 * i]);
-            const uint32_t h16 = ODT == UVMI_BF16 ? float_to_bf16(o[2 * i + 1]) : float_to_half_bits(o[2 * i + 1]);
-            w[i] = l16 | (h16 << 16);
+          for (int i = 0; i < 4; i++) {
+            const float4 x = *(const float4*)&sh_o[wave + w][head][16 * g + 4 * i];
+            o[4 * i] += ww * x.x; o[4 * i + 1] += ww * x.y; o[4 * i + 2] += ww * x.z; o[4 * i + 3] += ww * x.w;
           }
-          uint16_t* op = (uint16_t*)P.out + off;
-          *(uint4*)op = uint4{w[0], w[1], w[2], w[3]};
-          *(uint4*)(op + 8) = uint4{w[4], w[5], w[6], w[7]};
         }
-      } else if (ODT == UVMI_F32) {
-        float* op = (float*)P.out + off;
-#pragma unroll
-        for (int i = 0; i < 4; i++) *(float4*)(op + 4 * i) = float4{o[4 * i] * inv, o[4 * i + 1] * inv, o[4 * i + 2] * inv, o[4 * i + 3] * inv};
-      } else {
-        uint32_t w[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const float x0 = o[2 * i] * inv, x1 = o[2 * i + 1] * inv;
-          const uint32_t l16 = ODT == UVMI_BF16 ? float_to_bf16(x0) : float_to_half_bits(x0);
-          const uint32_t h16 = ODT == UVMI_BF16 ? float_to_bf16(x1) : float_to_half_bits(x1);
-          w[i] = l16 | (h16 << 16);
-        }
-        uint16_t* op = (uint16_t*)P.out + off;
-        *(uint4*)op = uint4{w[0], w[1], w[2], w[3]};
-        *(uint4*)(op + 8) = uint4{w[4], w[5], w[6], w[7]};
+        mfin = mall;
       }
-    } else {
+    }
+    if (strm == 0 && head < G) {
       const int64_t r = item * G + head;
       float* op = P.ws_o + r * 64 + 16 * g;
 #pragma unroll
@@ -832,6 +758,118 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
         P.ws_m[r] = mfin;
         P.ws_l[r] = lfin;
       }
+    }
+    return;
+  }
+  // ---- an uncut row: every wave parks its raw state in LDS - both streams' accumulators and (m, l, sum P') per column -
+  // and all lanes of the item's waves then share the merge and the epilogue: a thread owns NV consecutive dims of one head
+  // (with one wave per row 8, with four waves 2), merges the 2 WPR partial states of its dims, applies the epilogue and
+  // stores.  (Rows of sh_o are padded to 68 floats so that the 16 columns of a 16-byte access fall into different banks.)
+#pragma unroll
+  for (int i = 0; i < 4; i++) *(float4*)&sh_o[wave][m][16 * g + 4 * i] = float4{st.O[0][i], st.O[1][i], st.O[2][i], st.O[3][i]};
+  if (g == 0) *(float4*)&sh_ml[wave][m][0] = float4{m2, lsum, ps, 0.f};
+  if (WPR > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+  if (!live) return;
+  constexpr int NV = 8 / WPR, TPH = 64 / NV;       // values per thread, threads per head
+  const int ti = wsub * 64 + lane;
+  const int eh = ti / TPH, d0 = (ti % TPH) * NV;   // head and first dim of this thread
+  float mw[2 * WPR], mall = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < WPR; w++)
+#pragma unroll
+    for (int sx = 0; sx < 2; sx++) { mw[2 * w + sx] = sh_ml[iw + w][8 * sx + eh][0]; mall = fmaxf(mall, mw[2 * w + sx]); }
+  const float msf = mall == -INFINITY ? 0.f : mall;
+  float o[NV], lfin = 0.f, psf = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; j++) o[j] = 0.f;
+#pragma unroll
+  for (int w = 0; w < WPR; w++)
+#pragma unroll
+    for (int sx = 0; sx < 2; sx++) {
+      const float ww = __builtin_amdgcn_exp2f(mw[2 * w + sx] - msf);
+      lfin += ww * sh_ml[iw + w][8 * sx + eh][1];
+      psf += ww * sh_ml[iw + w][8 * sx + eh][2];
+      const float* src = &sh_o[iw + w][8 * sx + eh][d0];
+      if constexpr (NV == 8) {
+        const float4 x = *(const float4*)src, y = *(const float4*)(src + 4);
+        o[0] += ww * x.x; o[1] += ww * x.y; o[2] += ww * x.z; o[3] += ww * x.w; o[4] += ww * y.x; o[5] += ww * y.y; o[6] += ww * y.z; o[7] += ww * y.w;
+      } else if constexpr (NV == 4) {
+        const float4 x = *(const float4*)src;
+        o[0] += ww * x.x; o[1] += ww * x.y; o[2] += ww * x.z; o[3] += ww * x.w;
+      } else {
+        const float2 x = *(const float2*)src;
+        o[0] += ww * x.x; o[1] += ww * x.y;
+      }
+    }
+  if constexpr (!KV16) {  // undo the 2^-24 of the subnormal V operand and its +128 bias
+    const float pm = 128.0f * psf;
+#pragma unroll
+    for (int j = 0; j < NV; j++) o[j] = o[j] * 16777216.0f - pm;
+  }
+  float mfin = mall;
+  if constexpr (FUSE) {
+    if (rp.pc >= 0) {  // the own key joins the softmax after the streamed range
+      const float s2 = sh_cur[iw][eh] * c;
+      const float mnew = fmaxf(mfin, s2);
+      const float wa = mfin == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mfin - mnew), wb = __builtin_amdgcn_exp2f(s2 - mnew);
+      lfin = lfin * wa + wb;
+#pragma unroll
+      for (int j = 0; j < NV; j++) o[j] = o[j] * wa + wb * sh_cur[iw][8 + d0 + j];
+      mfin = mnew;
+    }
+  }
+  const float inv = lfin > 0.f ? 1.0f / lfin : 0.f;
+  if (has_post) {
+    // z (rounded to the q dtype, as the attention output tensor would be) -> XSA -> gate, written in the output type.
+    // The TPH threads of a head are consecutive lanes of one wave, all active, so the cross-lane sums are well defined.
+    auto rnd = [&](float x, int dt) -> float {
+      return dt == UVMI_F32 ? x : (dt == UVMI_BF16 ? bf16_to_float(float_to_bf16(x)) : (float)(half_t)x);
+    };
+    const bool dead = FUSE && rp.pc < 0;  // padding row of the fused path: nothing was parked for it, the output is zero
+    float vv[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) vv[j] = dead ? 0.f : sh_post[iw][d0 + j];
+    const float gate = dead ? 0.f : (FUSE || P.post_gate ? sh_post[iw][64 + eh] : 1.0f);
+    float proj = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      o[j] = rnd(o[j] * inv, QDT);
+      proj += o[j] * vv[j];
+    }
+    if (P.post_xsa) {
+      proj += lane_xor1(proj); proj += lane_xor2(proj); proj += lane_xor4(proj);
+      if constexpr (TPH >= 16) proj += lane_xor8(proj);
+      if constexpr (TPH >= 32) proj += lane_xor16(proj);
+      const float ah = dead ? 0.f : sh_post[iw][72 + eh] * proj;
+#pragma unroll
+      for (int j = 0; j < NV; j++) o[j] = rnd(o[j] - ah * vv[j], QDT);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++) o[j] *= gate;
+  } else {
+#pragma unroll
+    for (int j = 0; j < NV; j++) o[j] *= inv;
+  }
+  if (eh < G) {
+    const int64_t off = (int64_t)b * P.sob + (int64_t)(h * G + eh) * P.soh + d0;
+    if constexpr (ODT == UVMI_F32) {
+      float* op = (float*)P.out + off;
+      if constexpr (NV == 2) *(float2*)op = float2{o[0], o[1]};
+      else
+#pragma unroll
+        for (int j = 0; j < NV; j += 4) *(float4*)(op + j) = float4{o[j], o[j + 1], o[j + 2], o[j + 3]};
+    } else {
+      uint32_t w[NV / 2];
+#pragma unroll
+      for (int j = 0; j < NV / 2; j++) {
+        const uint32_t l16 = ODT == UVMI_BF16 ? float_to_bf16(o[2 * j]) : float_to_half_bits(o[2 * j]);
+        const uint32_t h16 = ODT == UVMI_BF16 ? float_to_bf16(o[2 * j + 1]) : float_to_half_bits(o[2 * j + 1]);
+        w[j] = l16 | (h16 << 16);
+      }
+      uint16_t* op = (uint16_t*)P.out + off;
+      if constexpr (NV == 8) *(uint4*)op = uint4{w[0], w[1], w[2], w[3]};
+      else if constexpr (NV == 4) *(uint2*)op = uint2{w[0], w[1]};
+      else *(uint32_t*)op = w[0];
     }
   }
 }
