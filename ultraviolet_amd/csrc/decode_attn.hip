@@ -1190,6 +1190,15 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
       const int64_t slots = (int64_t)cus * 16;
       while (wpr > 1 && P.n_items * wpr > slots && P.n_items * (wpr / 2) <= slots) wpr /= 2;
       if (wpr == 4 && P.n_items * 5 > slots) wpr = 2;
+      // Rows of a known, short length - a window or ring of at most 512 keys, 16 tiles - are a chain of latencies rather than
+      // a stream: they run fastest with about one wave per SIMD (measured on 256-key rings: 4 waves per row up to ~300 rows,
+      // 2 up to ~650, 1 beyond; 500 rows 6.1 us with 2 against 6.9 with 4, 1000 rows 9.5 us with 1 against 9.8 with 2).  With
+      // the fused QKV post-processing two waves keep sharing the row's own key and value up to the full device (1000 rows
+      // 11.9 us with 2 against 12.5 with 1).
+      if ((a->ring || (a->window > 0 && a->window < a->S)) && ctx <= 512) {
+        if (wpr == 4 && P.n_items * 4 > (int64_t)cus * 5) wpr = 2;
+        if (wpr == 2 && !a->fuse && P.n_items * 2 > (int64_t)cus * 5) wpr = 1;
+      }
     }
     P.gran = 32 * wpr;
     if (P.chunk_keys) P.chunk_keys = (P.chunk_keys + P.gran - 1) / P.gran * P.gran;
