@@ -406,7 +406,7 @@ def bench_c3(args):
     B = 512
     K = args.steps if args.steps > 0 else 256
     W = args.warmup
-    g = c3_rollout(eng, cfg, B, W + K)
+    g = c3_rollout(eng, cfg, B, W + K, device_admit=not args.host_admit)
     g.precapture()
 
     def run(n):
@@ -436,7 +436,10 @@ def bench_c3(args):
                                              "cache, Bernoulli(0.01) retirement per slot and step on the device, 64-token prompts admitted into "
                                              "freed slots inside decode passes, harvest every 4 steps (its results taken one step later)",
                                  "tokens_timed": gen_tok, "mixed_steps": g.n_mixed_steps - m0, "requests_finished": g.next_req - len(g.meta),
-                                 "active_at_end": g.n_active(), "full_slot_tok_per_s": round(B * steps / dt, 1)}}))
+                                 "active_at_end": g.n_active(), "mean_active_slots": round(gen_tok / steps, 1),
+                                 "admission": "host: free list and queue in Python" if args.host_admit else
+                                              "device: uvmi_sched_plan_admit takes staged prompts and reusable slots itself",
+                                 "full_slot_tok_per_s": round(B * steps / dt, 1)}}))
 
 
 def bench_copy(args):
@@ -467,6 +470,7 @@ def main():
     ap.add_argument("--steps", type=int, default=0, help="timed decode steps (0: the whole rollout after warm-up)")
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy"])
+    ap.add_argument("--host-admit", action="store_true", help="c3: the host chooses the slots of admitted prompts (default: the device does)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (rollouts shard by sequence with no communication between ranks); "

@@ -41,7 +41,7 @@ extern "C" {
 #define UVMI_I64 5
 
 /* Revision of the argument structs below (uvmi_version() returns the value the library was built with). */
-#define UVMI_ABI_VERSION 3
+#define UVMI_ABI_VERSION 4
 int uvmi_version(void);
 const char* uvmi_last_error(void);
 /* Number of compute units of the current device (used by the split heuristics); <0 on error. */
@@ -396,6 +396,13 @@ typedef struct uvmi_sched_state {
   int32_t* counters;    /* [0] active slots at the last compact, [1] completion records written, [2] bucket overflow flag */
   int64_t max_new; int64_t eos_id; /* eos_id < 0: none */
   int B; int done_cap;
+  /* Device-side admission (optional; all NULL / 0 when the host chooses the slots itself).  slot_hold: a slot that retires
+   * is held (1) until uvmi_sched_harvest has packed its output row, and only then becomes reusable - uvmi_sched_plan_admit
+   * never hands out a held slot.  The admission queue is a ring of q_cap staged prompts, q_stride int64 each:
+   * [length, request id, length limit, tokens ...]; q_ctl[0] = prompts staged so far (written by the host after the rows,
+   * on the launch stream), q_ctl[1] = prompts admitted so far, q_ctl[2] = prompts admitted by the last plan. */
+  int32_t* slot_hold; int64_t* q_buf; int64_t* q_ctl;
+  int q_cap; int q_stride;
 } uvmi_sched_state;
 
 /* List the active slots (ascending) and gather their token, position, start, request id and token index into dense
@@ -439,11 +446,34 @@ int uvmi_sched_admit(const uvmi_sched_state* s, int n, const int64_t* slots, con
 int uvmi_sched_expand(const uvmi_sched_state* s, int n_adm, int n_tokens, const int64_t* cu_seqlens, const int64_t* adm_slot,
                       const int64_t* adm_start, int64_t* pos_t, int64_t* row_t, int64_t* last_t, int64_t* last_idx, void* stream);
 
+/* The admission of a step decided on the device - the free-slot choice and the FIFO queue that the reference keeps in
+ * host Python (StreamGen._refill, scripts/rl_stream.py:76-93; generate_continuous' refill, ultraviolet/model.py:1293-1314).
+ * Takes prompts from the head of the staged ring while a reusable slot (slot_req < 0, not held) is left, at most admit_cap
+ * prompts and n_tokens packed tokens, and binds them to the free slots in ascending slot order.  Writes the step's admission
+ * tables - cu_seqlens (admit_cap + 1 entries, unused ones repeat the total), slot (-1 unused), start position (left_pad:
+ * longest admitted prompt - own length, else 0), length limit and request id per prompt - and the prompts' tokens packed
+ * back to back into tok_packed (n_tokens entries, zero filled), then advances q_ctl[1].  The tables are what
+ * uvmi_sched_expand and uvmi_sched_admit take, so a step that admits prompts needs nothing from the host but the launch.
+ * One workgroup. */
+int uvmi_sched_plan_admit(const uvmi_sched_state* s, int admit_cap, int n_tokens, int left_pad, int64_t* adm_cu, int64_t* adm_slot,
+                          int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req, int64_t* tok_packed, void* stream);
+
+/* uvmi_sched_compact, uvmi_sched_plan_admit and uvmi_sched_expand of a step that admits prompts in one launch (one
+ * workgroup): everything the step's kernels need - the dense arrays of the decode rows, the admission tables, the packed
+ * prompt tokens and their per-token position / cache row / last position tables - without a word from the host.
+ * last_c (optional, n_bucket entries): the decode rows' positions once more, as the "last position" column of a pass
+ * that runs prompt tokens and decode rows together. */
+int uvmi_sched_step_plan(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c, int64_t* starts_c,
+                         int64_t* req_c, int64_t* cnt_c, int admit_cap, int n_tokens, int left_pad, int64_t* adm_cu, int64_t* adm_slot,
+                         int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req, int64_t* tok_packed, int64_t* pos_t, int64_t* row_t,
+                         int64_t* last_t, int64_t* last_idx, int64_t* last_c, void* stream);
+
 /* Pack the completion records seen .. min(seen + max_rows, counters[1]) - 1 (seen = records the host has already taken)
  * and the output rows of their slots, so that the host harvests with one copy of the header and one of exactly the
- * finished tokens.  hdr (4 + 4 max_rows int64): [0..2] = counters[0..2], [3] = k, the records packed; then for packed
+ * finished tokens.  hdr (8 + 4 max_rows int64): [0..2] = counters[0..2], [3] = k, the records packed; then for packed
  * record j: request id, slot, token count (clamped to max_new), offset of its tokens in tok_dst / lp_dst (rows back to
- * back in record order).  tok_dst, lp_dst: max_rows * max_new elements; lp_dst may be NULL.  Replaces the whole-buffer
+ * back in record order); after the records, at 4 + 4 max_rows: the number of active slots at this point of the stream,
+ * q_ctl[1] and q_ctl[2] (0 without a queue).  With slot_hold the packed slots are released for reuse.  tok_dst, lp_dst: max_rows * max_new elements; lp_dst may be NULL.  Replaces the whole-buffer
  * .cpu() and the host loop over rows of StreamGen.chunk (scripts/rl_stream.py:126-143; ultraviolet/model.py:1321-1335). */
 int uvmi_sched_harvest(const uvmi_sched_state* s, int64_t seen, int max_rows, int64_t* hdr, int32_t* tok_dst,
                        float* lp_dst, void* stream);

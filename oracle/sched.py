@@ -7,6 +7,11 @@ EOS, inclusive (rl_stream.py:131-138); finished rows are parked at position 0 (m
 clamped to the buffer width (rl_stream.py:122).  The reference tests a row only every check_every steps and discards
 what it decoded past the end; retiring at the exact step returns the same rows.
 
+Device-side admission (plan_admit / harvest with holds) restates the refill policy of the same loops - idle rows are
+refilled from the head of a FIFO queue (rl_stream.py:76-93; model.py:1293-1314) - with two choices the reference leaves to
+Python list order made explicit: free slots are handed out in ascending order, and a slot whose finished row has not been
+harvested yet is not handed out.
+
 Pinned by: the invariants of the reference's tests (every request returned once, rows EOS-terminated or exactly limit
 long: tests/test_rl_stream.py:82-94) and brute-force comparison with a straight-line per-request loop in
 tests/test_oracle_sched.py.
@@ -30,10 +35,13 @@ class SlotTable:
         self.out_tok = np.zeros((B, max_new), np.int32)
         self.out_lp = np.zeros((B, max_new), np.float32)
         self.done: list[tuple[int, int, int]] = []   # (request, slot, count)
+        self.hold = np.zeros(B, np.int32)            # finished, output row not harvested yet: not reusable
+        self.harvested = 0                           # completion records already packed
 
     def _finish(self, slot, req, cnt):
         self.done.append((int(req), int(slot), int(cnt)))
         self.req[slot] = -1
+        self.hold[slot] = 1
         self.pos[slot] = 0
         self.starts[slot] = 0
 
@@ -69,6 +77,46 @@ class SlotTable:
                 fin = float(philox.request_uniform(seed, int(self.req[s]), c, philox.DOMAIN_RETIRE)) < np.float32(retire_p)
             if fin:
                 self._finish(s, self.req[s], c + 1)
+
+
+    def harvest(self, max_rows: int):
+        """Pack the next completion records (at most max_rows) and release their slots: [(request, slot, count, tokens,
+        log-probs)]."""
+        out = []
+        for req, slot, cnt in self.done[self.harvested:self.harvested + max_rows]:
+            c = min(cnt, self.max_new)
+            out.append((req, slot, c, self.out_tok[slot, :c].copy(), self.out_lp[slot, :c].copy()))
+            self.hold[slot] = 0
+        self.harvested += len(out)
+        return out
+
+    def plan_admit(self, queue, head: int, admit_cap: int, n_tokens: int, left_pad: bool):
+        """The admission of one step: queue[head:] are the staged prompts in arrival order, each (tokens, request id, limit).
+        Prompts are taken from the head while a reusable slot is left (not active, not held), at most admit_cap prompts and
+        n_tokens packed tokens; the k-th admitted prompt gets the k-th free slot in ascending order.  Returns the tables of
+        the step: cu_seqlens (admit_cap + 1, unused entries repeat the total), slot (-1 unused), start, limit, request id
+        per prompt, the packed tokens (zero filled), and the new head."""
+        free = [s for s in range(self.B) if self.req[s] < 0 and not self.hold[s]][:admit_cap]
+        na, ntok, lens = 0, 0, []
+        while na < len(free) and head + na < len(queue):
+            n = len(queue[head + na][0])
+            if ntok + n > n_tokens:
+                break
+            ntok += n
+            lens.append(n)
+            na += 1
+        tmax = max(lens, default=0)
+        cu = np.full(admit_cap + 1, ntok, np.int64)
+        cu[:na + 1] = np.concatenate([[0], np.cumsum(lens)]) if na else [0]
+        slot = np.full(admit_cap, -1, np.int64)
+        start, limit, req = (np.zeros(admit_cap, np.int64) for _ in range(3))
+        tok = np.zeros(n_tokens, np.int64)
+        for a in range(na):
+            ids, r, lim = queue[head + a]
+            slot[a], limit[a], req[a] = free[a], lim, r
+            start[a] = tmax - lens[a] if left_pad else 0
+            tok[cu[a]:cu[a + 1]] = ids
+        return cu, slot, start, limit, req, tok, head + na
 
 
 def expand_prompts(cu, slots, starts, n_tokens: int):

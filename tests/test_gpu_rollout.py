@@ -37,7 +37,7 @@ def test_slot_table_kernels_bit_exact(B, bucket, retire_p):
     nxt = 0
     dense = [torch.zeros(bucket, dtype=torch.long, device=DEV) for _ in range(6)]
     hv_rows, seen, harvested = 5, 0, []
-    hv_hdr = torch.zeros(4 + 4 * hv_rows, dtype=torch.long, device=DEV)
+    hv_hdr = torch.zeros(8 + 4 * hv_rows, dtype=torch.long, device=DEV)
     hv_tok, hv_lp = torch.zeros(hv_rows * max_new, dtype=torch.int32, device=DEV), torch.zeros(hv_rows * max_new, dtype=torch.float32, device=DEV)
     for step in range(30):
         free = np.nonzero(tab.req < 0)[0]
@@ -480,3 +480,114 @@ def test_shared_prompts_are_prefilled_once_and_copied(dtype, left_pad):
         assert outs[0][3 * grp] == outs[0][3 * grp + 1] == outs[0][3 * grp + 2]
     same = sum(outs[0][i] == outs[1][i] for i in range(12))
     assert same >= (12 if dtype == torch.float32 else 9), same
+
+
+@pytest.mark.parametrize("B,A,Np,left", [(8, 3, 40, False), (100, 8, 128, True), (1500, 24, 1536, False), (2048, 16, 700, True)])
+def test_plan_admit_kernel_bit_exact(B, A, Np, left):
+    """uvmi_sched_plan_admit against the oracle's policy on random slot tables and queues: the admission tables (cu_seqlens,
+    slots, starts, limits, request ids), the packed tokens and the queue head, bit for bit; held and active slots are never
+    handed out; the ring wraps."""
+    from oracle.sched import SlotTable
+    from ultraviolet_amd import _lib as L
+    lib = L.lib()
+    max_prompt, q_cap = 70, 16
+    stride = max_prompt + 3
+    rng = np.random.default_rng(B + A)
+    t, s = _dev_table(B, 8, 1)
+    hold = torch.zeros(B, dtype=torch.int32, device=DEV)
+    q_buf, q_ctl = torch.zeros(q_cap, stride, dtype=torch.long, device=DEV), torch.zeros(4, dtype=torch.long, device=DEV)
+    s.slot_hold, s.q_buf, s.q_ctl, s.q_cap, s.q_stride = hold.data_ptr(), q_buf.data_ptr(), q_ctl.data_ptr(), q_cap, stride
+    tab = SlotTable(B, 8, 1)
+    queue, head, tail = [], 0, 0
+    out = [torch.zeros(n, dtype=torch.long, device=DEV) for n in (A + 1, A, A, A, A, Np)]
+    tt = lambda a, dt=torch.long: torch.as_tensor(np.asarray(a), dtype=dt, device=DEV)
+    for step in range(40):
+        # a random table: mostly busy, some free, some of the free ones held
+        busy = rng.random(B) < rng.choice([0.5, 0.9, 0.99, 1.0]) if B > 50 else rng.random(B) < rng.choice([0.2, 0.6, 1.0])
+        tab.req[:] = np.where(busy, rng.integers(0, 1 << 40, size=B), -1)
+        tab.hold[:] = (~busy) & (rng.random(B) < 0.3)
+        t["slot_req"].copy_(tt(tab.req))
+        hold.copy_(tt(tab.hold, torch.int32))
+        for _ in range(int(rng.integers(0, q_cap - (tail - head) + 1))):    # stage more prompts (never over what is not admitted yet)
+            ids = rng.integers(1, 30000, size=int(rng.integers(1, min(max_prompt, Np) + 1))).tolist()   # (a prompt always fits a step's budget)
+            item = (ids, (1 << 35) + tail, int(rng.integers(1, 9)))
+            queue.append(item)
+            row = np.zeros(stride, np.int64)
+            row[0], row[1], row[2] = len(ids), item[1], item[2]
+            row[3:3 + len(ids)] = ids
+            q_buf[tail % q_cap].copy_(tt(row))
+            tail += 1
+        q_ctl[0] = tail
+        L.check(lib.uvmi_sched_plan_admit(C.byref(s), A, Np, int(left), *[o.data_ptr() for o in out], None), "plan_admit")
+        cu, slot, start, limit, req, tok, new_head = tab.plan_admit(queue, head, A, Np, left)
+        for name, got, want in zip(("cu", "slot", "start", "limit", "req", "tok"), out, (cu, slot, start, limit, req, tok)):
+            assert np.array_equal(got.cpu().numpy(), want), (step, name)
+        assert q_ctl.tolist()[:3] == [tail, new_head, new_head - head]
+        # the one-launch form of a step's bookkeeping: compaction + this plan + the prompts' per-token tables
+        q_ctl[1] = head
+        bucket = max(8, -(-B // 8) * 8)
+        dense = [torch.zeros(bucket, dtype=torch.long, device=DEV) for _ in range(6)]
+        out2 = [torch.zeros_like(o) for o in out]
+        tabs = [torch.full((Np,), 7, dtype=torch.long, device=DEV) for _ in range(3)] + [torch.full((A,), 7, dtype=torch.long, device=DEV)]
+        last_c = torch.full((bucket,), 7, dtype=torch.long, device=DEV)
+        t["pos"].copy_(tt(rng.integers(0, 90, size=B)))
+        L.check(lib.uvmi_sched_step_plan(C.byref(s), bucket, *[d.data_ptr() for d in dense], A, Np, int(left), *[o.data_ptr() for o in out2],
+                                         *[x.data_ptr() for x in tabs], last_c.data_ptr(), None), "step_plan")
+        for got, want in zip(out2, out):
+            assert torch.equal(got, want)
+        dense1 = [torch.zeros(bucket, dtype=torch.long, device=DEV) for _ in range(6)]
+        tabs1 = [torch.zeros(Np, dtype=torch.long, device=DEV) for _ in range(3)] + [torch.zeros(A, dtype=torch.long, device=DEV)]
+        pos_before, st_before = t["pos"].clone(), t["starts"].clone()
+        pos_after, st_after = t["pos"].clone(), t["starts"].clone()      # (step_plan has set the admitted slots' pos / starts)
+        L.check(lib.uvmi_sched_compact(C.byref(s), bucket, *[d.data_ptr() for d in dense1], None), "compact")
+        L.check(lib.uvmi_sched_expand(C.byref(s), A, Np, out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(), *[x.data_ptr() for x in tabs1],
+                                      None), "expand")
+        for got, want in zip(dense + tabs, dense1 + tabs1):
+            assert torch.equal(got, want)
+        assert torch.equal(last_c, dense[2]) and torch.equal(t["pos"], pos_after) and torch.equal(t["starts"], st_after)
+        assert q_ctl.tolist()[:3] == [tail, new_head, new_head - head]
+        na = new_head - head
+        got_slots = out[1].cpu().numpy()[:na]
+        assert (tab.req[got_slots] < 0).all() and (tab.hold[got_slots] == 0).all()
+        head = new_head
+    assert head > q_cap                                        # the ring wrapped at least once
+
+
+def test_rollout_device_admission_equals_host_admission():
+    """The rollout with the queue and the free-slot choice on the device (device_admit) returns what the host-managed
+    driver returns - greedy streams per request, every request once, limits respected - graph-replayed and eager, with and
+    without the overlapped harvest; start versions follow the caller's counter at the admitting step."""
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg, eng = _engine(torch.float32, window=32)
+    rng = np.random.default_rng(14)
+    prompts = [rng.integers(2, cfg.vocab_size, size=int(rng.integers(3, 30))).tolist() for _ in range(30)]
+    limits = [int(rng.integers(1, 21)) for _ in prompts]
+    ref = Rollout(eng, slots=6, max_prompt=32, max_new=20, temperature=0.0, check_every=3, bucket=4, mixed=True)
+    for i, p in enumerate(prompts):
+        ref.add(p, i, limit=limits[i])
+    want = {m: row for m, row, _, _ in ref.run(max_chunks=500)}
+    for use_graph, overlap in ((True, False), (False, False), (True, True)):
+        g = Rollout(eng, slots=6, max_prompt=32, max_new=20, temperature=0.0, check_every=3, bucket=4, mixed=True, admit_cap=4,
+                    device_admit=True, use_graph=use_graph, overlap_harvest=overlap)
+        for i, p in enumerate(prompts[:20]):
+            g.add(p, i, limit=limits[i])
+        res, bumped = [], False
+        for it in range(500):
+            if g.n_outstanding() == 0:
+                break
+            res += g.chunk()
+            if it == 2:                                        # more requests arrive later; the caller's counter moves
+                for i, p in enumerate(prompts[20:]):
+                    g.add(p, 20 + i, limit=limits[20 + i])
+                g.version += 1
+                bumped = True
+        res += g.harvest_end() if g.harvest_pending else []
+        got = {m: row for m, row, _, _ in res}
+        assert sorted(got) == list(range(30)) and len(res) == 30 and bumped
+        assert all(len(got[i]) == limits[i] for i in range(30))
+        same = sum(got[i] == want[i] for i in range(30))
+        assert same >= 27, (use_graph, overlap, same)          # near-ties may flip under a different batch composition
+        v0 = {m: v for m, _, _, v in res}
+        assert set(v0.values()) <= {0, 1} and all(v0[i] == 1 for i in range(20, 30)) and v0[0] == 0
+        assert g.n_mixed_steps > 0 and int(g.slot_hold.sum()) == 0 and (g.slot_req < 0).all()
+        assert g.q_ctl.tolist()[:2] == [30, 30]

@@ -20,9 +20,9 @@ def _uv50m(max_tokens):
     return cfg, params, UVEngine(UVWeights(cfg, params, torch.bfloat16, DEV), max_tokens=max_tokens)
 
 
-def _run_c3(eng, cfg, n_steps, use_graph):
+def _run_c3(eng, cfg, n_steps, use_graph, device_admit=False):
     from ultraviolet_amd.engine import workloads
-    g = workloads.c3_rollout(eng, cfg, 512, n_steps, use_graph=use_graph)
+    g = workloads.c3_rollout(eng, cfg, 512, n_steps, use_graph=use_graph, device_admit=device_admit)
     ctx0 = g.st.pos.cpu().numpy().copy()
     if use_graph:
         g.precapture()
@@ -36,21 +36,26 @@ def _run_c3(eng, cfg, n_steps, use_graph):
     return g, ctx0, done
 
 
-def test_c3_full_size_churn_properties_and_graph_equals_eager():
-    """BASELINE configs[2] at its size for 64+ steps (reference semantics: scripts/rl_stream.py:105-146,
+@pytest.mark.parametrize("device_admit", [False, True])
+def test_c3_full_size_churn_properties_and_graph_equals_eager(device_admit):
+    """BASELINE configs[2] at its size for 64+ steps, with the admission queue and the free-slot choice on the host and on
+    the device (reference semantics: scripts/rl_stream.py:105-146,
     tests/test_rl_stream.py:82-94): every request is returned exactly once or still holds a slot; a returned row is as long
     as its token count; a slot's position is its context plus the tokens it generated; freed slots are refilled from the
     queue in order; and the graph-replayed run equals the eagerly launched one token for token."""
     cfg, params, eng = _uv50m(2048)
     runs = []
     for use_graph in (True, False):
-        g, ctx0, done = _run_c3(eng, cfg, 72, use_graph)
+        g, ctx0, done = _run_c3(eng, cfg, 72, use_graph, device_admit)
         req, cnt, pos = g.slot_req.cpu().numpy(), g.slot_cnt.cpu().numpy(), g.st.pos.cpu().numpy()
         live = req >= 0
         returned = [m for m, *_ in done]
         assert len(returned) == len(set(returned))                                   # exactly once
         assert set(returned).isdisjoint(req[live].tolist())
-        assert sorted(returned + req[live].tolist()) == list(range(g.next_req))     # admitted ids are 0 .. next_req - 1, FIFO
+        n_adm = 512 + int(g.q_ctl[1]) if device_admit else g.next_req                # (device: ids are given at staging)
+        assert sorted(returned + req[live].tolist()) == list(range(n_adm))           # admitted ids are 0 .. n_adm - 1, FIFO
+        if device_admit:                                                             # no slot handed out while its row waited
+            assert int(g.slot_hold.sum()) == 0 and (g.slot_hold[torch.as_tensor(live, device=DEV)] == 0).all()
         assert g.n_mixed_steps > 10 and len(returned) > 150                           # churn happened: ~5 retirements per step
         for m, row, lp, _ in done:
             assert len(row) == len(lp) >= 1 and all(0 <= t < cfg.vocab_size for t in row) and np.isfinite(lp).all()

@@ -110,7 +110,8 @@ class SchedState(C.Structure):
     _fields_ = [("slot_req", C.c_void_p), ("slot_cnt", C.c_void_p), ("slot_limit", C.c_void_p), ("slot_tok", C.c_void_p),
                 ("pos", C.c_void_p), ("starts", C.c_void_p), ("out_tok", C.c_void_p), ("out_lp", C.c_void_p),
                 ("done_req", C.c_void_p), ("done_slot", C.c_void_p), ("done_cnt", C.c_void_p), ("counters", C.c_void_p),
-                ("max_new", C.c_int64), ("eos_id", C.c_int64), ("B", C.c_int), ("done_cap", C.c_int)]
+                ("max_new", C.c_int64), ("eos_id", C.c_int64), ("B", C.c_int), ("done_cap", C.c_int),
+                ("slot_hold", C.c_void_p), ("q_buf", C.c_void_p), ("q_ctl", C.c_void_p), ("q_cap", C.c_int), ("q_stride", C.c_int)]
 
 
 class SampleCommit(C.Structure):
@@ -119,7 +120,7 @@ class SampleCommit(C.Structure):
 
 
 _lib = None
-ABI_VERSION = 3   # UVMI_ABI_VERSION of include/uvmi.h
+ABI_VERSION = 4   # UVMI_ABI_VERSION of include/uvmi.h
 
 
 def lib() -> C.CDLL:
@@ -173,6 +174,9 @@ def lib() -> C.CDLL:
                                        C.c_void_p]
         L.uvmi_sched_expand.argtypes = [C.POINTER(SchedState), C.c_int, C.c_int] + [C.c_void_p] * 8
         L.uvmi_sched_harvest.argtypes = [C.POINTER(SchedState), C.c_int64, C.c_int] + [C.c_void_p] * 4
+        L.uvmi_sched_plan_admit.argtypes = [C.POINTER(SchedState), C.c_int, C.c_int, C.c_int] + [C.c_void_p] * 7
+        L.uvmi_sched_step_plan.argtypes = ([C.POINTER(SchedState), C.c_int] + [C.c_void_p] * 6 + [C.c_int, C.c_int, C.c_int] +
+                                           [C.c_void_p] * 12)
         L.uvmi_rope_table.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
         L.uvmi_gemm_tn_supported.argtypes = [C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int]
         L.uvmi_gemm_tn_ex.argtypes = [C.POINTER(GemmArgs), C.c_void_p]
@@ -204,4 +208,4 @@ EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_
            "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_decode_attn_noalloc", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu", "uvmi_swiglu_norm",
-           "uvmi_prefill_attn_bwd", "uvmi_prefill_attn_bwd_workspace_bytes", "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_commit_dense", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]
+           "uvmi_prefill_attn_bwd", "uvmi_prefill_attn_bwd_workspace_bytes", "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_commit_dense", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_sched_plan_admit", "uvmi_sched_step_plan", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]

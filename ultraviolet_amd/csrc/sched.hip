@@ -19,10 +19,8 @@
 namespace uvmi {
 
 // One workgroup of 1024 threads; slots are handled in tiles of 1024 with a running base (ordered compaction).
-__global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, int64_t* tok_c,
-                                                             int64_t* pos_c, int64_t* starts_c, int64_t* req_c, int64_t* cnt_c) {
-  __shared__ int wsum[16];
-  __shared__ int base_sh;
+__device__ __forceinline__ void compact_phase(const uvmi_sched_state& S, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c,
+                                              int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, int* wsum, int& base_sh) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   if (tid == 0) base_sh = 0;
   __syncthreads();
@@ -63,6 +61,14 @@ __global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S,
     S.counters[0] = n_act;                              // active slots seen by this step
     if (n_act > n_bucket) S.counters[2] = 1;            // bucket too small: the overflow slots idle this step
   }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(1024) void sched_compact_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, int64_t* tok_c,
+                                                             int64_t* pos_c, int64_t* starts_c, int64_t* req_c, int64_t* cnt_c) {
+  __shared__ int wsum[16];
+  __shared__ int base_sh;
+  compact_phase(S, n_bucket, act_slot, tok_c, pos_c, starts_c, req_c, cnt_c, wsum, base_sh);
 }
 
 // One thread per dense row (see commit_row).
@@ -93,8 +99,140 @@ __global__ __launch_bounds__(256) void sched_admit_kernel(uvmi_sched_state S, in
     const int k = atomicAdd(&S.counters[1], 1) % S.done_cap;
     S.done_req[k] = req_ids[i]; S.done_slot[k] = slot; S.done_cnt[k] = 1;
     S.slot_req[slot] = -1;
+    if (S.slot_hold) S.slot_hold[slot] = 1;
     S.pos[slot] = 0;
     S.starts[slot] = 0;
+  }
+}
+
+// The admission of a step planned on the device (see uvmi_sched_plan_admit): one workgroup of 1024 threads.  Phase 1 lists
+// the first admit_cap reusable slots in ascending order (ballot / popcount prefix over tiles of 1024 slots, as the
+// compaction does); phase 2 (one thread) walks the staged ring from its head while slots, the prompt cap and the token
+// budget last; phase 3 (all threads) writes the tables and copies the admitted prompts' tokens back to back.
+constexpr int PLAN_MAXA = 256;
+struct PlanShared {
+  int wsum[16];
+  int base, na, tmax;
+  int free_slot[PLAN_MAXA];
+  int cu[PLAN_MAXA + 1];
+};
+
+__device__ __forceinline__ void plan_phase(const uvmi_sched_state& S, int A, int n_tokens, int left_pad, int64_t* adm_cu, int64_t* adm_slot,
+                                           int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req, int64_t* tok_packed, PlanShared& sh) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) sh.base = 0;
+  __syncthreads();
+  for (int t0 = 0; t0 < S.B && sh.base < A; t0 += 1024) {
+    const int slot = t0 + tid;
+    const bool fr = slot < S.B && S.slot_req[slot] < 0 && !(S.slot_hold && S.slot_hold[slot]);
+    const unsigned long long bal = __ballot(fr);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) sh.wsum[wave] = __popcll(bal);
+    __syncthreads();
+    int woff = 0;
+    for (int w = 0; w < wave; w++) woff += sh.wsum[w];
+    const int base = sh.base;
+    if (fr && base + woff + before < A) sh.free_slot[base + woff + before] = slot;
+    __syncthreads();
+    if (tid == 0) {
+      int tot = 0;
+      for (int w = 0; w < 16; w++) tot += sh.wsum[w];
+      sh.base = base + tot;
+    }
+    __syncthreads();
+  }
+  const int64_t head = S.q_ctl[1], tail = S.q_ctl[0];
+  __syncthreads();   // (every thread has read the head before one thread moves it)
+  if (tid == 0) {
+    const int nfree = sh.base < A ? sh.base : A;
+    int na = 0, ntok = 0, tmax = 0;
+    sh.cu[0] = 0;
+    while (na < nfree && head + na < tail) {
+      const int64_t* row = S.q_buf + ((head + na) % S.q_cap) * (int64_t)S.q_stride;
+      int len = (int)row[0];
+      len = len < 0 ? 0 : (len > S.q_stride - 3 ? S.q_stride - 3 : len);
+      if (ntok + len > n_tokens) break;
+      ntok += len;
+      tmax = len > tmax ? len : tmax;
+      sh.cu[++na] = ntok;
+    }
+    sh.na = na;
+    sh.tmax = tmax;
+    S.q_ctl[1] = head + na;
+    S.q_ctl[2] = na;
+  }
+  __syncthreads();
+  const int na = sh.na, total = sh.cu[na];
+  for (int a = tid; a <= A; a += 1024) adm_cu[a] = a <= na ? sh.cu[a] : total;
+  for (int a = tid; a < A; a += 1024) {
+    const bool ok = a < na;
+    const int64_t* row = S.q_buf + ((head + (ok ? a : 0)) % S.q_cap) * (int64_t)S.q_stride;
+    adm_slot[a] = ok ? sh.free_slot[a] : -1;
+    adm_start[a] = ok && left_pad ? sh.tmax - (sh.cu[a + 1] - sh.cu[a]) : 0;
+    adm_limit[a] = ok ? row[2] : 0;
+    adm_req[a] = ok ? row[1] : 0;
+  }
+  // tokens: packed token i belongs to the prompt a with cu[a] <= i < cu[a + 1] (binary search, na <= 256)
+  for (int i = tid; i < n_tokens; i += 1024) {
+    int64_t v = 0;
+    if (i < total) {
+      int lo = 0, hi = na;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (sh.cu[mid] <= i) lo = mid; else hi = mid;
+      }
+      v = S.q_buf[((head + lo) % S.q_cap) * (int64_t)S.q_stride + 3 + (i - sh.cu[lo])];
+    }
+    tok_packed[i] = v;
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(1024) void sched_plan_admit_kernel(uvmi_sched_state S, int A, int n_tokens, int left_pad, int64_t* adm_cu,
+                                                                int64_t* adm_slot, int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req,
+                                                                int64_t* tok_packed) {
+  __shared__ PlanShared sh;
+  plan_phase(S, A, n_tokens, left_pad, adm_cu, adm_slot, adm_start, adm_limit, adm_req, tok_packed, sh);
+}
+
+// The whole bookkeeping ahead of a step that admits prompts, in one launch of one workgroup: the compaction of the active
+// slots, the admission plan, and the per-token tables of the admitted prompts (what uvmi_sched_compact, uvmi_sched_plan_admit
+// and uvmi_sched_expand do in three).
+__global__ __launch_bounds__(1024) void sched_step_plan_kernel(uvmi_sched_state S, int n_bucket, int64_t* act_slot, int64_t* tok_c,
+                                                               int64_t* pos_c, int64_t* starts_c, int64_t* req_c, int64_t* cnt_c, int A,
+                                                               int n_tokens, int left_pad, int64_t* adm_cu, int64_t* adm_slot,
+                                                               int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req, int64_t* tok_packed,
+                                                               int64_t* pos_t, int64_t* row_t, int64_t* last_t, int64_t* last_idx, int64_t* last_c) {
+  __shared__ PlanShared sh;
+  compact_phase(S, n_bucket, act_slot, tok_c, pos_c, starts_c, req_c, cnt_c, sh.wsum, sh.base);
+  if (last_c)   // a decode row's own position is the last position it may attend (and append at)
+    for (int i = threadIdx.x; i < n_bucket; i += 1024) last_c[i] = pos_c[i];
+  plan_phase(S, A, n_tokens, left_pad, adm_cu, adm_slot, adm_start, adm_limit, adm_req, tok_packed, sh);
+  const int tid = threadIdx.x, na = sh.na;
+  for (int a = tid; a < A; a += 1024) {
+    const bool ok = a < na && sh.cu[a + 1] > sh.cu[a];
+    last_idx[a] = ok ? sh.cu[a + 1] - 1 : 0;
+    if (ok) {
+      const int slot = sh.free_slot[a], st = left_pad ? sh.tmax - (sh.cu[a + 1] - sh.cu[a]) : 0;
+      S.starts[slot] = st;
+      S.pos[slot] = st + (sh.cu[a + 1] - sh.cu[a]);
+    }
+  }
+  const int total = sh.cu[na];
+  for (int i = tid; i < n_tokens; i += 1024) {
+    int64_t p = 0, r = -1, l = 0;
+    if (i < total) {
+      int lo = 0, hi = na;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (sh.cu[mid] <= i) lo = mid; else hi = mid;
+      }
+      const int st = left_pad ? sh.tmax - (sh.cu[lo + 1] - sh.cu[lo]) : 0;
+      p = st + (i - sh.cu[lo]);
+      r = sh.free_slot[lo];
+      l = st + (sh.cu[lo + 1] - sh.cu[lo]) - 1;
+    }
+    pos_t[i] = p; row_t[i] = r; last_t[i] = l;
   }
 }
 
@@ -138,6 +276,21 @@ __global__ __launch_bounds__(256) void sched_harvest_kernel(uvmi_sched_state S, 
   int64_t k = (int64_t)S.counters[1] - seen;
   k = k < 0 ? 0 : (k > max_rows ? max_rows : k);
   if (j == 0 && tid < 4) hdr[tid] = tid < 3 ? (int64_t)S.counters[tid] : k;
+  if (j == gridDim.x - 1) {   // the last workgroup (never one with a long copy ahead of it) counts the active slots
+    int64_t n = 0;
+    for (int s0 = tid; s0 < S.B; s0 += 256) n += S.slot_req[s0] >= 0;
+    for (int o = 32; o > 0; o >>= 1) n += __shfl_xor(n, o, 64);
+    if ((tid & 63) == 0) wsum[tid >> 6] = n;
+    __syncthreads();
+    if (tid == 0) {
+      int64_t* x = hdr + 4 + 4 * (int64_t)max_rows;
+      x[0] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+      x[1] = S.q_ctl ? S.q_ctl[1] : 0;
+      x[2] = S.q_ctl ? S.q_ctl[2] : 0;
+      x[3] = 0;
+    }
+    __syncthreads();
+  }
   if (j >= k) return;
   auto count_of = [&](int64_t rec) {
     const int64_t c = S.done_cnt[rec % S.done_cap];
@@ -165,6 +318,10 @@ __global__ __launch_bounds__(256) void sched_harvest_kernel(uvmi_sched_state S, 
   for (int64_t t = tid; t < cnt; t += 256) {
     tok_dst[off + t] = src_t[t];
     if (lp_dst && src_l) lp_dst[off + t] = src_l[t];
+  }
+  if (S.slot_hold && ok) {   // the row is packed: the slot may be handed out again
+    __syncthreads();
+    if (tid == 0) S.slot_hold[slot] = 0;
   }
 }
 
@@ -237,6 +394,36 @@ extern "C" int uvmi_sched_expand(const uvmi_sched_state* s, int n_adm, int n_tok
   hipLaunchKernelGGL(sched_expand_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, *s, n_adm, n_tokens, cu_seqlens, adm_slot,
                      adm_start, pos_t, row_t, last_t, last_idx);
   UVMI_CHECK_LAUNCH("uvmi_sched_expand");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_plan_admit(const uvmi_sched_state* s, int admit_cap, int n_tokens, int left_pad, int64_t* adm_cu, int64_t* adm_slot,
+                                     int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req, int64_t* tok_packed, void* stream) {
+  int rc = check_state(s, "uvmi_sched_plan_admit");
+  if (rc) return rc;
+  UVMI_REQUIRE(s->q_buf && s->q_ctl && s->q_cap > 0 && s->q_stride > 3, UVMI_EINVAL, "uvmi_sched_plan_admit: the state has no admission queue");
+  UVMI_REQUIRE(admit_cap > 0 && admit_cap <= 256 && n_tokens > 0 && adm_cu && adm_slot && adm_start && adm_limit && adm_req && tok_packed,
+               UVMI_EINVAL, "uvmi_sched_plan_admit: bad arguments (admit_cap 1..256)");
+  hipLaunchKernelGGL(sched_plan_admit_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, *s, admit_cap, n_tokens, left_pad ? 1 : 0, adm_cu,
+                     adm_slot, adm_start, adm_limit, adm_req, tok_packed);
+  UVMI_CHECK_LAUNCH("uvmi_sched_plan_admit");
+  return UVMI_OK;
+}
+
+extern "C" int uvmi_sched_step_plan(const uvmi_sched_state* s, int n_bucket, int64_t* act_slot, int64_t* tok_c, int64_t* pos_c, int64_t* starts_c,
+                                    int64_t* req_c, int64_t* cnt_c, int admit_cap, int n_tokens, int left_pad, int64_t* adm_cu, int64_t* adm_slot,
+                                    int64_t* adm_start, int64_t* adm_limit, int64_t* adm_req, int64_t* tok_packed, int64_t* pos_t,
+                                    int64_t* row_t, int64_t* last_t, int64_t* last_idx, int64_t* last_c, void* stream) {
+  int rc = check_state(s, "uvmi_sched_step_plan");
+  if (rc) return rc;
+  UVMI_REQUIRE(s->q_buf && s->q_ctl && s->q_cap > 0 && s->q_stride > 3, UVMI_EINVAL, "uvmi_sched_step_plan: the state has no admission queue");
+  UVMI_REQUIRE(n_bucket > 0 && act_slot && tok_c && pos_c && starts_c && req_c && cnt_c && admit_cap > 0 && admit_cap <= 256 && n_tokens > 0 &&
+                   adm_cu && adm_slot && adm_start && adm_limit && adm_req && tok_packed && pos_t && row_t && last_t && last_idx,
+               UVMI_EINVAL, "uvmi_sched_step_plan: bad arguments (admit_cap 1..256)");
+  hipLaunchKernelGGL(sched_step_plan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, *s, n_bucket, act_slot, tok_c, pos_c, starts_c, req_c,
+                     cnt_c, admit_cap, n_tokens, left_pad ? 1 : 0, adm_cu, adm_slot, adm_start, adm_limit, adm_req, tok_packed, pos_t, row_t,
+                     last_t, last_idx, last_c);
+  UVMI_CHECK_LAUNCH("uvmi_sched_step_plan");
   return UVMI_OK;
 }
 

@@ -53,6 +53,7 @@ __device__ __forceinline__ void commit_row(const uvmi_sched_state S, const Dense
     S.done_slot[k] = slot;
     S.done_cnt[k] = c + 1;
     S.slot_req[slot] = -1;
+    if (S.slot_hold) S.slot_hold[slot] = 1;   // its output row is not harvested yet: not reusable by a device-side admission
     S.pos[slot] = 0;      // parked: never overruns the cache (model.py:1345-1350)
     S.starts[slot] = 0;
   }

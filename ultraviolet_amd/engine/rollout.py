@@ -30,7 +30,7 @@ class Rollout:
                  seed: int = 0, eos_id: int | None = None, check_every: int = 16, bucket: int = 128,
                  use_graph: bool = True, retire_p: float = 0.0, left_pad: bool = False, mixed: bool = False,
                  admit_cap: int = 16, top_k: int = 0, top_p: float = 1.0, kv_dtype: str = "int8", overlap_harvest: bool = False,
-                 share_prompts: bool = False):
+                 share_prompts: bool = False, device_admit: bool = False):
         self.e, self.cfg = engine, engine.cfg
         self.top_k, self.top_p = int(top_k), float(top_p)   # truncated sampling (sample(), model.py:1200-1209); off by default
         self.B, self.max_prompt, self.max_new = slots, max_prompt, max_new
@@ -38,6 +38,8 @@ class Rollout:
         self.ce, self.bucket, self.use_graph = check_every, bucket, use_graph
         self.retire_p, self.left_pad = float(retire_p), left_pad
         self.mixed = mixed                        # admit while decoding: prompts ride in the same pass as the decode rows
+        self.device_admit = bool(device_admit)    # the free-slot choice and the FIFO queue of a mixed step live on the device
+        assert not device_admit or mixed, "device_admit plans the admissions of mixed steps: it needs mixed=True"
         self.n_mixed_steps = 0
         dev = engine.device
         self.dev = dev
@@ -85,10 +87,25 @@ class Rollout:
             self.gather_idx = torch.cat([z(A), Np + torch.arange(slots, device=dev)])   # rows of the hidden that get sampled
             self.adm_slot.fill_(-1)
             self._stage_ev = torch.cuda.Event()
+        if self.device_admit:
+            # the admission queue: a ring of staged prompts [length, request id, limit, tokens ...] the planning kernel takes
+            # from; the host only appends rows (and the staged count after them) and learns what was admitted from the harvest
+            self.q_cap = 1 << max(6, (4 * A - 1).bit_length())
+            self.q_stride = max_prompt + 3
+            self.q_buf, self.q_ctl = z(self.q_cap, self.q_stride), z(4)
+            self.q_rows_h = torch.zeros(self.q_cap, self.q_stride, dtype=torch.long, pin_memory=True)
+            self.q_ctl_h = torch.zeros(1, dtype=torch.long, pin_memory=True)
+            self.slot_hold = z(slots, dt=torch.int32)
+            s.slot_hold, s.q_buf, s.q_ctl, s.q_cap, s.q_stride = self.slot_hold.data_ptr(), self.q_buf.data_ptr(), self.q_ctl.data_ptr(), self.q_cap, self.q_stride
+            self.q_tail = 0                           # prompts staged so far
+            self.q_head = 0                           # prompts the device is known to have admitted (as of the last harvest)
+            self.staged = collections.deque()         # (request id, meta) of staged prompts not yet known to be admitted
+            self.n_free_dev = slots                   # reusable slots as of the last harvest, minus what may have been admitted since
+            self._q_ev = torch.cuda.Event()
         # harvest staging: a launch packs up to hv_rows new completion records and their output rows; the host takes the header
         # and then exactly the finished tokens, through pinned buffers (no indexing launches, no pageable copies)
         self.hv_rows = min(slots, 128)
-        self.hv_hdr, self.hv_tok, self.hv_lp = z(4 + 4 * self.hv_rows), z(self.hv_rows * max_new, dt=torch.int32), z(self.hv_rows * max_new, dt=torch.float32)
+        self.hv_hdr, self.hv_tok, self.hv_lp = z(8 + 4 * self.hv_rows), z(self.hv_rows * max_new, dt=torch.int32), z(self.hv_rows * max_new, dt=torch.float32)
         self.hv_hdr_h, self.hv_tok_h, self.hv_lp_h = (torch.zeros(t.shape, dtype=t.dtype, pin_memory=True) for t in (self.hv_hdr, self.hv_tok, self.hv_lp))
         self._hv_ev, self._hv_ev2 = torch.cuda.Event(), torch.cuda.Event()
         self._hv_stream = torch.cuda.Stream(device=dev)   # default priority; carries only the harvest's device -> host copies
@@ -105,6 +122,7 @@ class Rollout:
         self.done_seen = 0
         self._dense_n = None                      # bucket the dense step arrays are valid for (None: stale, compact first)
         self.version = 0                          # advanced by the caller after each weight update (scripts/rl_grpo.py:1309)
+        self._admit_version = 0                   # version at the launch of the last step that admitted on the device
         self._scalar_epoch = getattr(self.e.w, "scalar_epoch", 0)
         self.n_decode_steps = 0
         self.n_tokens = 0
@@ -117,12 +135,17 @@ class Rollout:
         self.queue.append((ids, meta, self.max_new if limit is None else min(int(limit), self.max_new), np.asarray(ids, dtype=np.int64)))
 
     def n_active(self) -> int:
+        if self.device_admit:
+            return self.n_active_host      # an upper bound between harvests, exact after one
         return self.B - len(self.free)
 
     def n_outstanding(self) -> int:
+        if self.device_admit:
+            return len(self.queue) + len(self.meta)
         return len(self.queue) + self.n_active()
 
     def drop_queued(self, pred) -> int:
+        """Drop the queued requests whose meta satisfies pred (prompts already staged on the device stay)."""
         keep = [x for x in self.queue if not pred(x[1])]
         n = len(self.queue) - len(keep)
         self.queue = collections.deque(keep)
@@ -258,17 +281,77 @@ class Rollout:
         self.n_mixed_steps += 1
         return True
 
+    # ---- device-side admission: the host stages prompts and launches; the slot choice and the queue are the device's
+    @torch.no_grad()
+    def _stage_prompts(self):
+        """Append queued prompts to the device ring while it has room (room is counted against the admissions the host has
+        seen, a lower bound of the device's), then publish the staged count.  Request ids are assigned here, in arrival
+        order.  Copies are stream-ordered ahead of the next step's planning kernel."""
+        room = self.q_cap - (self.q_tail - self.q_head)
+        k = min(room, len(self.queue))
+        if k <= 0:
+            return
+        self._q_ev.synchronize()                            # the previous upload has left the pinned rows
+        rows = self.q_rows_h.numpy()
+        first = self.q_tail % self.q_cap
+        for j in range(k):
+            ids, meta, limit, arr = self.queue.popleft()
+            r = rows[(first + j) % self.q_cap]
+            r[0], r[1], r[2] = len(ids), self.next_req, limit
+            r[3:3 + len(ids)] = arr
+            self.meta[self.next_req] = (meta, None)         # start_version is set when the admission is seen
+            self.staged.append(self.next_req)
+            self.next_req += 1
+        n1 = min(k, self.q_cap - first)
+        self.q_buf[first:first + n1].copy_(self.q_rows_h[first:first + n1], non_blocking=True)
+        if k > n1:
+            self.q_buf[:k - n1].copy_(self.q_rows_h[:k - n1], non_blocking=True)
+        self.q_tail += k
+        self.q_ctl_h[0] = self.q_tail
+        self.q_ctl[:1].copy_(self.q_ctl_h, non_blocking=True)
+        self._q_ev.record()
+
+    @torch.no_grad()
+    def _admit_device(self) -> bool:
+        """A decode step that also admits what the device finds admissible: one graph replay, nothing uploaded.  The host's
+        part is the decision to launch it - it knows how many prompts are staged and, from the last harvest, how many slots
+        were reusable - and an upper bound on the active slots for the bucket.  Returns False when there is nothing to admit."""
+        pending = self.q_tail - self.q_head
+        if pending <= 0 or self.n_free_dev <= 0:
+            return False
+        may = min(self.A, pending, self.n_free_dev)
+        n = self.bucket_for(self.n_active_host)
+        if self.use_graph:
+            (self.mixed_graphs.get(n) or self._capture(n, mixed=True)).replay()
+        else:
+            self._mixed_body(n)
+        self.n_active_host = min(self.B, self.n_active_host + may)   # upper bound until the next harvest tells
+        self.n_free_dev -= may
+        self._admit_version = self.version
+        self._dense_n = None
+        self.n_decode_steps += 1
+        self.n_mixed_steps += 1
+        return True
+
     def _mixed_body(self, n: int):
         """compact -> prompt tables -> one trunk pass over Np prompt tokens + n decode rows -> head -> sampler -> commit
         (decode rows) + admit (prompts).  Every launch has fixed shapes; what varies lives in device arrays."""
         e, lib, A, Np = self.e, L.lib(), self.A, self.Np
         sp = L.stream_ptr(self.act)
-        L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
-                                       self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
-        L.check(lib.uvmi_sched_expand(C.byref(self.sched), A, Np, self.adm_cu.data_ptr(), self.adm_slot.data_ptr(), self.adm_start.data_ptr(),
-                                      self.pos_all.data_ptr(), self.row_all.data_ptr(), self.last_all.data_ptr(), self.gather_idx.data_ptr(),
-                                      sp), "uvmi_sched_expand")
-        self.last_all[Np:Np + n].copy_(self.pos_all[Np:Np + n])
+        if self.device_admit:   # compaction, admission plan and prompt tables in one launch
+            L.check(lib.uvmi_sched_step_plan(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                             self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), A, Np, int(self.left_pad),
+                                             self.adm_cu.data_ptr(), self.adm_slot.data_ptr(), self.adm_start.data_ptr(),
+                                             self.adm_limit.data_ptr(), self.req_all.data_ptr(), self.tok_all.data_ptr(),
+                                             self.pos_all.data_ptr(), self.row_all.data_ptr(), self.last_all.data_ptr(),
+                                             self.gather_idx.data_ptr(), self.last_all[Np:].data_ptr(), sp), "uvmi_sched_step_plan")
+        else:
+            L.check(lib.uvmi_sched_compact(C.byref(self.sched), n, self.act.data_ptr(), self.tok_c.data_ptr(), self.pos_c.data_ptr(),
+                                           self.starts_c.data_ptr(), self.req_c.data_ptr(), self.cnt_c.data_ptr(), sp), "uvmi_sched_compact")
+            L.check(lib.uvmi_sched_expand(C.byref(self.sched), A, Np, self.adm_cu.data_ptr(), self.adm_slot.data_ptr(), self.adm_start.data_ptr(),
+                                          self.pos_all.data_ptr(), self.row_all.data_ptr(), self.last_all.data_ptr(), self.gather_idx.data_ptr(),
+                                          sp), "uvmi_sched_expand")
+            self.last_all[Np:Np + n].copy_(self.pos_all[Np:Np + n])
         h = e.mixed_trunk(self.tok_all, self.pos_all, self.row_all, self.last_all, Np, n, self.adm_cu, self.starts_c[:n], self.st)
         x = e.head(h.index_select(0, self.gather_idx[:A + n]))
         tok, lp = self._sample(x, self.req_all[:A + n], self.cnt_all[:A + n])
@@ -339,7 +422,7 @@ class Rollout:
             for n in range(self.bucket, self.bucket_for(self.n_active_host) + 1, self.bucket):
                 if n not in self.graphs:
                     self._capture(min(n, self.B))
-                if self.mixed and self.queue and n not in self.mixed_graphs:
+                if self.mixed and (self.queue or (self.device_admit and self.q_tail > self.q_head)) and n not in self.mixed_graphs:
                     self._capture(min(n, self.B), mixed=True)
 
     @torch.no_grad()
@@ -367,9 +450,10 @@ class Rollout:
     def _mutable(self):
         """State a decode step writes.  The KV cache is left out on purpose: the warm-up step writes K/V at the current
         positions, and the real replay rewrites exactly those slots with identical inputs (as in model.py:1126-1127)."""
-        return [self.slot_req, self.slot_cnt, self.slot_limit, self.slot_tok, self.st.pos, self.st.starts, self.out_tok, self.out_lp,
-                self.done_req, self.done_slot, self.done_cnt, self.counters, self.act, self.tok_c, self.pos_c, self.starts_c, self.req_c,
-                self.cnt_c]
+        m = [self.slot_req, self.slot_cnt, self.slot_limit, self.slot_tok, self.st.pos, self.st.starts, self.out_tok, self.out_lp,
+             self.done_req, self.done_slot, self.done_cnt, self.counters, self.act, self.tok_c, self.pos_c, self.starts_c, self.req_c,
+             self.cnt_c]
+        return m + [self.q_ctl, self.slot_hold] if self.device_admit else m
 
     # ------------------------------------------------------------------------------------------------ harvest
     @torch.no_grad()
@@ -411,18 +495,37 @@ class Rollout:
                     self._hv_ev2.record()
                 self._hv_ev2.synchronize()
             toks, lps = self.hv_tok_h.numpy(), self.hv_lp_h.numpy()
+            self._see_admissions(hdr)
             # arrival order inside one step is not deterministic: sort by request
             for r, s_, c, o in rec[np.argsort(rec[:, 0], kind="stable")].tolist():
                 meta, v0 = self.meta.pop(r)
                 out.append((meta, toks[o:o + c].tolist(), lps[o:o + c].copy(), v0))
                 self.n_tokens += c
-                self.free.append(s_)
+                if not self.device_admit:
+                    self.free.append(s_)
             self.done_seen += k
             if self.done_seen >= n_done:
                 break
             self.harvest_begin()   # more records than one launch packs
-        self.n_active_host = self.n_active()
+        if self.device_admit:
+            self._see_admissions(hdr)
+            x = hdr[4 + 4 * self.hv_rows:]
+            self.n_active_host = int(x[0])                                    # exact at the packing launch; only retirements since
+            self.n_free_dev = self.B - int(x[0]) - (n_done - self.done_seen)  # finished rows not packed yet keep their slots
+        else:
+            self.n_active_host = self.n_active()
         return out
+
+    def _see_admissions(self, hdr):
+        """Device-side admission: the harvest header carries the number of prompts the device has admitted so far; the
+        requests that crossed from staged to admitted since the last look get their start version."""
+        if not self.device_admit:
+            return
+        head = int(hdr[4 + 4 * self.hv_rows + 1])
+        while self.q_head < head:
+            r = self.staged.popleft()
+            self.meta[r] = (self.meta[r][0], self._admit_version)
+            self.q_head += 1
 
     def poll(self):
         """Harvest now: harvest_begin() + harvest_end()."""
@@ -441,7 +544,11 @@ class Rollout:
                 self.step()
                 steps -= 1
             out = self.harvest_end()
-        if self.queue and self.free:
+        if self.device_admit:
+            self._stage_prompts()
+            while steps > 0 and self._admit_device():
+                steps -= 1
+        elif self.queue and self.free:
             if self.mixed and self.n_active() > 0:
                 while self.queue and self.free and steps > 0 and self._admit_mixed():
                     steps -= 1

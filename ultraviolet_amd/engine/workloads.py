@@ -29,7 +29,7 @@ def fill_cache(st, rows, ctx, gen):
     st.starts[rows] = 0
 
 
-def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0):
+def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0, device_admit=False, check_every=4, admit_cap=24):
     """The C3 workload as a Rollout ready to step: B running slots whose contexts U{128..2048} are materialised in the cache
     (request ids 0..B-1, one token generated so far), Bernoulli(0.01) retirement per slot and step on the device, and a
     queue of 64-token prompts (ids B, B + 1, ..) long enough for n_steps steps, admitted inside decode passes."""
@@ -37,8 +37,8 @@ def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0):
     dev = eng.device
     rng = np.random.default_rng(seed)
     gen = torch.Generator(device=dev).manual_seed(seed)
-    g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + n_steps + 64, temperature=1.0, seed=seed, eos_id=None, check_every=4, bucket=128,
-                retire_p=0.01, mixed=True, admit_cap=24, overlap_harvest=True, use_graph=use_graph)
+    g = Rollout(eng, slots=B, max_prompt=64, max_new=2048 + n_steps + 64, temperature=1.0, seed=seed, eos_id=None, check_every=check_every, bucket=128,
+                retire_p=0.01, mixed=True, admit_cap=admit_cap, overlap_harvest=True, use_graph=use_graph, device_admit=device_admit)
     rows = torch.arange(B, device=dev)
     fill_cache(g.st, rows, torch.from_numpy(rng.integers(128, 2049, size=B)).to(dev), gen)
     g.slot_req.copy_(rows)
@@ -46,6 +46,8 @@ def c3_rollout(eng, cfg, B, n_steps, use_graph=True, seed=0):
     g.slot_limit.fill_(g.max_new)
     g.slot_tok.copy_(torch.from_numpy(rng.integers(1, cfg.vocab_size, size=B)).to(dev))
     g.free, g.next_req, g.n_active_host = [], B, B
+    if device_admit:
+        g.n_free_dev = 0
     for r in range(B):
         g.meta[r] = (r, 0)
     for i in range(int(n_steps * B * 0.01 * 2) + 64):
