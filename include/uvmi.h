@@ -93,7 +93,8 @@ int uvmi_kv_append(const uvmi_kv_append_args* a, void* stream);
  * ---------------------------------------------------------------------------------------------------------- */
 struct uvmi_attn_qkv_fuse;
 typedef struct uvmi_attn_args {
-  const void* q; int q_dtype;              /* (B, H, hd) F16 or BF16, inner stride 1 */
+  const void* q; int q_dtype;              /* (B, H, hd) F16 / BF16 (the MFMA kernel multiplies in 16 bits) or F32 (the generic
+                                              kernel: every product and probability stays fp32), inner stride 1 */
   int64_t sqb, sqh;
   const void* k_cache; const void* v_cache; int kv_dtype; /* (B, KH, S, hd) I8, F16, BF16 or F32, inner stride 1 */
   int64_t skb, skh, sks, svb, svh, svs;
@@ -230,7 +231,7 @@ int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream);
  * Query i of a segment sees keys j of the same segment with i - window < j <= i (window 0: every j <= i).
  * ---------------------------------------------------------------------------------------------------------- */
 typedef struct uvmi_prefill_attn_args {
-  const void* q; int q_dtype;              /* (N, H, hd) F16 / BF16, inner stride 1 */
+  const void* q; int q_dtype;              /* (N, H, hd) F16 / BF16, or F32 (generic kernel), inner stride 1 */
   int64_t sqn, sqh;                        /* strides in elements */
   const void* k; const void* v; int kv_dtype; /* (N, KH, hd) F16 / BF16 / F32, inner stride 1 */
   int64_t skn, skh, svn, svh;
@@ -339,7 +340,7 @@ typedef struct uvmi_qkv_post_args {
   const int64_t* rows;                 /* (n,) cache row of each token; NULL = identity */
   const int64_t* last_pos;             /* (n,) last position of the token's prompt, or NULL (decode rows) */
   const float* inv_freq;               /* (n_pairs,) RoPE frequencies, fp32 */
-  void* q_out; int q_dtype;            /* (n, H, hd) F16 or BF16 */
+  void* q_out; int q_dtype;            /* (n, H, hd) F16, BF16 or F32 */
   void* k_out; void* v_out;            /* (n, KH, hd) in dtype, or NULL */
   int8_t* k_cache; int8_t* v_cache;    /* (B, KH, S, hd) or NULL (no append) */
   uint16_t* k_scale; uint16_t* v_scale;
@@ -364,7 +365,7 @@ int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream);
 
 /* Attention.post before the output projection (ultraviolet/model.py:321-333): XSA z -= xsa[h] (z . v_hat) v_hat with
  * the unquantized current v (fp32), then z *= 2 sigmoid(gate_w[h] . xn[:gate_ch]).  xsa = tanh(alpha) (H,) fp32 or NULL;
- * gate_w (H, gate_ch) fp32 or NULL.  z (n, H, hd) in z_dtype (F16 / BF16); out (n, H * hd) in dtype. */
+ * gate_w (H, gate_ch) fp32 or NULL.  z (n, H, hd) in z_dtype (F16 / BF16 / F32); out (n, H * hd) in dtype. */
 int uvmi_attn_post(const void* z, int z_dtype, const void* v, const void* xn, int dtype, const float* gate_w,
                    const float* xsa, float xsa_eps, int64_t n, int H, int KH, int hd, int d, int gate_ch, void* out,
                    void* stream);

@@ -101,8 +101,11 @@ def test_greedy_64_tokens_identical_fp32(name, over):
     out = np.array(eng.generate(prompts, 64, temperature=0.0))
     ref, lgs, _ = OracleModel(cfg, params, torch.float32).generate_greedy(prompts, 64, return_logits=True)
     assert len(np.unique(ref)) > 8                                  # the stream is not one repeated token
-    # A stream may only leave the oracle's at a step where the oracle's own top-2 logits are closer than the numeric
-    # noise of the GPU path (fp16 q and P in the attention kernel, a different GEMM summation order): ~2e-3.
+    # An fp32 engine keeps fp32 queries and probabilities (the plain fp32 attention kernel), so what separates it from the
+    # oracle is the summation order of the GEMMs and, through it, an int8 code of the cache that sits on a rounding tie
+    # and lands one step away (one code step of one key moves the logits by ~1e-4).  A stream may therefore leave the
+    # oracle's only where the oracle's own top-2 logits are closer than 1e-3 (on logits of magnitude ~18), every such
+    # row is printed with its step and gap, and most rows stay identical over all 64 steps.
     identical = 0
     for b in range(len(prompts)):
         d = np.nonzero(out[b] != ref[b])[0]
@@ -111,7 +114,8 @@ def test_greedy_64_tokens_identical_fp32(name, over):
             continue
         t = int(d[0])
         top2 = np.sort(lgs[b, t])[-2:]
-        assert top2[1] - top2[0] < 2e-3, f"row {b} diverges at step {t} with top-2 logit gap {top2[1] - top2[0]:.2e}"
+        print(f"row {b} leaves the oracle's stream at step {t}: oracle top-2 logit gap {top2[1] - top2[0]:.2e}")
+        assert top2[1] - top2[0] < 1e-3, f"row {b} diverges at step {t} with top-2 logit gap {top2[1] - top2[0]:.2e}"
     assert identical >= len(prompts) - 2, identical
 
 
@@ -301,7 +305,7 @@ def test_patch_model_binds_the_reference_entry_points():
     assert h.shape == (3, cfg.d_model)
     # in-place refresh: new parameters, same device addresses
     ptr = m._uvmi_engine.w.layers[0]["wqkv"].data_ptr()
-    m._sd = {k: v * 1.01 if k.endswith("wq") else v for k, v in m._sd.items()}
+    m._sd = {k: v * 1.01 if k.endswith("wv") else v for k, v in m._sd.items()}
     fd.sync_patched_weights(m)
     assert m._uvmi_engine.w.layers[0]["wqkv"].data_ptr() == ptr
     lg2 = m.decode_step(tok, st, 64)
@@ -542,12 +546,13 @@ def test_patched_model_follows_in_place_parameter_updates():
     idx = torch.tensor([[5, 6, 7, 8], [9, 10, 11, 12]], device=DEV)
     l0 = m.prefill(idx, torch.zeros(2, dtype=torch.long, device=DEV), st)
     ptr = m._uvmi_engine.w.layers[0]["wqkv"].data_ptr()
-    m._sd["blocks.0.attn.wq"].mul_(1.05)                       # an optimizer step / sync_weights_inplace writes like this
+    m._sd["blocks.0.attn.wv"].mul_(1.05)                       # an optimizer step / sync_weights_inplace writes like this
+    #                                                            (wv: QK-norm makes a uniform scaling of wq or wk invisible)
     st2 = m.new_state(2, 48)
     l1 = m.prefill(idx, torch.zeros(2, dtype=torch.long, device=DEV), st2)
     assert m._uvmi_engine.w.layers[0]["wqkv"].data_ptr() == ptr and not torch.allclose(l0, l1)
     cfg2, params2, eng2, _ = _setup(window=32)
-    params2["blocks.0.attn.wq"] = params2["blocks.0.attn.wq"] * np.float32(1.05)
+    params2["blocks.0.attn.wv"] = params2["blocks.0.attn.wv"] * np.float32(1.05)
     from ultraviolet_amd.engine import KVState, UVEngine, UVWeights
     e3 = UVEngine(UVWeights(cfg2, params2, torch.float32, DEV), max_tokens=256)
     ref = e3.logits(e3.prefill([[5, 6, 7, 8], [9, 10, 11, 12]], [0, 1], KVState(cfg2, 2, 48, DEV)))

@@ -426,12 +426,33 @@ def test_error_paths_are_loud():
     from ultraviolet_amd.kernels import decode_attention, quantize_kv
     with pytest.raises(L.UvmiError):
         quantize_kv(torch.zeros(4, 64))  # CPU tensor: no fallback
-    q = torch.zeros(2, 8, 64, device=DEV)  # fp32 q is not supported
+    q = torch.zeros(2, 8, 64, device=DEV, dtype=torch.float64)  # queries are fp16, bf16 or fp32
     kc = torch.zeros(2, 1, 64, 64, dtype=torch.int8, device=DEV)
     sc = torch.zeros(2, 1, 64, dtype=torch.half, device=DEV)
     p = torch.zeros(2, dtype=torch.long, device=DEV)
-    with pytest.raises(L.UvmiError):
+    with pytest.raises((L.UvmiError, KeyError)):
         decode_attention(q, kc, kc, p, p, 0.1, k_scale=sc, v_scale=sc)
+    with pytest.raises((L.UvmiError, AssertionError)):
+        decode_attention(q.half(), kc, kc, p, p, 0.1)          # an int8 cache without its scales
+
+
+def test_fp32_queries_stay_fp32():
+    """q in fp32 takes the plain fp32 kernel - no 16-bit rounding of q or of the probabilities: against the float64 oracle
+    it is two orders of magnitude closer than the 2e-3 bar of the 16-bit paths (int8 and fp32 caches, ring and linear)."""
+    from oracle import decode_attn as odec
+    from ultraviolet_amd.kernels import decode_attention
+    from util import attn_case
+    for ring in (False, True):
+        q, k, v, ks, vs = attn_case(7, 1, 8, 64, 128, True, seed=21 + ring, dtype=torch.float32)
+        pos = torch.tensor([0, 5, 127, 200, 64, 31, 129]) if ring else torch.tensor([0, 5, 127, 90, 64, 31, 100])
+        starts = torch.tensor([0, 2, 0, 120, 0, 30, 60]) if ring else torch.tensor([0, 2, 0, 50, 0, 30, 60])
+        w = 128 if ring else 0
+        out = decode_attention(q.to(DEV), k.to(DEV), v.to(DEV), pos.to(DEV), starts.to(DEV), 0.14125, window=w, ring=ring,
+                               k_scale=ks.to(DEV), v_scale=vs.to(DEV))
+        assert out.dtype == torch.float32
+        ref = odec.decode_attention_ref(q.double().numpy(), k.numpy(), v.numpy(), pos.numpy(), starts.numpy(), 0.14125, window=w, ring=ring,
+                                        k_scale=ks.numpy(), v_scale=vs.numpy())
+        np.testing.assert_allclose(out.cpu().numpy(), ref, atol=2e-5, rtol=2e-5)
 
 
 @pytest.mark.gpu

@@ -142,8 +142,11 @@ def test_error_paths():
     with pytest.raises(L.UvmiError):
         packed_attention(q, k, v, cu, SC)                       # host tensors
     d = lambda t: t.to(DEV)
-    with pytest.raises(L.UvmiError):
-        packed_attention(d(q).float(), d(k), d(v), d(cu), SC)    # fp32 q is not supported
+    with pytest.raises((L.UvmiError, KeyError)):
+        packed_attention(d(q).double(), d(k), d(v), d(cu), SC)   # queries are fp16, bf16 or fp32
+    o32 = packed_attention(d(q).float(), d(k).float(), d(v).float(), d(cu), SC)   # fp32 throughout: the plain fp32 kernel
+    o16 = packed_attention(d(q), d(k), d(v), d(cu), SC, out_fp32=True)
+    assert o32.dtype == torch.float32 and (o32 - o16).abs().max() < 2e-3
     with pytest.raises(AssertionError):
         packed_attention(d(q), d(k), d(v), d(cu), SC, workspace=torch.empty(64, dtype=torch.uint8, device=DEV))  # too small
 

@@ -1042,7 +1042,8 @@ static int check_common(const uvmi_attn_args* a) {
   UVMI_REQUIRE(a->q && a->k_cache && a->v_cache && a->pos && a->starts && a->out, UVMI_EINVAL, "uvmi_decode_attn: null pointer");
   UVMI_REQUIRE(a->B >= 0 && a->H > 0 && a->KH > 0 && a->S > 0 && a->hd > 0, UVMI_EINVAL, "uvmi_decode_attn: bad sizes");
   UVMI_REQUIRE(a->H % a->KH == 0, UVMI_EINVAL, "uvmi_decode_attn: H=%d is not a multiple of KH=%d", a->H, a->KH);
-  UVMI_REQUIRE(a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16, UVMI_EUNSUPPORTED, "uvmi_decode_attn: q must be F16 or BF16");
+  UVMI_REQUIRE(a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16 || a->q_dtype == UVMI_F32, UVMI_EUNSUPPORTED,
+               "uvmi_decode_attn: q must be F16, BF16 or F32");
   UVMI_REQUIRE(a->out_dtype == UVMI_F16 || a->out_dtype == UVMI_BF16 || a->out_dtype == UVMI_F32, UVMI_EUNSUPPORTED,
                "uvmi_decode_attn: out must be F16, BF16 or F32");
   UVMI_REQUIRE(a->kv_dtype == UVMI_I8 || a->kv_dtype == UVMI_F16 || a->kv_dtype == UVMI_BF16 || a->kv_dtype == UVMI_F32, UVMI_EUNSUPPORTED,
@@ -1059,6 +1060,7 @@ static int check_common(const uvmi_attn_args* a) {
 static bool mfma_ok(const uvmi_attn_args* a) {
   const int G = a->H / a->KH;
   if (a->hd != 64 || a->kv_dtype != UVMI_I8 || G > 8) return false;
+  if (a->q_dtype == UVMI_F32) return false;  // fp32 queries keep every product and probability in fp32: the generic kernel
   if (!(a->scale > 0.f)) return false;  // the running maximum is tracked before the (positive) softmax scale
   if (a->ring && (a->S % 32 != 0)) return false;
   if (a->sks > (1 << 20) || a->svs > (1 << 20) || a->sks < 0 || a->svs < 0) return false;  // 32-bit tile offsets
@@ -1262,7 +1264,7 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
 #define UVMI_L(QD, KD, OD) hipLaunchKernelGGL((attn_generic<QD, KD, OD>), grid, blk, sh, st, P)
 #define UVMI_LO(QD, KD) do { if (od == UVMI_F16) UVMI_L(QD, KD, UVMI_F16); else if (od == UVMI_BF16) UVMI_L(QD, KD, UVMI_BF16); else UVMI_L(QD, KD, UVMI_F32); } while (0)
 #define UVMI_LK(QD) do { if (a->kv_dtype == UVMI_I8) UVMI_LO(QD, UVMI_I8); else if (a->kv_dtype == UVMI_F16) UVMI_LO(QD, UVMI_F16); else if (a->kv_dtype == UVMI_F32) UVMI_LO(QD, UVMI_F32); else UVMI_LO(QD, UVMI_BF16); } while (0)
-    if (a->q_dtype == UVMI_F16) UVMI_LK(UVMI_F16); else UVMI_LK(UVMI_BF16);
+    if (a->q_dtype == UVMI_F16) UVMI_LK(UVMI_F16); else if (a->q_dtype == UVMI_F32) UVMI_LK(UVMI_F32); else UVMI_LK(UVMI_BF16);
 #undef UVMI_LK
 #undef UVMI_LO
 #undef UVMI_L

@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
       }
       if (h < A.H) {
         const int64_t o = (r * A.H + h) * 64 + 8 * c;
-        if (A.q_dt == UVMI_BF16) st8<UVMI_BF16>(A.q_out, o, x); else st8<UVMI_F16>(A.q_out, o, x);
+        if (A.q_dt == UVMI_BF16) st8<UVMI_BF16>(A.q_out, o, x); else if (A.q_dt == UVMI_F32) st8<UVMI_F32>(A.q_out, o, x); else st8<UVMI_F16>(A.q_out, o, x);
       }
     }
     // ---- per-head output gate 2 sigmoid(W_h . xn[:gate_ch]) for the attention epilogue (model.py:330-333)
@@ -322,7 +322,8 @@ __global__ __launch_bounds__(256) void attn_post_kernel(PostArgs A) {
   const int G = A.H / A.KH;
   for (int h = 0; h < A.H; h++) {
     const int kh = h / G;
-    float z = A.z_dt == UVMI_BF16 ? elem<UVMI_BF16>::ld(A.z, (r * A.H + h) * 64 + lane) : elem<UVMI_F16>::ld(A.z, (r * A.H + h) * 64 + lane);
+    const int64_t zi = (r * A.H + h) * 64 + lane;
+    float z = A.z_dt == UVMI_BF16 ? elem<UVMI_BF16>::ld(A.z, zi) : (A.z_dt == UVMI_F32 ? elem<UVMI_F32>::ld(A.z, zi) : elem<UVMI_F16>::ld(A.z, zi));
     if (A.xsa) {  // z -= tanh(alpha_h) (z . v_hat) v_hat, v_hat = v / max(|v|, eps), in fp32
       const float v = elem<DT>::ld(A.v, (r * A.KH + kh) * 64 + lane);
       const float nv = sqrtf(wave_sum(v * v));
@@ -449,7 +450,7 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_qkv_post: null args");
   UVMI_REQUIRE(a->qkv && a->pos && a->q_out, UVMI_EINVAL, "uvmi_qkv_post: null pointer");
   UVMI_REQUIRE(a->hd == 64, UVMI_EUNSUPPORTED, "uvmi_qkv_post: head_dim %d (only 64)", a->hd);
-  UVMI_REQUIRE(is_float_dtype(a->dtype) && (a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16), UVMI_EINVAL, "uvmi_qkv_post: bad dtype");
+  UVMI_REQUIRE(is_float_dtype(a->dtype) && is_float_dtype(a->q_dtype), UVMI_EINVAL, "uvmi_qkv_post: bad dtype");
   UVMI_REQUIRE(a->n >= 0 && a->H > 0 && a->KH > 0 && a->H % a->KH == 0, UVMI_EINVAL, "uvmi_qkv_post: bad sizes");
   UVMI_REQUIRE(!a->rope || (a->inv_freq && a->n_pairs >= 8 && a->n_pairs <= 32 && (a->n_pairs & (a->n_pairs - 1)) == 0), UVMI_EUNSUPPORTED,
                "uvmi_qkv_post: rope needs inv_freq and 8, 16 or 32 rotated pairs");
@@ -512,7 +513,7 @@ extern "C" int uvmi_attn_post(const void* z, int z_dtype, const void* v, const v
                               float xsa_eps, int64_t n, int H, int KH, int hd, int d, int gate_ch, void* out, void* stream) {
   UVMI_REQUIRE(z && out, UVMI_EINVAL, "uvmi_attn_post: null pointer");
   UVMI_REQUIRE(hd == 64, UVMI_EUNSUPPORTED, "uvmi_attn_post: head_dim %d (only 64)", hd);
-  UVMI_REQUIRE(is_float_dtype(dtype) && (z_dtype == UVMI_F16 || z_dtype == UVMI_BF16), UVMI_EINVAL, "uvmi_attn_post: bad dtype");
+  UVMI_REQUIRE(is_float_dtype(dtype) && is_float_dtype(z_dtype), UVMI_EINVAL, "uvmi_attn_post: bad dtype");
   UVMI_REQUIRE(!xsa || v, UVMI_EINVAL, "uvmi_attn_post: XSA needs v");
   UVMI_REQUIRE(!gate_w || (xn && gate_ch > 0 && gate_ch <= d), UVMI_EINVAL, "uvmi_attn_post: gate needs xn and gate_ch");
   UVMI_REQUIRE(n >= 0 && H > 0 && KH > 0 && H % KH == 0, UVMI_EINVAL, "uvmi_attn_post: bad sizes");

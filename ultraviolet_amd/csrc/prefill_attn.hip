@@ -336,7 +336,8 @@ static int check_prefill(const uvmi_prefill_attn_args* a) {
   UVMI_REQUIRE(a->q && a->k && a->v && a->cu_seqlens && a->out, UVMI_EINVAL, "uvmi_prefill_attn: null pointer");
   UVMI_REQUIRE(a->n_seg >= 1, UVMI_EINVAL, "uvmi_prefill_attn: N > 0 needs at least one sequence");
   UVMI_REQUIRE(a->H % a->KH == 0, UVMI_EINVAL, "uvmi_prefill_attn: H=%d is not a multiple of KH=%d", a->H, a->KH);
-  UVMI_REQUIRE(a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16, UVMI_EUNSUPPORTED, "uvmi_prefill_attn: q must be F16 or BF16");
+  UVMI_REQUIRE(a->q_dtype == UVMI_F16 || a->q_dtype == UVMI_BF16 || a->q_dtype == UVMI_F32, UVMI_EUNSUPPORTED,
+               "uvmi_prefill_attn: q must be F16, BF16 or F32");
   UVMI_REQUIRE(is_float_dtype(a->kv_dtype), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: k/v must be F16, BF16 or F32");
   UVMI_REQUIRE(is_float_dtype(a->out_dtype), UVMI_EUNSUPPORTED, "uvmi_prefill_attn: out must be F16, BF16 or F32");
   UVMI_REQUIRE(a->idx_dtype == UVMI_I64 || a->idx_dtype == UVMI_I32, UVMI_EINVAL, "uvmi_prefill_attn: cu_seqlens must be I32 or I64");
@@ -351,7 +352,7 @@ static int check_prefill(const uvmi_prefill_attn_args* a) {
 }
 
 static bool prefill_mfma_ok_stats(const uvmi_prefill_attn_args* a) {   // (as below, without an output tensor)
-  if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype) return false;
+  if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype || a->q_dtype == UVMI_F32) return false;   // 16-bit operands
   if (!(a->scale > 0.f)) return false;
   auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
   if (!al(a->q, 16) || a->sqn % 8 || a->sqh % 8) return false;
@@ -362,7 +363,7 @@ static bool prefill_mfma_ok_stats(const uvmi_prefill_attn_args* a) {   // (as be
 }
 
 static bool prefill_mfma_ok(const uvmi_prefill_attn_args* a) {
-  if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype) return false;
+  if (a->hd != 64 || a->H / a->KH > 8 || a->kv_dtype != a->q_dtype || a->q_dtype == UVMI_F32) return false;   // 16-bit operands
   if (!(a->scale > 0.f)) return false;  // the running maximum is tracked before the (positive) softmax scale
   auto al = [](const void* p, int n) { return ((uintptr_t)p % n) == 0; };
   if (!al(a->q, 16) || a->sqn % 8 || a->sqh % 8) return false;

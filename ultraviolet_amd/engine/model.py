@@ -109,7 +109,9 @@ class UVEngine:
         self.dtype, self.device, self.max_tokens = dt, dev, max_tokens
         self.dt_code = L.dtype_code(dt)
         self.eps = rms_norm_eps(dt)
-        self.q_dtype = torch.bfloat16 if dt == torch.bfloat16 else torch.float16
+        # the attention kernels' query operand: the activation type; an fp32 engine keeps fp32 queries, which run on the plain
+        # fp32 attention kernel (no 16-bit rounding of q or of the probabilities anywhere on its path)
+        self.q_dtype = dt
         n, d, H, K, hd, f = max_tokens, cfg.d_model, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.d_ff
         e = lambda *s, dtype=dt: torch.empty(*s, dtype=dtype, device=dev)
         self.buf = dict(x=e(n, d), xn=e(n, d), h=e(n, d), qkv=e(n, (H + 2 * K) * hd), q=e(n, H, hd, dtype=self.q_dtype),
@@ -246,7 +248,7 @@ class UVEngine:
         kw = dict(window=0 if glob else cfg.window, ring=not glob, k_scale=st.k_scale[l], v_scale=st.v_scale[l], rows=rows)
         # the MFMA kernel (which carries the epilogue) streams 32-key tiles: rings need S % 32 == 0, linear int8 caches
         # S % 4 == 0; it serves int8 caches and caches in the q dtype
-        mfma_cache = st.quantized or (st.k[l].dtype == q.dtype and q.dtype in (torch.float16, torch.bfloat16))
+        mfma_cache = q.dtype != torch.float32 and (st.quantized or (st.k[l].dtype == q.dtype and q.dtype in (torch.float16, torch.bfloat16)))
         if mfma_cache and cfg.xsa and cfg.n_heads // cfg.n_kv_heads <= 8 and S % (4 if glob else 32) == 0 and S >= 32:
             out = b["zg"][off:off + n].view(n, cfg.n_heads, cfg.head_dim)
             decode_attention_post(q, st.k[l], st.v[l], pos, starts, cfg.attn_scale, vhat=b["vhat"][off:off + n],
