@@ -643,3 +643,32 @@ def test_uncompressed_decode_state_entry_points(dtype):
     ref2 = om.logits(hid2).float().numpy()
     assert np.abs(lg.float().cpu().numpy()[0] - ref2[0, 4]).max() < (0.15 if dtype == torch.bfloat16 else 0.04)   # 5 real tokens
     assert np.abs(lg.float().cpu().numpy()[1] - ref2[1, 8]).max() < (0.15 if dtype == torch.bfloat16 else 0.04)
+
+
+def test_bf16_engine_greedy_against_the_bf16_oracle_reports_every_divergence():
+    """The benchmarked configuration - UV-50M, bf16 activations, int8 KV - on the first configuration's shape (8 prompts of
+    32..128 tokens, 64 greedy tokens) against the oracle run in the same 16-bit arithmetic.  bf16 logits of magnitude ~18
+    sit on a grid of 2^-4 and the two implementations sum in different orders, so streams separate where the oracle's own
+    top two logits are within that noise; the test prints, per row, the first step at which the stream leaves the oracle's
+    and the oracle's top-2 gap there, and requires that no row leaves at a gap above the noise between the two paths'
+    logits - 0.15, the bar test_16bit_engine_close_to_oracle holds their teacher-forced logits to (measured: 0.07; the
+    reference's own bar for int8-vs-reference logits is 0.25, tests/test_math_kernels.py:170-172)."""
+    cfg, params, eng, OracleModel = _setup("uv-50m-alpha", dtype=torch.bfloat16, perturb=0.06)
+    rng = np.random.default_rng(0)
+    lens = rng.integers(32, 129, size=8)
+    prompts = [rng.integers(1, cfg.vocab_size, size=int(n)).tolist() for n in lens]
+    out = np.array(eng.generate(prompts, 64, temperature=0.0))
+    ref, lgs, _ = OracleModel(cfg, params, torch.bfloat16).generate_greedy(prompts, 64, return_logits=True)
+    first, gaps = [], []
+    for b in range(len(prompts)):
+        d = np.nonzero(out[b] != ref[b])[0]
+        t = int(d[0]) if len(d) else 64
+        first.append(t)
+        if t < 64:
+            top2 = np.sort(lgs[b, t])[-2:]
+            gaps.append(float(top2[1] - top2[0]))
+            print(f"row {b}: identical for {t} steps, then the oracle's top-2 gap is {gaps[-1]:.3f}")
+        else:
+            print(f"row {b}: identical for all 64 steps")
+    assert all(g_ < 0.15 for g_ in gaps), gaps
+    assert (ref[:, 0] == out[:, 0]).sum() >= 6  # (the first token comes from the prefill alone: most rows agree on it)

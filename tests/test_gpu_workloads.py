@@ -180,3 +180,68 @@ def test_c5_long_rollout_sixteen_sequences_teacher_forced_through_the_oracle():
     print("teacher-forced log-prob gap: mean %.4f p99 %.4f max %.4f over %d tokens" % (d.mean(), np.quantile(d, 0.99), d.max(), d.size))
     # measured: mean 0.006, p99 0.020, max 0.031 (bf16 logits of magnitude ~10 carry 2^-5 spacing); the bars are twice that
     assert d.mean() < 0.015 and np.quantile(d, 0.99) < 0.05 and d.max() < 0.1, (d.mean(), np.quantile(d, 0.99), d.max())
+
+
+def test_c5_at_its_real_length_properties_and_four_longest_sequences_through_the_oracle():
+    """BASELINE configs[4] exactly as the benchmark runs it: stop lengths min(Geom(1/600), 2048), ~2040 decode steps, the
+    global layers past two thousand keys, the live rows shrinking from 2048 to a handful (every row bucket, every choice of
+    waves per row, re-compactions).  Token accounting for all 2048 requests - every request once, len(row) == len(logp) ==
+    its stop length - positions = prompt length + tokens at step 500, and the four longest sequences of the group that
+    runs longest teacher-forced through OracleModel(bf16) on the CPU (same int8 cache, same rounding points): the
+    behaviour log-probs the rollout recorded against the oracle's log softmax of the same tokens, to the bars of the
+    shorter run above (reference: tests/test_rl_stream.py:96-120)."""
+    from ultraviolet_amd.engine import workloads
+    from oracle.model import OracleModel, OracleState
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg, params, eng = _uv50m(16384)
+    prompts, limits = workloads.c5_requests(cfg)
+    assert max(limits) == 2048 and len(prompts) == 2048
+    g = Rollout(eng, slots=2048, max_prompt=256, max_new=2048, temperature=1.0, seed=0, eos_id=None, check_every=16, bucket=128,
+                share_prompts=True, overlap_harvest=True)
+    for i, (p, l) in enumerate(zip(prompts, limits)):
+        g.add(p, i, limit=l)
+    done = []
+    while g.n_decode_steps < 500:
+        done += g.chunk()
+    if g.harvest_pending:
+        done += g.harvest_end()
+    torch.cuda.synchronize()
+    req, cnt, pos = g.slot_req.cpu().numpy(), g.slot_cnt.cpu().numpy(), g.st.pos.cpu().numpy()
+    live = req >= 0
+    n500 = g.n_decode_steps
+    assert (cnt[live] == n500 + 1).all() and 300 < live.sum() < 1200
+    assert np.array_equal(pos[live], np.array([len(prompts[r]) for r in req[live]]) + n500)
+    done += g.run()
+    res = {m: (row, lp) for m, row, lp, _ in done}
+    assert sorted(res) == list(range(2048)) and len(done) == 2048
+    assert all(len(res[i][0]) == limits[i] == len(res[i][1]) for i in range(2048))
+    assert all(0 <= t < cfg.vocab_size for i in range(0, 2048, 37) for t in res[i][0])
+    assert 2047 <= g.n_decode_steps < 2047 + g.ce and g.n_tokens == sum(limits)
+    # ---- the group whose longest member runs to the cap: its four longest sequences through the oracle
+    lim = np.array(limits).reshape(256, 8)
+    gi = int(np.argmax(lim.max(1) * 10000 + np.sort(lim, 1)[:, -4:].sum(1)))
+    ids = [8 * gi + int(j) for j in np.argsort(-lim[gi])[:4]]
+    p = prompts[ids[0]]
+    n = max(limits[i] for i in ids)
+    assert n == 2048 and len(p) + n > 2100
+    toks, lps = np.ones((4, n), np.int64), np.full((4, n), np.nan, np.float32)
+    for j, i in enumerate(ids):
+        toks[j, :limits[i]] = res[i][0]
+        lps[j, :limits[i]] = res[i][1]
+    m = OracleModel(cfg, params, torch.bfloat16)
+    st = OracleState(cfg, 4, len(p) + n + 1)
+    lg = m.logits(m.prefill([p] * 4, list(range(4)), st))
+    ref = np.full((4, n), np.nan, np.float32)
+    ref[:, 0] = torch.log_softmax(lg.float(), -1).gather(1, torch.as_tensor(toks[:, :1])).numpy()[:, 0]
+    for t in range(1, n):
+        lg = m.logits(m.decode_step(toks[:, t - 1], st))
+        ref[:, t] = torch.log_softmax(lg.float(), -1).gather(1, torch.as_tensor(toks[:, t:t + 1])).numpy()[:, 0]
+    ok = ~np.isnan(lps)
+    assert ok.sum() == sum(limits[i] for i in ids) and ok.sum() > 3000
+    d = np.abs(lps[ok] - ref[ok])
+    late = np.abs(lps[:, 1024:][ok[:, 1024:]] - ref[:, 1024:][ok[:, 1024:]])   # past a thousand global keys, few live rows
+    assert np.isfinite(d).all() and late.size > 1000
+    print("teacher-forced log-prob gap over %d tokens: mean %.4f p99 %.4f max %.4f; beyond token 1024 (%d tokens): mean %.4f max %.4f"
+          % (d.size, d.mean(), np.quantile(d, 0.99), d.max(), late.size, late.mean(), late.max()))
+    assert d.mean() < 0.015 and np.quantile(d, 0.99) < 0.05 and d.max() < 0.1, (d.mean(), np.quantile(d, 0.99), d.max())
+    assert late.mean() < 0.015 and late.max() < 0.1
