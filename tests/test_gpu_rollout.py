@@ -200,6 +200,31 @@ def test_rollout_greedy_equals_static_generation():
     assert same >= 11, same     # a near-tie in the top-2 logits may flip under a different GEMM batch shape
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rollout_streams_do_not_depend_on_slot_placement(dtype):
+    """With the launch plan held fixed - the same requests, admitted together, the same number of rows in every step - the
+    slot a request lands in must not matter at all: tokens identical and log-probs bit-equal when the free list hands the
+    slots out in another order (the draws are keyed by request; GEMM and attention results of a row do not depend on where
+    the row sits in the batch).  What other batch SHAPES may change is the next test's subject."""
+    from ultraviolet_amd.engine.rollout import Rollout
+    cfg, eng = _engine(dtype, window=32)
+    rng = np.random.default_rng(21)
+    prompts = [rng.integers(2, cfg.vocab_size, size=int(rng.integers(3, 30))).tolist() for _ in range(8)]
+    outs = []
+    for order in (None, [3, 7, 0, 5, 1, 6, 2, 4], list(range(8))):
+        g = Rollout(eng, slots=8, max_prompt=32, max_new=40, temperature=1.0, seed=11, check_every=8, bucket=8)
+        if order is not None:
+            g.free = list(order)
+        for i, p in enumerate(prompts):
+            g.add(p, i, limit=40)
+        outs.append({m: (row, np.asarray(lp)) for m, row, lp, _ in g.run(max_chunks=50)})
+        assert sorted(outs[-1]) == list(range(8))
+    for o in outs[1:]:
+        for k in range(8):
+            assert o[k][0] == outs[0][k][0], k
+            assert np.array_equal(o[k][1].view(np.int32), outs[0][k][1].view(np.int32)), k
+
+
 def test_rollout_sampling_is_slot_and_batch_independent():
     from ultraviolet_amd.engine.rollout import Rollout
     cfg, eng = _engine(torch.float32)
