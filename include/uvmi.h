@@ -128,14 +128,15 @@ typedef struct uvmi_attn_args {
 } uvmi_attn_args;
 
 /* Fused QKV post-processing for decode rows (uvmi_attn_args.fuse).  The attention kernel then does what uvmi_qkv_post
- * does for the row's own token (QK-norm, partial rotation, value embedding, int8 append at pos[b] - the reference's
- * Attention.qkv + fast_decode.py:291-294, 315-317) and attends the cached range lo..pos-1 plus that key from registers,
+ * does for the row's own token (QK-norm, partial rotation, value embedding, append at pos[b]: int8 codes and fp16 scales,
+ * or k and v themselves on a cache held in the q dtype - the reference's Attention.qkv + fast_decode.py:291-294, 315-317) and attends the cached range lo..pos-1 plus that key from registers,
  * so the step needs no separate post-processing launch.  `qkv` is the output of the projection GEMM, (B, row_stride)
  * in the q dtype: H*64 q values, KH*64 k, KH*64 v, then at column ext_col the H gate logits (W_gate[h] . xn[:gate_ch],
  * formed by appending the gate rows to the projection weight) and the KH value-embedding gate logits.  q / sqb / sqh of
  * the attention arguments are ignored; k_cache, v_cache and the scales are written at the rows' positions.  The XSA /
  * gate epilogue is always applied (post_vhat and post_gate are ignored: the kernel forms them; post_xsa may be NULL).
- * Needs the MFMA path (head_dim 64, int8 cache), num_splits == 1, q dtype = activation dtype, n_pairs 16 when rope. */
+ * Needs the MFMA path (head_dim 64, an int8 cache or one in the q dtype), num_splits == 1, q dtype = activation dtype,
+ * n_pairs 16 when rope. */
 typedef struct uvmi_attn_qkv_fuse {
   const void* qkv; int64_t row_stride;     /* elements */
   int ext_col;                             /* first gate-logit column */

@@ -317,7 +317,7 @@ def test_patch_model_binds_the_reference_entry_points():
         fd.patch_model(_StubModel(cfg, params), kv_dtype="fp8")
 
 
-def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 26), max_len=96):
+def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 26), max_len=96, kv_dtype="int8"):
     """Run the same teacher-forced decode with and without the fused QKV path from identical prefilled states; after every
     step the fused state's caches are overwritten with the unfused ones so that differences do not accumulate.  Returns
     per-step hidden differences, argmax agreement of the logits and per-layer cache statistics."""
@@ -326,7 +326,8 @@ def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 2
     prompts = _prompts(cfg, lens, seed=11)
     B = len(prompts)
     cont = np.random.default_rng(12).integers(1, cfg.vocab_size, size=(B, steps))
-    sts = [KVState(cfg, B, max_len, DEV) for _ in range(2)]
+    sts = [KVState(cfg, B, max_len, DEV, kv_dtype=kv_dtype, dtype=eng.dtype) for _ in range(2)]
+    bits = (lambda t: t.int()) if kv_dtype == "int8" else (lambda t: t.view(torch.int16).int())   # an unquantized cache: compared bit for bit
     for st in sts:
         eng.prefill(prompts, list(range(B)), st)
     hdiff, agree, cmax, cfrac, sfrac = [], [], np.zeros(cfg.n_layers), np.zeros(cfg.n_layers), np.zeros(cfg.n_layers)
@@ -345,13 +346,15 @@ def _fused_vs_unfused(cfg, eng, steps=40, resync=True, lens=(5, 40, 17, 33, 1, 2
         for l in range(cfg.n_layers):
             for a, b_, sa, sb in ((sts[0].k[l], sts[1].k[l], sts[0].k_scale[l], sts[1].k_scale[l]),
                                   (sts[0].v[l], sts[1].v[l], sts[0].v_scale[l], sts[1].v_scale[l])):
-                d = (a.int() - b_.int()).abs()
+                d = (bits(a) - bits(b_)).abs()
                 cmax[l] = max(cmax[l], int(d.max()))
                 cfrac[l] = max(cfrac[l], float((d > 0).float().sum()) / (B * cfg.n_kv_heads * cfg.head_dim))   # of the bytes written this step
-                sfrac[l] = max(sfrac[l], float((sa.view(torch.int16) != sb.view(torch.int16)).float().sum()) / (B * cfg.n_kv_heads))
+                if sa is not None:
+                    sfrac[l] = max(sfrac[l], float((sa.view(torch.int16) != sb.view(torch.int16)).float().sum()) / (B * cfg.n_kv_heads))
                 if resync:
                     b_.copy_(a)
-                    sb.copy_(sa)
+                    if sa is not None:
+                        sb.copy_(sa)
     assert sts[0].pos.tolist() == sts[1].pos.tolist()
     return hdiff, agree, cmax, cfrac, sfrac
 
@@ -437,6 +440,33 @@ def test_fused_qkv_single_layer_is_exact_with_several_waves_per_row(dtype, lens,
         assert cmax.max() == 0 and sfrac.max() == 0
         ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
         assert max(hdiff) <= 4 * 2 * ulp, max(hdiff)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_qkv_on_an_unquantized_cache(dtype):
+    """kv_dtype="fp16" (K/V cached in the activation type): the fused launch appends the token's k and v as they are.  One
+    layer: the appended cache words equal the separate post-processing kernel's bit for bit - ring layer with rotation and
+    value embedding through wrap-around, and a global layer; 1, 2 and 4 waves per row - and the layer output agrees to a
+    few units in the last place (the own key's score is an fp32 dot product here and an MFMA column there).  Whole models:
+    layer 0's words stay identical and the final hidden states within the bound of the int8 tests."""
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for over, lens, max_len in ((dict(window=32, global_every=0, ve_every=1), (5, 40, 17, 33, 1, 26), 96),
+                                (dict(window=0, global_every=1, ve_every=0), (5, 40, 17, 33, 1, 26), 96),
+                                (dict(window=128, global_every=0, ve_every=1), (100, 130, 90, 150, 129, 64), 192),
+                                (dict(window=0, global_every=1, ve_every=0), (300, 20, 260, 330, 1, 300), 1056)):
+        cfg, params, eng, _ = _setup("uv-test", dtype=dtype, perturb=0.05, n_layers=1, attn_gate_channels=128, **over)
+        assert eng.fuse_qkv
+        from ultraviolet_amd.engine import KVState
+        assert eng.fused_layer_ok(0, KVState(cfg, 2, max_len, DEV, kv_dtype="fp16", dtype=dtype))
+        hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=16, lens=lens, max_len=max_len, kv_dtype="fp16")
+        assert cmax.max() == 0, cmax
+        assert max(hdiff) <= 4 * 2 * ulp, max(hdiff)
+    for name, over in (("uv-test", dict(window=32)), ("uv-50m-alpha", dict())):
+        cfg, params, eng, _ = _setup(name, dtype=dtype, perturb=0.05, **over)
+        hdiff, agree, cmax, cfrac, sfrac = _fused_vs_unfused(cfg, eng, steps=24, kv_dtype="fp16")
+        assert cmax[0] == 0
+        assert max(hdiff) < 16 * 2 * ulp, max(hdiff)
+        _check_agreement(agree, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

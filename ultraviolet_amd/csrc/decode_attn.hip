@@ -171,7 +171,8 @@ struct AttnState {
 // into SGPRs with the wave, so the plan's loads go out without first waiting for a load of the kernel arguments.
 // KV16: the cache holds K / V unquantized in the q dtype (no scales): the same work split, plan, online softmax, merge and
 // epilogue around tiles that go into the MFMAs as they are loaded - no conversion, no bias terms, probabilities rounded to
-// the cache type (a tile is 32 dwords per lane, still 4 waves per SIMD).  Not combined with FUSE.
+// the cache type (a tile is 32 dwords per lane, still 4 waves per SIMD).  With FUSE the own token's k and v are appended
+// as they are (on the cache type's grid already) and the own key's score is q . k in fp32.
 // FAST: the shape of the engine's decode step as compile-time constants - one kv head, 8 query heads, uncut rows, 64-bit
 // indices - so that the item arithmetic, the head masks, the split bookkeeping and the partial-result path fold away
 // (the fixed part of a wave's life is as long as its streaming loop on rows of a few hundred keys).
@@ -321,9 +322,13 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
     float qs = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const uint16_t l16 = float_to_half_bits(x[2 * i]), h16 = float_to_half_bits(x[2 * i + 1]);
-      o[i] = (uint32_t)l16 | ((uint32_t)h16 << 16);
-      qs += half_bits_to_float(l16) + half_bits_to_float(h16);
+      if constexpr (KV16 && QDT == UVMI_BF16) {   // the product runs in the q dtype itself (x is on its grid already)
+        o[i] = (uint32_t)float_to_bf16(x[2 * i]) | ((uint32_t)float_to_bf16(x[2 * i + 1]) << 16);
+      } else {
+        const uint16_t l16 = float_to_half_bits(x[2 * i]), h16 = float_to_half_bits(x[2 * i + 1]);
+        o[i] = (uint32_t)l16 | ((uint32_t)h16 << 16);
+        qs += half_bits_to_float(l16) + half_bits_to_float(h16);
+      }
     }
     qs += dpp_mov<0xb1>(qs); qs += dpp_mov<0x4e>(qs); qs += lane_xor4(qs);
     *(uint4*)&sh_q[iw][hh][8 * cc] = uint4{o[0], o[1], o[2], o[3]};
@@ -358,25 +363,36 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       const float kr = rope_rot(k, lane_xor16(k), kcs, ksn, lane < 16, rq);
       k = lane < 32 ? kr : k;
     }
-    uint16_t sbk;
-    const float kq = quant1(k, sbk);
+    uint16_t sbk = 0;
+    float kq;   // what the cache holds for this lane's dim: the int8 code, or (16-bit cache) k itself
     const int slot = ring_slot(P, rp.pc);
-    if (slot < P.S) {
-      ((int8_t*)P.kc)[(int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + lane] = (int8_t)(int)kq;
-      if (lane == 0) ((uint16_t*)P.ks)[(int64_t)rp.cb * P.ssb + (int64_t)h * P.ssh + slot] = sbk;
+    if constexpr (KV16) {
+      kq = k;   // on the cache type's grid already
+      if (slot < P.S)
+        ((uint16_t*)P.kc)[(int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + lane] =
+            QDT == UVMI_BF16 ? float_to_bf16(k) : float_to_half_bits(k);
+    } else {
+      kq = quant1(k, sbk);
+      if (slot < P.S) {
+        ((int8_t*)P.kc)[(int64_t)rp.cb * P.skb + (int64_t)h * P.skh + (int64_t)slot * P.sks + lane] = (int8_t)(int)kq;
+        if (lane == 0) ((uint16_t*)P.ks)[(int64_t)rp.cb * P.ssb + (int64_t)h * P.ssh + slot] = sbk;
+      }
     }
-    // score of the own key against every head: q as the fp16 operand holds it (lane (head, g): dims 16g..16g+15) . the
-    // int8 codes * k scale, in the units of the streamed scores
+    // score of the own key against every head: q as the operand holds it (lane (head, g): dims 16g..16g+15) . the int8
+    // codes * k scale (16-bit cache: . k), in the units of the streamed scores
     sh_kq[iw][lane] = kq;
     __builtin_amdgcn_wave_barrier();
+    auto qlo = [&](uint32_t w) -> float { return KV16 && QDT == UVMI_BF16 ? __uint_as_float(w << 16) : half_bits_to_float(w & 0xffff); };
+    auto qhi = [&](uint32_t w) -> float { return KV16 && QDT == UVMI_BF16 ? __uint_as_float(w & 0xffff0000u) : half_bits_to_float(w >> 16); };
     float dq = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const float4 c4 = *(const float4*)&sh_kq[iw][16 * g + 4 * i];
-      dq += half_bits_to_float(qr[2 * i] & 0xffff) * c4.x + half_bits_to_float(qr[2 * i] >> 16) * c4.y;
-      dq += half_bits_to_float(qr[2 * i + 1] & 0xffff) * c4.z + half_bits_to_float(qr[2 * i + 1] >> 16) * c4.w;
+      dq += qlo(qr[2 * i]) * c4.x + qhi(qr[2 * i]) * c4.y;
+      dq += qlo(qr[2 * i + 1]) * c4.z + qhi(qr[2 * i + 1]) * c4.w;
     }
-    dq = xsum32(xsum16(dq)) * half_bits_to_float(sbk);
+    dq = xsum32(xsum16(dq));
+    if constexpr (!KV16) dq *= half_bits_to_float(sbk);
     if (lane < 8) {
       sh_cur[iw][lane] = dq;
       sh_post[iw][64 + lane] = P.f_has_gate ? rq(2.0f * rq(1.0f / (1.0f + __expf(-cvt_in(glog))))) : 1.0f;
@@ -390,14 +406,21 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
       v = ve_add(v, gv, cvt_in(raw_ve), rq);
     }
     const float nv = fmaxf(sqrtf(bfly_sum(v * v)), P.f_xsa_eps);
-    uint16_t sbv;
-    const float vq = quant1(v, sbv);
     const int slot = ring_slot(P, rp.pc);
-    if (slot < P.S) {
-      ((int8_t*)P.vc)[(int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + lane] = (int8_t)(int)vq;
-      if (lane == 0) ((uint16_t*)P.vs)[(int64_t)rp.cb * P.stb + (int64_t)h * P.sth + slot] = sbv;
+    if constexpr (KV16) {
+      if (slot < P.S)
+        ((uint16_t*)P.vc)[(int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + lane] =
+            QDT == UVMI_BF16 ? float_to_bf16(v) : float_to_half_bits(v);
+      sh_cur[iw][8 + lane] = v;
+    } else {
+      uint16_t sbv;
+      const float vq = quant1(v, sbv);
+      if (slot < P.S) {
+        ((int8_t*)P.vc)[(int64_t)rp.cb * P.svb + (int64_t)h * P.svh + (int64_t)slot * P.svs + lane] = (int8_t)(int)vq;
+        if (lane == 0) ((uint16_t*)P.vs)[(int64_t)rp.cb * P.stb + (int64_t)h * P.sth + slot] = sbv;
+      }
+      sh_cur[iw][8 + lane] = half_bits_to_float(sbv) * vq;
     }
-    sh_cur[iw][8 + lane] = half_bits_to_float(sbv) * vq;
     sh_post[iw][lane] = v / nv;
   };
 
@@ -1080,7 +1103,6 @@ static bool mfma_ok(const uvmi_attn_args* a) {
 static bool mfma16_ok(const uvmi_attn_args* a) {
   const int G = a->H / a->KH;
   if (a->hd != 64 || G > 8 || a->kv_dtype != a->q_dtype || (a->q_dtype != UVMI_F16 && a->q_dtype != UVMI_BF16)) return false;
-  if (a->fuse) return false;
   if (!(a->scale > 0.f)) return false;
   if (a->ring && (a->S % 32 != 0)) return false;
   if (a->S < 32) return false;  // a whole 32-key tile at slot 0 must exist
@@ -1148,8 +1170,8 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
   P.post_vhat = a->post_vhat; P.post_gate = a->post_gate; P.post_xsa = a->post_xsa; P.post_dt = a->post_round_dtype;
   P.f_qkv = nullptr; P.f_rope_tab = nullptr; P.f_rope_n = 1; P.f_rope = 0;
   if (const uvmi_attn_qkv_fuse* f = a->fuse) {
-    UVMI_REQUIRE(mfma_ok(a) && a->num_splits == 1, UVMI_EUNSUPPORTED,
-                 "uvmi_decode_attn: fused QKV post-processing needs the MFMA kernel (head_dim 64, int8 cache, aligned rows) and num_splits == 1");
+    UVMI_REQUIRE((mfma_ok(a) || mfma16_ok(a)) && a->num_splits == 1, UVMI_EUNSUPPORTED,
+                 "uvmi_decode_attn: fused QKV post-processing needs the MFMA kernel (head_dim 64, int8 cache or one of the q dtype, aligned rows) and num_splits == 1");
     UVMI_REQUIRE(a->out_dtype == a->q_dtype, UVMI_EUNSUPPORTED, "uvmi_decode_attn: fused QKV post-processing writes the q dtype");
     UVMI_REQUIRE(f->qkv && ((uintptr_t)f->qkv % 16) == 0 && f->row_stride % 8 == 0 && f->ext_col >= (a->H + 2 * a->KH) * 64 &&
                      f->row_stride >= f->ext_col + a->H + a->KH, UVMI_EINVAL, "uvmi_decode_attn: bad fused qkv layout");
@@ -1234,10 +1256,18 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 2, false, true>), grid, blk, 0, st, UVMI_LEAD, P); \
     else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, OD, 1, false, true>), grid, blk, 0, st, UVMI_LEAD, P);               \
   } while (0)
+#define UVMI_LF16(QD)                                                                                 \
+  do {                                                                                                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 4, true, true>), grid, blk, 0, st, UVMI_LEAD, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 2, true, true>), grid, blk, 0, st, UVMI_LEAD, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<QD, QD, 1, true, true>), grid, blk, 0, st, UVMI_LEAD, P);               \
+  } while (0)
     const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
     // the engine's decode-step shape has an instantiation of its own (see FAST)
     const bool fast = !kv16 && a->num_splits == 1 && a->KH == 1 && a->H == 8 && a->idx_dtype == UVMI_I64;
-    if (kv16) {
+    if (kv16 && a->fuse) {
+      if (a->q_dtype == UVMI_F16) UVMI_LF16(UVMI_F16); else UVMI_LF16(UVMI_BF16);
+    } else if (kv16) {
       if (a->q_dtype == UVMI_F16) {
         if (od == UVMI_F16) UVMI_L16(UVMI_F16, UVMI_F16); else if (od == UVMI_BF16) UVMI_L16(UVMI_F16, UVMI_BF16); else UVMI_L16(UVMI_F16, UVMI_F32);
       } else {
@@ -1256,6 +1286,7 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
 #undef UVMI_LF
 #undef UVMI_LFAST
 #undef UVMI_L16
+#undef UVMI_LF16
 #undef UVMI_LEAD
   } else {
     const dim3 grid((unsigned)P.n_items), blk(64);

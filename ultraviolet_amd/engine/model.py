@@ -275,7 +275,7 @@ class UVEngine:
     def fused_layer_ok(self, l: int, st: KVState) -> bool:
         """Whether layer l's decode attention can take the fused path: the MFMA kernel streams 32-key tiles."""
         S = st.k[l].size(2)
-        return self.fuse_qkv and st.quantized and S % 32 == 0 and S >= 32
+        return self.fuse_qkv and (st.quantized or st.k[l].dtype == self.dtype) and S % 32 == 0 and S >= 32
 
     def rope_table(self, n_positions: int) -> Tensor:
         """cos / sin of every position below n_positions in the activation type's rounding, built once per size."""

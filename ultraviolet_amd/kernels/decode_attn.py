@@ -217,7 +217,8 @@ def decode_attention_fused(qkv: Tensor, H: int, k_cache: Tensor, v_cache: Tensor
                            window: int, ring: bool, k_scale: Tensor, v_scale: Tensor, xsa: Tensor | None, out: Tensor,
                            fuse: dict, rows: Tensor | None = None) -> Tensor:
     """A decode step's attention straight from the projection output: the kernel normalises and rotates q and k of each
-    row's token, adds the value embedding to v, appends k and v (int8) to the cache at pos, attends lo..pos and applies
+    row's token, adds the value embedding to v, appends k and v to the cache at pos (int8 codes and scales, or the values
+    themselves on a cache of the activation type), attends lo..pos and applies
     the XSA / gate epilogue (ultraviolet/model.py:302-333, kernels/fast_decode.py:291-325 of the reference in one launch).
     qkv (B, row) holds H*64 q, K*64 k, K*64 v and, from column fuse["ext_col"], the H gate logits and K value-embedding
     gate logits; see uvmi_attn_qkv_fuse in include/uvmi.h for the other entries of `fuse`.  The caches are written."""
