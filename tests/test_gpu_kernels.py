@@ -770,3 +770,63 @@ def test_big_tile_gemm_rejects_what_it_cannot_do():
         with pytest.raises(UvmiError):
             gemm_tn(a, w, torch.empty(300, 68, device="cuda", dtype=torch.bfloat16)[:, :64], config=config)   # pitch 68
         gemm_tn(a, w, config=config)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rope,ring,has_ve,gate", [(1, 1, 1, 1), (0, 0, 0, 1), (1, 1, 0, 0), (1, 0, 1, 1)])
+def test_qkv_post_engine_shape_kernel_equals_the_general_kernel(dtype, rope, ring, has_ve, gate):
+    """uvmi_qkv_post runs a kernel of its own for the engine's shape (8 heads on 1 kv head, 16 rotated pairs, rotation
+    table, logits from the projection, q in the activation type) that requests a row's inputs in two rounds.  Asked for
+    fp32 queries the same call runs the general kernel; the two must agree bit for bit in everything they write - q (the
+    same values), k, v, v_hat, the gates, the appended int8 rows and their scales - on rows inside and past the rotation
+    table, rows without a cache row, and a ring that keeps only a prompt's last S positions."""
+    import ctypes as C
+    from ultraviolet_amd import _lib as L
+    from ultraviolet_amd.kernels.decode_attn import rope_table
+    g = torch.Generator(device="cuda").manual_seed(5 + rope + 2 * ring + 4 * has_ve)
+    n, H, S, B, vocab, ld = 333, 8, 64, 40, 500, 656
+    qkv = (torch.randn(n, ld, device="cuda", generator=g) * 1.5).to(dtype)
+    pos = torch.randint(0, 150, (n,), device="cuda", generator=g)
+    rows = torch.randint(-1, B, (n,), device="cuda", generator=g)
+    seen, rl = set(), rows.tolist()
+    for i, (rw, ps) in enumerate(zip(rl, pos.tolist())):     # no two rows write the same cache slot (the winner would be a race)
+        cell = (rw, ps % S if ring else ps)
+        if cell in seen:
+            rl[i] = -1
+        seen.add(cell)
+    rows = torch.tensor(rl, device="cuda")
+    last = pos + torch.randint(0, 100, (n,), device="cuda", generator=g)
+    tok = torch.randint(-3, vocab + 3, (n,), device="cuda", generator=g)     # (out-of-range ids are clamped)
+    ve = torch.randn(vocab, 64, device="cuda", generator=g).to(dtype)
+    inv_freq = (1.0 / (1024.0 ** (torch.arange(16, device="cuda").float() / 16))).contiguous()
+    tab = rope_table(inv_freq, 100, dtype)                                    # positions 100 .. 149 lie past the table
+    outs = []
+    for qdt in (dtype, torch.float32):
+        q = torch.zeros(n, H, 64, device="cuda", dtype=qdt)
+        k, v = torch.zeros(n, 64, device="cuda", dtype=dtype), torch.zeros(n, 64, device="cuda", dtype=dtype)
+        vhat, gt = torch.zeros(n, 64, device="cuda"), torch.zeros(n, H, device="cuda")
+        kc, vc = (torch.zeros(B, 1, S, 64, device="cuda", dtype=torch.int8) for _ in range(2))
+        ks, vs = (torch.zeros(B, 1, S, device="cuda", dtype=torch.float16) for _ in range(2))
+        a = L.QkvPostArgs()
+        a.qkv, a.dtype, a.qkv_ld, a.ext_logits = qkv.data_ptr(), L.dtype_code(dtype), ld, 1
+        a.pos, a.rows, a.last_pos, a.inv_freq = pos.data_ptr(), rows.data_ptr(), last.data_ptr() if ring else None, inv_freq.data_ptr()
+        if has_ve:
+            a.ve_table, a.tok = ve.data_ptr(), tok.data_ptr()
+        a.q_out, a.q_dtype, a.k_out, a.v_out = q.data_ptr(), L.dtype_code(qdt), k.data_ptr(), v.data_ptr()
+        a.k_cache, a.v_cache, a.k_scale, a.v_scale = kc.data_ptr(), vc.data_ptr(), ks.data_ptr(), vs.data_ptr()
+        a.scb, a.sch, a.scs, a.ssb, a.ssh, a.S = kc.stride(0), kc.stride(1), kc.stride(2), ks.stride(0), ks.stride(1), S
+        a.n, a.vocab, a.H, a.KH, a.hd, a.d, a.n_pairs = n, vocab, H, 1, 64, 640, 16
+        a.ring, a.has_ve, a.rope, a.eps, a.xsa_eps = ring, has_ve, rope, 1e-6, 1e-4
+        if rope:
+            a.rope_table, a.rope_positions = tab.data_ptr(), tab.size(0)
+        a.vhat_out = vhat.data_ptr()
+        if gate:
+            a.gate_out = gt.data_ptr()
+        L.check(L.lib().uvmi_qkv_post(C.byref(a), L.stream_ptr(qkv)), "uvmi_qkv_post")
+        torch.cuda.synchronize()
+        outs.append((q.float(), k, v, vhat, gt, kc, vc, ks, vs))
+    names = ("q", "k", "v", "v_hat", "gate", "k cache", "v cache", "k scale", "v scale")
+    for nm, x, y in zip(names, *outs):
+        assert torch.equal(x, y), nm
+    assert float(outs[0][5].float().abs().sum()) > 0 and float(outs[0][0].abs().sum()) > 0

@@ -308,6 +308,118 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
   }
 }
 
+// The same post-processing for the engine's shape - 8 query heads on one kv head, 16 rotated pairs with the rotation
+// table, gate logits formed by the projection (ext), q written in the activation type - with everything a row needs
+// requested in two rounds: first what depends on the row index alone (position, cache row, token, the row's q / k / v and
+// logits), then what depends on those (the rotation table's row, the value embedding).  The general kernel above meets
+// these loads one after the other between branches and loops, a chain of six memory latencies per row; the arithmetic,
+// its order and its roundings are the same, so the two kernels agree bit for bit.
+template <int DT>
+__global__ __launch_bounds__(256) void qkv_post_fast_kernel(QkvArgs A) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= A.n) return;
+  constexpr int W = 10 * 64;
+  auto rnd = [](float f) { return round_t<DT>(f); };
+  const int64_t base = r * A.ld;
+  const int hh = lane >> 3, c = lane & 7;
+  // ---- round 1
+  const int64_t p = A.pos[r];
+  const int64_t row = A.rows ? A.rows[r] : r;
+  const int64_t lastp = A.last_pos ? A.last_pos[r] : 0;
+  int64_t t = A.has_ve ? A.tok[r] : 0;
+  float x[8];
+  ld8<DT>(A.qkv, base + hh * 64 + 8 * c, x);
+  float k = elem<DT>::ld(A.qkv, base + 8 * 64 + lane);
+  float v = elem<DT>::ld(A.qkv, base + 9 * 64 + lane);
+  const float glog = A.gate_out ? elem<DT>::ld(A.qkv, base + W + hh) : 0.f;
+  const float vlog = A.has_ve ? elem<DT>::ld(A.qkv, base + W + 8) : 0.f;
+  // ---- round 2
+  const bool in_tab = p >= 0 && p < A.rope_n;   // (wave-uniform)
+  const float* tab = A.rope_tab + (in_tab ? p : 0) * 32;
+  float cs[8], sn[8], cs1 = 1.f, sn1 = 0.f;
+  if (A.rope) {
+    const float* tq = tab + 8 * (c & 1);   // dim 8 c + j turns by frequency (8 c + j) % 16
+    const float4 c0 = *(const float4*)tq, c1 = *(const float4*)(tq + 4), s0 = *(const float4*)(tq + 16), s1 = *(const float4*)(tq + 20);
+    cs[0] = c0.x; cs[1] = c0.y; cs[2] = c0.z; cs[3] = c0.w; cs[4] = c1.x; cs[5] = c1.y; cs[6] = c1.z; cs[7] = c1.w;
+    sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+    cs1 = tab[lane & 15];
+    sn1 = tab[16 + (lane & 15)];
+  }
+  if (t < 0) t = 0;
+  if (t >= A.vocab) t = A.vocab - 1;
+  const float ve = A.has_ve ? elem<DT>::ld(A.ve_table, t * 64 + lane) : 0.f;
+  if (A.rope && !in_tab) {   // a position outside the table: the angles are formed here, as the general kernel does
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float th = (float)p * A.inv_freq[8 * (c & 1) + j];
+      cs[j] = rnd(cosf(th));
+      sn[j] = rnd(sinf(th));
+    }
+    const float th = (float)p * A.inv_freq[lane & 15];
+    cs1 = rnd(cosf(th));
+    sn1 = rnd(sinf(th));
+  }
+  // ---- queries: lane (hh, c) owns dims 8c..8c+7 of head hh
+  {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+    ss += lane_xor1(ss); ss += lane_xor2(ss); ss += lane_xor4(ss);
+    const float rs = rsqrtf(ss * (1.0f / 64.0f) + A.eps);
+#pragma unroll
+    for (int j = 0; j < 8; j++) x[j] = rnd(x[j] * rs);
+    if (A.rope) {
+      float y[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) y[j] = lane_xor2(x[j]);   // partner chunk: c <-> c ^ 2 inside the head
+      if (c < 4) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = rope_rot(x[j], y[j], cs[j], sn[j], c < 2, rnd);
+      }
+    }
+    st8<DT>(A.q_out, (r * 8 + hh) * 64 + 8 * c, x);
+    if (A.gate_out && c == 0) A.gate_out[r * 8 + hh] = rnd(2.0f * rnd(1.0f / (1.0f + __expf(-glog))));
+  }
+  // ---- key and value: lane = dim
+  {
+    const float rs = rsqrtf(wave_sum(k * k) * (1.0f / 64.0f) + A.eps);
+    k = rnd(k * rs);
+    if (A.rope) {
+      const float other = lane_xor16(k);
+      if (lane < 32) k = rope_rot(k, other, cs1, sn1, lane < 16, rnd);
+    }
+  }
+  if (A.has_ve) {
+    const float g = rnd(2.0f * rnd(1.0f / (1.0f + __expf(-vlog))));
+    v = ve_add(v, g, ve, rnd);
+  }
+  if (A.k_out) elem<DT>::st(A.k_out, r * 64 + lane, k);
+  if (A.v_out) elem<DT>::st(A.v_out, r * 64 + lane, v);
+  if (A.vhat_out) {
+    const float nv = sqrtf(wave_sum(v * v));
+    A.vhat_out[r * 64 + lane] = v / fmaxf(nv, A.xsa_eps);
+  }
+  const int64_t slot = A.ring ? (p % A.S) : p;
+  bool wr = A.k_cache && row >= 0 && p >= 0 && slot < A.S;
+  if (wr && A.ring && A.last_pos) wr = p > lastp - A.S;
+  if (wr) {
+    const float vals[2] = {k, v};
+    int8_t* caches[2] = {A.k_cache, A.v_cache};
+    uint16_t* scales[2] = {A.k_scale, A.v_scale};
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const float am = wave_max(fabsf(vals[j]));
+      const uint16_t sb = float_to_half_bits(__fdiv_rn(am, 127.0f));
+      const float sf = fmaxf(half_bits_to_float(sb), 1e-30f);
+      float qv = __builtin_rintf(__fdiv_rn(vals[j], sf));
+      qv = fminf(fmaxf(qv, -127.0f), 127.0f);
+      caches[j][row * A.scb + slot * A.scs + lane] = (int8_t)(int)qv;
+      if (lane == 0) scales[j][row * A.ssb + slot] = sb;
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ attn_post (hd = 64)
 struct PostArgs {
   const void* z; const void* v; const void* xn; const float* gate_w; const float* xsa;
@@ -479,7 +591,14 @@ extern "C" int uvmi_qkv_post(const uvmi_qkv_post_args* a, void* stream) {
   A.ld = a->qkv_ld ? a->qkv_ld : qkv_w;
   A.ext = a->ext_logits != 0;
   const dim3 grid((unsigned)((a->n + 3) / 4)), blk(256);
-  dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
+  const bool fast = (a->dtype == UVMI_F16 || a->dtype == UVMI_BF16) && a->q_dtype == a->dtype && a->H == 8 && a->KH == 1 && A.ext &&
+                    (!a->rope || (a->n_pairs == 16 && A.rope_tab && ((uintptr_t)A.rope_tab % 16) == 0));
+  if (fast) {
+    if (a->dtype == UVMI_F16) hipLaunchKernelGGL((qkv_post_fast_kernel<UVMI_F16>), grid, blk, 0, (hipStream_t)stream, A);
+    else hipLaunchKernelGGL((qkv_post_fast_kernel<UVMI_BF16>), grid, blk, 0, (hipStream_t)stream, A);
+  } else {
+    dispatch_dt(a->dtype, [&](auto DT) { hipLaunchKernelGGL((qkv_post_kernel<decltype(DT)::value>), grid, blk, 0, (hipStream_t)stream, A); });
+  }
   UVMI_CHECK_LAUNCH("uvmi_qkv_post");
   return UVMI_OK;
 }
