@@ -139,6 +139,8 @@ class UVEngine:
         # the folded plan's down projection runs on this library's tiled GEMM between these row counts (measured inside the
         # decode step: 4 - 11 us per step faster than the vendor library's there, slower below and above)
         self.fold_down_rows = (int(fold_down_rows[0]), int(fold_down_rows[1]))
+        self.head_own_rows = 448       # decode steps of at most this many rows run the head GEMM on this library's kernel (own_head_ok)
+        self.hidden_is_raw = False
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
             self.buf["qkvx"] = e(n, UVWeights.qkv_ext_rows(cfg))
@@ -327,10 +329,12 @@ class UVEngine:
                                (b["vhat"][:n], None if W["attn_gate"] is None else b["gate"][:n], W["xsa"], out.dtype))
 
     def _trunk(self, tok: Tensor, pos: Tensor, n: int, attn, rows=None, last_pos=None, st: KVState | None = None,
-               fused_attn=None) -> Tensor:
+               fused_attn=None, defer_final_norm: bool = False) -> Tensor:
         """n token rows through all layers; attn(l, q (n, H, hd)) -> z (n, H, hd) (or None when it wrote the post-processed
         result to buf zg itself) runs after K/V of the layer have been appended to the cache and written unquantized to
-        buf k / v.  Returns the final normed hidden (n, d) (a buffer)."""
+        buf k / v.  Returns the final normed hidden (n, d) (a buffer).  defer_final_norm: a plan whose last block leaves the
+        hidden un-normalised returns it as it is and sets self.hidden_is_raw - the caller's head GEMM then carries the final
+        norm as the row scale of its product (head_of), and the norm launch goes away."""
         cfg, b = self.cfg, self.buf
         assert n <= self.max_tokens
         self._embed_norm(tok, n)
@@ -350,8 +354,9 @@ class UVEngine:
         # the QKV projection with the pre-norm in it is still faster on the skinny kernel).
         folded = (not skinny and fused_attn is not None and self.fold and self.dtype != torch.float32
                   and all(self.fused_layer_ok(l, st) for l in range(cfg.n_layers)) and cfg.d_ff % 8 == 0)
+        self.hidden_is_raw = False
         if folded:
-            return self._trunk_folded(n, fused_attn)
+            return self._trunk_folded(n, fused_attn, defer_final_norm)
         fold_mlp = not skinny and self.dtype != torch.float32 and cfg.d_ff % 8 == 0 and self.fold
         tiled_gu = (fold_mlp and self.tiled_prefill and n >= 448 and cfg.d_model % 64 == 0
                     and all("gu_il" in W for W in self.w.layers))
@@ -439,10 +444,13 @@ class UVEngine:
                 # x = resid_mlp * h + post_mlp * m ; xn = rmsnorm(x) (next block's pre-norm, or the final norm)
                 self._add_norm(b["h"][:n], b["m"][:n], W["resid_mlp"], W["post_mlp"], n, b["x"], b["xn"])
         if not x_is_normed:
+            if defer_final_norm and self.own_head_ok(n):
+                self.hidden_is_raw = True
+                return x
             self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
         return xn
 
-    def _trunk_folded(self, n: int, fused_attn) -> Tensor:
+    def _trunk_folded(self, n: int, fused_attn, defer_final_norm: bool = False) -> Tensor:
         """The layers of _trunk for a pass of many rows whose every layer takes the fused attention; buf x and xn hold the
         embedded rows and their norm on entry.  Five launches per layer: QKV projection with the block's pre-norm as a row
         scale, fused attention, output projection with the residual update in place, gate-up projection with the MLP's
@@ -484,8 +492,33 @@ class UVEngine:
                 gemm_tn(b["act"][:n], W["down"], x, epilogue=RESID, resid=x, ca=W["resid_mlp"], cb=W["post_mlp"], config=gc)
             else:
                 torch.addmm(x, b["act"][:n], W["down"].t(), beta=W["resid_mlp"], alpha=W["post_mlp"], out=x)
+        if defer_final_norm and self.own_head_ok(n):
+            self.hidden_is_raw = True
+            return x
         self._add_norm(x, x, 1.0, 0.0, n, None, b["xn"])   # the final norm
         return xn
+
+    def own_head_ok(self, n: int) -> bool:
+        """Whether head_of runs the head GEMM of n rows on this library's kernel with the final norm in it: 16-bit engines up
+        to head_own_rows rows.  Measured on UV-50M (32 768 x 640 head) as the time of a whole graph-replayed decode step
+        against the vendor library's GEMM behind a norm launch: 0.327 against 0.335 ms at 128 rows, 0.369 against 0.373 at
+        256, equal at 512 and 1024, 0.546 against 0.543 at 768 - so the switch sits at 448 rows.  (Alone, on cold weights, the
+        kernel takes 11.5 - 25 us at 32 - 384 rows where the vendor library's takes 10 - 22 us plus ~6 us of norm launch; at
+        2048 rows 105 against 87 us.)"""
+        cfg = self.cfg
+        return (self.dtype in (torch.bfloat16, torch.float16) and n <= self.head_own_rows and cfg.d_model % 64 == 0
+                and cfg.d_model >= 128 and cfg.vocab_size % 16 == 0)
+
+    def head_of(self, hidden: Tensor) -> Tensor:
+        """head() of what _trunk(defer_final_norm=True) returned: a raw hidden goes through this library's GEMM with the
+        final norm as the row scale of the product (128 x 128 tiles; 256 x 256 where they fill the device in whole
+        rounds), a normalised one through head()."""
+        if not self.hidden_is_raw:
+            return self.head(hidden)
+        n = hidden.size(0)
+        blocks = -(-n // 256)
+        config = 5 if n > 384 and blocks % 2 == 0 else 6
+        return gemm_tn(hidden, self.w.embed, norm_eps=self.eps, config=config)
 
     def head(self, hidden: Tensor) -> Tensor:
         """Raw tied-head output (n, V) in the activation dtype: the GEMM MathLM.logits runs before .float() and the

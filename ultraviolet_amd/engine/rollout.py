@@ -380,8 +380,8 @@ class Rollout:
             return self._attention(l, q, st, pos, starts, n, act)
 
         fused = (lambda l: e.fused_cache_attention(l, self.tok_c[:n], st, pos, starts, n, rows=act)) if e.fuse_qkv else None
-        h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st, fused_attn=fused)
-        x = e.head(h)
+        h = e._trunk(self.tok_c[:n], pos, n, attn, rows=act, st=st, fused_attn=fused, defer_final_norm=True)
+        x = e.head_of(h)
         # the sampler's launch also commits the rows' tokens (what uvmi_sched_commit_dense does in a launch of its own)
         self._sample(x, self.req_c[:n], self.cnt_c[:n], commit=self._commit_args)
 
