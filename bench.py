@@ -179,17 +179,19 @@ def roofline_c5(make_rollout, eng, cfg, W, K, K_all, every=16, reps=3):
     samples = []   # (events A, events B, bytes global, bytes ring)
     ev_plain = []  # events of the attention-only kernel's sequence A (when the step runs the fused kernel)
 
-    def timed_seq(args_list):
+    def timed_seq(args_list, probe=0):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         scratch.zero_()
         e0.record()
         for _ in range(reps):
             for a in args_list:
-                rc = lib.uvmi_decode_attn(C.byref(a), stream)
+                rc = lib.uvmi_decode_attn_probe(C.byref(a), probe, stream) if probe else lib.uvmi_decode_attn(C.byref(a), stream)
                 if rc:
                     L.check(rc, "uvmi_decode_attn")
         e1.record()
         return e0, e1
+
+    ev_probe = {1: [], 2: []}   # the attention-only launches with half of the kernel's work taken out (uvmi_decode_attn_probe)
 
     in_window = []
     for s in range(W + K_all):
@@ -209,6 +211,10 @@ def roofline_c5(make_rollout, eng, cfg, W, K, K_all, every=16, reps=3):
                         # the engine's buffers hold: only the timing is used)
                 plain = {l: eng.cache_attention_args(l, g.st, pos, starts, n, rows=act) for l in layers}
                 ev_plain.append(timed_seq([plain[l][0] for l in layers]))
+                out_keep = eng.buf["zg"][:n].clone()     # (the probes write meaningless values to the layer output buffer)
+                for mode in (1, 2):
+                    ev_probe[mode].append(timed_seq([plain[l][0] for l in layers], probe=mode))
+                eng.buf["zg"][:n].copy_(out_keep)
             torch.cuda.synchronize()
             live = act.cpu().numpy() >= 0
             p, st = pos.cpu().numpy()[live], starts.cpu().numpy()[live]   # what the kernels saw (padding rows: no keys)
@@ -243,6 +249,12 @@ def roofline_c5(make_rollout, eng, cfg, W, K, K_all, every=16, reps=3):
                           "costs a separate ~10 us launch per layer)",
                 "achieved": round(all_bytes / plain_us / 1e3, 1), "frac": round(all_bytes / plain_us / 1e3 / HBM_PEAK_GBS, 4),
                 "avg_launch_us": round(plain_us, 2), "launches_timed": n_all * ns * reps}
+            pr = {m: sum(a.elapsed_time(b) for (a, b), k in zip(ev_probe[m], sel) if k) * 1e3 / reps / (n_all * ns) for m in (1, 2)}
+            extra["ceiling_probes"] = {
+                "what": "the attention-only launches re-issued through uvmi_decode_attn_probe: mode 1 keeps the kernel's memory stream and drops "
+                        "its arithmetic, mode 2 keeps the arithmetic and reads no cache",
+                "stream_only_us": round(pr[1], 2), "stream_only_frac": round(all_bytes / pr[1] / 1e3 / HBM_PEAK_GBS, 4),
+                "arithmetic_only_us": round(pr[2], 2), "kernel_us": round(plain_us, 2)}
         return {"bound": "hbm", "achieved": round(ab, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ab / HBM_PEAK_GBS, 4),
                 "traffic": int(all_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
                 "kernel": "uvmi::attn_mfma_i8_hd64<1, 1, WPR, FUSE=true> (bf16; all ten layers' launches of a step; the kernel also does the "
@@ -319,6 +331,75 @@ def bench_c2(args):
                       "config": {"workload": "C2 single-layer ragged int8-KV decode attention, cold (32 rotating cache sets)"},
                       "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}))
+
+
+def bench_attn_ceiling(args):
+    """Where the decode-attention kernel's time goes at the rollout's launch shape (2000 rows, 8 heads on 1 kv head, int8 KV,
+    bf16 q, post epilogue): rows of n keys each, n swept from 1 to 1024, over 16 rotating cache sets (more bytes than the
+    last-level cache holds, as in a real step), timed three ways - the kernel, its memory stream without its arithmetic
+    and its arithmetic without the stream (uvmi_decode_attn_probe).  Prints the table and the line fitted through the
+    stream-only times: a fixed cost per launch plus bytes at a marginal rate."""
+    import ctypes as C
+    from ultraviolet_amd import _lib as L
+    from ultraviolet_amd.kernels.decode_attn import build_attn_args
+    lib = L.lib()
+    dev = "cuda:0"
+    B, S, nsets = 2000, 1056, 16
+    g = torch.Generator(device=dev).manual_seed(0)
+    sets = [(torch.randint(-127, 128, (B, 1, S, 64), device=dev, dtype=torch.int8, generator=g),
+             torch.randint(-127, 128, (B, 1, S, 64), device=dev, dtype=torch.int8, generator=g),
+             (torch.rand(B, 1, S, device=dev, generator=g) * 0.03 + 0.01).half(),
+             (torch.rand(B, 1, S, device=dev, generator=g) * 0.03 + 0.01).half()) for _ in range(nsets)]
+    q = torch.randn(B, 8, 64, device=dev, generator=g).bfloat16()
+    out = torch.empty_like(q)
+    vhat = torch.nn.functional.normalize(torch.randn(B, 1, 64, device=dev, generator=g), dim=-1).contiguous()
+    gate = torch.rand(B, 8, device=dev, generator=g) + 0.5
+    xsa = torch.full((8,), 0.3, device=dev)
+    starts = torch.zeros(B, dtype=torch.long, device=dev)
+    rows = torch.arange(B, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    scratch = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    reps = max(2, args.steps // nsets) if args.steps > 0 else 4
+    table = []
+    for n in (1, 64, 128, 192, 256, 512, 1024):
+        pos = torch.full((B,), n - 1, dtype=torch.long, device=dev)
+        built = [build_attn_args(q, s[0], s[1], pos, starts, 0.14125, 0, False, s[2], s[3], 1, out, 0, rows, (vhat, gate, xsa, out.dtype))
+                 for s in sets]
+        byts = _attn_bytes(np.full(B, n - 1), np.zeros(B, np.int64), 0, B)
+        us = {}
+        for mode in (0, 1, 2):
+            def run():
+                for a, _ in built:
+                    rc = lib.uvmi_decode_attn_probe(C.byref(a), mode, stream) if mode else lib.uvmi_decode_attn(C.byref(a), stream)
+                    if rc:
+                        L.check(rc, "uvmi_decode_attn")
+            run()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            scratch.zero_()
+            e0.record()
+            for _ in range(reps):
+                run()
+            e1.record()
+            torch.cuda.synchronize()
+            us[mode] = e0.elapsed_time(e1) * 1e3 / (reps * nsets)
+        table.append({"keys_per_row": n, "bytes_per_launch": int(byts), "kernel_us": round(us[0], 2), "stream_only_us": round(us[1], 2),
+                      "arithmetic_only_us": round(us[2], 2), "kernel_GBs": round(byts / us[0] / 1e3, 1),
+                      "stream_only_GBs": round(byts / us[1] / 1e3, 1)})
+    x = np.array([t["bytes_per_launch"] for t in table], float)
+    y = np.array([t["stream_only_us"] for t in table], float)
+    slope, icpt = np.polyfit(x, y, 1)
+    yk = np.array([t["kernel_us"] for t in table], float)
+    slope_k, icpt_k = np.polyfit(x, yk, 1)
+    at = 50.8e6
+    print(json.dumps({"metric": "decode attention launch time by row length (kernel / stream only / arithmetic only)", "value": round(1e-3 / slope, 1),
+                      "unit": "GB/s", "n_gpus": 1, "steps": reps * nsets, "warmup": 1, "ms_per_step": None, "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "decode attention, 2000 rows x n keys (n = 1 .. 1024), int8 KV, 16 rotating cache sets"},
+                      "table": table,
+                      "fit": {"stream_only": {"fixed_us": round(icpt, 2), "marginal_GBs": round(1e-3 / slope, 1)},
+                              "kernel": {"fixed_us": round(icpt_k, 2), "marginal_GBs": round(1e-3 / slope_k, 1)},
+                              "at_50.8_MB": {"stream_only_us": round(icpt + slope * at, 2), "kernel_us": round(icpt_k + slope_k * at, 2),
+                                             "frac_if_only_the_stream_remained": round(at / (icpt + slope * at) / 1e3 / HBM_PEAK_GBS, 4)}}}))
 
 
 def bench_c4(args):
@@ -469,7 +550,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed decode steps (0: the whole rollout after warm-up)")
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy"])
+    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy", "attn-ceiling"])
     ap.add_argument("--host-admit", action="store_true", help="c3: the host chooses the slots of admitted prompts (default: the device does)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -490,6 +571,8 @@ def main():
         bench_c3(args)
     elif args.workload == "c4":
         bench_c4(args)
+    elif args.workload == "attn-ceiling":
+        bench_attn_ceiling(args)
     else:
         bench_c5(args)
 

@@ -167,6 +167,14 @@ int uvmi_default_splits(int64_t n_bk, int ctx, int n_cus);
  * hd <= 256, G <= 16), negative if unsupported.  Mirrors decode_attn_cuda.supported (decode_attn_cuda.py:265-270). */
 int uvmi_decode_attn_path(const uvmi_attn_args* a);
 
+/* Measurement aid, no counterpart in the reference: the launch uvmi_decode_attn would make for these arguments with one
+ * half of the kernel's work taken out - mode 1 keeps the memory stream (every K / V / scale tile is loaded as in the real
+ * kernel and folded into the state with a few xors; no products, no exponentials), mode 2 keeps the arithmetic (tiles are
+ * made up in registers; the cache is not read).  `out` is written with meaningless values.  Timed beside the real launch
+ * the two say which of the kernel's resources bounds it.  Only the engine's decode shape: int8 cache, bf16 q and out, 8
+ * query heads on one kv head, I64 indices, num_splits 1, no fuse; anything else returns UVMI_EUNSUPPORTED. */
+int uvmi_decode_attn_probe(const uvmi_attn_args* a, int mode, void* stream);
+
 /* uvmi_decode_attn for callers that cannot allocate device memory - code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  No counterpart in the reference (its op allocates its split partials per call,
  * ultraviolet/kernels/decode_attn.py:157-159).  Same arguments, kernels and results as uvmi_decode_attn, except that

@@ -830,3 +830,35 @@ def test_qkv_post_engine_shape_kernel_equals_the_general_kernel(dtype, rope, rin
     for nm, x, y in zip(names, *outs):
         assert torch.equal(x, y), nm
     assert float(outs[0][5].float().abs().sum()) > 0 and float(outs[0][0].abs().sum()) > 0
+
+
+@pytest.mark.gpu
+def test_attention_probe_runs_the_engine_shape_and_refuses_the_rest():
+    """uvmi_decode_attn_probe (a measurement aid: the kernel's memory stream without its arithmetic, or the reverse)
+    launches for the engine's decode shape, leaves the caches untouched, returns, and refuses other shapes and modes with an
+    error instead of running something else.  Its output is meaningless and is not checked."""
+    import ctypes as C
+    from ultraviolet_amd import _lib as L
+    from ultraviolet_amd.kernels.decode_attn import build_attn_args
+    g = torch.Generator(device="cuda").manual_seed(3)
+    B, S = 37, 320
+    k, v = (torch.randint(-127, 128, (B, 1, S, 64), device=DEV, dtype=torch.int8, generator=g) for _ in range(2))
+    ks, vs = ((torch.rand(B, 1, S, device=DEV, generator=g) * 0.03 + 0.01).half() for _ in range(2))
+    q = torch.randn(B, 8, 64, device=DEV, generator=g).bfloat16()
+    pos = torch.randint(0, S, (B,), device=DEV, generator=g)
+    starts = torch.zeros(B, dtype=torch.long, device=DEV)
+    out = torch.zeros_like(q)
+    keep = [t.clone() for t in (k, v, ks, vs)]
+    stream = torch.cuda.current_stream().cuda_stream
+    a, alive = build_attn_args(q, k, v, pos, starts, 0.14125, 0, False, ks, vs, 1, out)
+    for mode in (1, 2):
+        assert L.lib().uvmi_decode_attn_probe(C.byref(a), mode, stream) == 0, L.lib().uvmi_last_error()
+    torch.cuda.synchronize()
+    for t, t0 in zip((k, v, ks, vs), keep):
+        assert torch.equal(t, t0)
+    assert L.lib().uvmi_decode_attn_probe(C.byref(a), 3, stream) != 0                     # no such mode
+    a2, alive2 = build_attn_args(q.half(), k, v, pos, starts, 0.14125, 0, False, ks, vs, 1, out.half())
+    assert L.lib().uvmi_decode_attn_probe(C.byref(a2), 1, stream) != 0                    # fp16 queries: not the engine's shape
+    a3, alive3 = build_attn_args(q, k, v, pos.int(), starts.int(), 0.14125, 0, False, ks, vs, 1, out)
+    assert L.lib().uvmi_decode_attn_probe(C.byref(a3), 1, stream) != 0                    # 32-bit indices
+    assert b"probe" in L.lib().uvmi_last_error()

@@ -141,6 +141,7 @@ def lib() -> C.CDLL:
         L.uvmi_decode_attn.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
         L.uvmi_decode_attn_path.argtypes = [C.POINTER(AttnArgs)]
         L.uvmi_decode_attn_noalloc.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+        L.uvmi_decode_attn_probe.argtypes = [C.POINTER(AttnArgs), C.c_int, C.c_void_p]
         L.uvmi_prefill_attn.argtypes = [C.POINTER(PrefillAttnArgs), C.c_void_p]
         L.uvmi_prefill_attn_path.argtypes = [C.POINTER(PrefillAttnArgs)]
         L.uvmi_prefill_attn_workspace_bytes.restype = C.c_size_t
@@ -205,7 +206,7 @@ def require_cuda(*ts: torch.Tensor) -> None:
 
 EXPORTS = ["uvmi_version", "uvmi_last_error", "uvmi_device_cus", "uvmi_quantize_rows", "uvmi_dequantize_rows",
            "uvmi_kv_write", "uvmi_kv_append", "uvmi_decode_attn", "uvmi_decode_attn_workspace_bytes",
-           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_decode_attn_noalloc", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
+           "uvmi_default_splits", "uvmi_decode_attn_path", "uvmi_decode_attn_noalloc", "uvmi_decode_attn_probe", "uvmi_prefill_attn", "uvmi_prefill_attn_workspace_bytes",
            "uvmi_prefill_attn_path", "uvmi_fused_sample", "uvmi_philox4x32_10",
            "uvmi_embed_norm", "uvmi_add_norm", "uvmi_qkv_post", "uvmi_attn_post", "uvmi_swiglu", "uvmi_swiglu_norm",
            "uvmi_prefill_attn_bwd", "uvmi_prefill_attn_bwd_workspace_bytes", "uvmi_sched_compact", "uvmi_sched_commit", "uvmi_sched_commit_dense", "uvmi_sched_admit", "uvmi_sched_expand", "uvmi_sched_harvest", "uvmi_sched_plan_admit", "uvmi_sched_step_plan", "uvmi_rope_table", "uvmi_gemm_tn_supported", "uvmi_gemm_tn", "uvmi_gemm_tn_ex"]

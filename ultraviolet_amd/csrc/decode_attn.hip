@@ -176,7 +176,10 @@ struct AttnState {
 // FAST: the shape of the engine's decode step as compile-time constants - one kv head, 8 query heads, uncut rows, 64-bit
 // indices - so that the item arithmetic, the head masks, the split bookkeeping and the partial-result path fold away
 // (the fixed part of a wave's life is as long as its streaming loop on rows of a few hundred keys).
-template <int QDT, int ODT, int WPR, bool FUSE, bool KV16 = false, bool FAST = false>
+// PROBE (uvmi_decode_attn_probe; measurement only, the output is meaningless): 1 - the kernel's memory stream without its
+// arithmetic: every tile is loaded exactly as in the real kernel and folded into the state with a few xors; 2 - its
+// arithmetic without the stream: tiles are made up in registers, nothing is loaded from the cache.
+template <int QDT, int ODT, int WPR, bool FUSE, bool KV16 = false, bool FAST = false, int PROBE = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_rows, const void* a_q, int64_t a_items, int a_idx64,
                        int a_splits, int a_kh, AttnParams P) {
@@ -473,6 +476,14 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
         T.vA[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + j * usvs, 0);
         T.vB[j] = __builtin_amdgcn_raw_buffer_load_b64(rV, voA, ov + (16 + j) * usvs, 0);
       }
+    } else if constexpr (PROBE == 2) {
+      const uint32_t w = (uint32_t)slot0 * 0x9E3779B1u + (uint32_t)lane * 0x85EBCA6Bu;
+      T.kA = uint4{w, w ^ 0x01234567u, w * 3u, w * 5u};
+      T.kB = uint4{~w, w ^ 0x76543210u, w * 7u, w * 9u};
+#pragma unroll
+      for (int j = 0; j < 4; j++) { T.vA[j] = w + 0x01010101u * j; T.vB[j] = ~w + 0x01010101u * j; }
+      T.ksc = uint2{0x21202120u, 0x21202120u};   // fp16 0.0100 four times
+      T.vsc = uint2{0x21202120u, 0x21202120u};
     } else {
     u4 ka = __builtin_amdgcn_raw_buffer_load_b128(rK, koA, ok, 0);
     u4 kb = __builtin_amdgcn_raw_buffer_load_b128(rK, koB, ok, 0);
@@ -516,6 +527,12 @@ void attn_mfma_i8_hd64(const void* a_pos, const void* a_starts, const void* a_ro
   };
 
   auto step = [&](const TileX& T, int tb, bool edge) {
+    if constexpr (PROBE == 1 && !KV16) {
+      const uint32_t x = T.kA.x ^ T.kA.y ^ T.kA.z ^ T.kA.w ^ T.kB.x ^ T.kB.y ^ T.kB.z ^ T.kB.w ^ T.vA[0] ^ T.vA[1] ^ T.vA[2] ^ T.vA[3] ^
+                         T.vB[0] ^ T.vB[1] ^ T.vB[2] ^ T.vB[3] ^ T.ksc.x ^ T.ksc.y ^ T.vsc.x ^ T.vsc.y;
+      st.psum = __uint_as_float(__float_as_uint(st.psum) ^ x);
+      return;
+    }
     // ---- S^T = K' . Q^T - 1152 sum(q), K' = 1024 + (k ^ 0x80) as fp16 0x64uu (16-bit cache: K as loaded, no bias)
     f4 acc = f4{cinit, cinit, cinit, cinit};
     if constexpr (KV16) {
@@ -1150,7 +1167,7 @@ extern "C" int uvmi_decode_attn_path(const uvmi_attn_args* a) {
 
 // The launch sequence of uvmi_decode_attn with the split partials in `ws` (ws_bytes of device memory; unused when
 // num_splits == 1): the caller's workspace, or this library's own scratch array.
-static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes, const char* who, void* stream) {
+static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes, const char* who, void* stream, int probe = 0) {
   int rc = check_common(a);
   if (rc) return rc;
   if (a->B == 0) return UVMI_OK;
@@ -1265,7 +1282,18 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
     const int od = a->out_dtype;  // rows that fit one chunk are written directly even when num_splits > 1
     // the engine's decode-step shape has an instantiation of its own (see FAST)
     const bool fast = !kv16 && a->num_splits == 1 && a->KH == 1 && a->H == 8 && a->idx_dtype == UVMI_I64;
-    if (kv16 && a->fuse) {
+    if (probe) {
+      UVMI_REQUIRE(fast && !a->fuse && od == a->q_dtype && a->q_dtype == UVMI_BF16, UVMI_EUNSUPPORTED,
+                   "uvmi_decode_attn_probe: only the engine's decode shape (int8 cache, bf16 q and output, 8 heads on 1 kv head, 64-bit indices, one split, no fused QKV)");
+#define UVMI_LP(PR)                                                                                                                   \
+  do {                                                                                                                                \
+    if (wpr == 4) hipLaunchKernelGGL((attn_mfma_i8_hd64<UVMI_BF16, UVMI_BF16, 4, false, false, true, PR>), grid, blk, 0, st, UVMI_LEAD, P);      \
+    else if (wpr == 2) hipLaunchKernelGGL((attn_mfma_i8_hd64<UVMI_BF16, UVMI_BF16, 2, false, false, true, PR>), grid, blk, 0, st, UVMI_LEAD, P); \
+    else hipLaunchKernelGGL((attn_mfma_i8_hd64<UVMI_BF16, UVMI_BF16, 1, false, false, true, PR>), grid, blk, 0, st, UVMI_LEAD, P);               \
+  } while (0)
+      if (probe == 1) UVMI_LP(1); else UVMI_LP(2);
+#undef UVMI_LP
+    } else if (kv16 && a->fuse) {
       if (a->q_dtype == UVMI_F16) UVMI_LF16(UVMI_F16); else UVMI_LF16(UVMI_BF16);
     } else if (kv16) {
       if (a->q_dtype == UVMI_F16) {
@@ -1315,6 +1343,12 @@ static int decode_attn_launch(const uvmi_attn_args* a, void* ws, size_t ws_bytes
 extern "C" int uvmi_decode_attn(const uvmi_attn_args* a, void* stream) {
   UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_decode_attn: null args");
   return decode_attn_launch(a, a->workspace, a->workspace_bytes, "uvmi_decode_attn", stream);
+}
+
+extern "C" int uvmi_decode_attn_probe(const uvmi_attn_args* a, int mode, void* stream) {
+  UVMI_REQUIRE(a, UVMI_EINVAL, "uvmi_decode_attn_probe: null args");
+  UVMI_REQUIRE(mode == 1 || mode == 2, UVMI_EINVAL, "uvmi_decode_attn_probe: mode %d (1: memory stream only, 2: arithmetic only)", mode);
+  return decode_attn_launch(a, a->workspace, a->workspace_bytes, "uvmi_decode_attn_probe", stream, mode);
 }
 
 // ------------------------------------------------------------------------------------ the entry point that allocates nothing
