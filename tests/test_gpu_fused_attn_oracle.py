@@ -224,6 +224,105 @@ def test_fused_launch_matches_oracle_composition(dtype, KH, S, ring, gate):
         assert (dq > 0).sum() <= max(2, 0.004 * n_el), ((dq > 0).sum(), n_el)
 
 
+def _run16(dtype, KH, S, ring, gate, seed, n_live=20):
+    """_run for a cache that holds K / V unquantized in the activation type (the reference's KernelDecodeState with
+    kv_dtype="fp16", kernels/fast_decode.py:21-57): the oracle appends the post-processed k and v as they are
+    (fast_decode.py:315-326 with no quantizer) and attends the float cache."""
+    from oracle import decode_attn as odec
+    from ultraviolet_amd.engine.model import rms_norm_eps
+    from ultraviolet_amd.engine.weights import UVWeights
+    from ultraviolet_amd.kernels.decode_attn import decode_attention_fused, rope_table
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    cfg, params, m = _layer(dtype, KH, S, ring, True, gate, ring, seed)
+    rope = ring
+    d = cfg.d_model
+    n_cache = n_live + 5
+    pos, starts = _positions(S, ring, n_live, rng)
+    tok = rng.integers(0, cfg.vocab_size, size=n_live)
+    xn = torch.randn(n_live, 1, d, generator=g).to(dtype)
+    rnd = lambda a: torch.from_numpy(a).to(dtype).float().numpy()          # onto the cache type's grid
+    kc = rnd(rng.standard_normal((n_cache, KH, S, HD)).astype(np.float32))
+    vc = rnd(rng.standard_normal((n_cache, KH, S, HD)).astype(np.float32))
+    rows_live = rng.permutation(n_cache)[:n_live].astype(np.int64)
+    ok_, ov_ = kc[rows_live].copy(), vc[rows_live].copy()
+    if rope:
+        cos, sin = m._cos_sin(torch.as_tensor(pos))
+        cos, sin = cos[:, None, :], sin[:, None, :]
+    else:
+        cos = sin = torch.zeros(n_live, 1, 0)
+    vemb = m.value_embed[torch.as_tensor(tok)].view(n_live, 1, KH, HD)
+    q, k, v = m._qkv(0, xn, vemb, cos, sin)
+    slot = pos % S if ring else pos
+    ok_[np.arange(n_live), :, slot] = k.reshape(n_live, KH, HD).float().numpy()
+    ov_[np.arange(n_live), :, slot] = v.reshape(n_live, KH, HD).float().numpy()
+
+    def attend(kk, vv):
+        z = odec.decode_attention_ref(q.reshape(n_live, H, HD).float().numpy(), kk, vv, pos, starts, cfg.attn_scale,
+                                      window=S if ring else 0, ring=ring)
+        z = torch.from_numpy(z).to(dtype).view(n_live, 1, H, HD)
+        return m._post(0, z, xn, v)[:, 0, :H * HD].float().numpy().reshape(n_live, H, HD)
+
+    ref = attend(ok_, ov_)
+    exp_k, exp_v = kc.copy(), vc.copy()
+    exp_k[rows_live], exp_v[rows_live] = ok_, ov_
+    n = n_live + 3
+    where = np.sort(rng.permutation(n)[:n_live])
+    rows_d = np.full(n, -1, np.int64)
+    rows_d[where] = rows_live
+    pos_d, starts_d, tok_d = np.zeros(n, np.int64), np.zeros(n, np.int64), np.zeros(n, np.int64)
+    pos_d[where], starts_d[where], tok_d[where] = pos, starts, tok
+    ext = UVWeights.qkv_ext_rows(cfg)
+    qkvx = torch.zeros(n, ext, dtype=dtype)
+    qkvx[where, :d] = xn[:, 0]
+    W0 = m.layers[0]
+    if gate:
+        qkvx[where, d:d + H] = F.linear(xn[..., :cfg.gate_ch], W0["attn_gate"])[:, 0]
+    gw = W0["ve_gate"]
+    qkvx[where, d + H:d + H + KH] = F.linear(xn[..., :gw.size(-1)], gw)[:, 0]
+    dv = lambda a: torch.as_tensor(a).to(DEV)
+    kc_d, vc_d = dv(kc).to(dtype), dv(vc).to(dtype)
+    inv_freq = ((1.0 / cfg.rope_base) ** torch.linspace(0, 1, cfg.n_pairs, dtype=torch.float32)).to(DEV) if rope else None
+    fuse = dict(ext_col=d, has_gate=gate, tok=dv(tok_d), ve_table=m.value_embed.to(DEV).contiguous(), vocab=cfg.vocab_size,
+                rope_table=rope_table(inv_freq, int(pos.max()) + 1, dtype) if rope else None, n_pairs=cfg.n_pairs, rope=rope,
+                eps=rms_norm_eps(dtype), xsa_eps=cfg.xsa_eps)
+    out = torch.full((n, H, HD), float("nan"), dtype=dtype, device=DEV)
+    decode_attention_fused(qkvx.to(DEV), H, kc_d, vc_d, dv(pos_d), dv(starts_d), cfg.attn_scale, window=S if ring else 0, ring=ring,
+                           k_scale=None, v_scale=None, xsa=W0["xsa"].to(DEV).contiguous(), out=out, fuse=fuse, rows=dv(rows_d))
+    torch.cuda.synchronize()
+    out = out.float().cpu().numpy()
+    pad = np.setdiff1d(np.arange(n), where)
+    assert np.all(out[pad] == 0), "padding rows must produce zeros"
+    got_k, got_v = kc_d.float().cpu().numpy(), vc_d.float().cpu().numpy()
+    written = np.zeros((n_cache, KH, S), bool)
+    written[rows_live, :, slot] = True
+    ref_got = attend(got_k[rows_live], got_v[rows_live])
+    return dict(out=out[where], ref=ref, ref_got=ref_got, got=(got_k, got_v), exp=(exp_k, exp_v), written=written)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("KH", [1, 2])
+@pytest.mark.parametrize("S,ring", [(64, True), (128, True), (256, True), (64, False), (160, False), (1056, False)])
+@pytest.mark.parametrize("gate", [False, True])
+def test_fused_launch_on_an_unquantized_cache_matches_oracle_composition(dtype, KH, S, ring, gate):
+    """The same launch on a cache held in the activation type: the appended k and v words equal the oracle's post-processed
+    k and v except where a last-place difference of the reciprocal square root or the sigmoid moved a value by one unit of
+    the activation type (rare), nothing else in the cache changes, and the gated outputs match the oracle's attention over
+    the cache the launch produced to the attention bar (1, 2 and 4 waves per row; ring wrap-around; 8 and 4 heads per kv head)."""
+    r = _run16(dtype, KH, S, ring, gate, seed=11 * S + KH + int(gate))
+    w = r["written"]
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for g_, e_ in zip(r["got"], r["exp"]):
+        assert np.array_equal(g_[~w], e_[~w])
+        diff = np.abs(g_[w] - e_[w])
+        assert (diff <= 2 * ulp * np.maximum(np.abs(e_[w]), 1.0)).all(), float(diff.max())
+        assert (diff > 0).mean() < 0.01, float((diff > 0).mean())
+    err = np.abs(r["out"] - r["ref_got"])
+    tol = _tol(r["ref_got"], dtype, 1 + int(gate))
+    assert (err <= tol).all(), float((err / tol).max())
+    assert err.mean() < (2e-4 if dtype == torch.bfloat16 else 1e-4), err.mean()
+
+
 def test_dequantize_rows_is_the_exact_product():
     """dequantize_kv (kernels/kv_quant.py:22-23): q * s is exact in fp32 (7 + 11 significant bits), so the kernel's fp32
     output must equal it bit for bit and its 16-bit outputs the round-to-nearest-even cast of it."""
