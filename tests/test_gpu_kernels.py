@@ -777,7 +777,7 @@ def test_big_tile_gemm_rejects_what_it_cannot_do():
 @pytest.mark.parametrize("rope,ring,has_ve,gate", [(1, 1, 1, 1), (0, 0, 0, 1), (1, 1, 0, 0), (1, 0, 1, 1)])
 def test_qkv_post_engine_shape_kernel_equals_the_general_kernel(dtype, rope, ring, has_ve, gate):
     """uvmi_qkv_post runs a kernel of its own for the engine's shape (8 heads on 1 kv head, 16 rotated pairs, rotation
-    table, logits from the projection, q in the activation type) that requests a row's inputs in two rounds.  Asked for
+    table, logits from the projection, q in the activation type) that requests a row's inputs in two batches.  Asked for
     fp32 queries the same call runs the general kernel; the two must agree bit for bit in everything they write - q (the
     same values), k, v, v_hat, the gates, the appended int8 rows and their scales - on rows inside and past the rotation
     table, rows without a cache row, and a ring that keeps only a prompt's last S positions."""

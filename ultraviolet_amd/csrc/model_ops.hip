@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvArgs A) {
 
 // The same post-processing for the engine's shape - 8 query heads on one kv head, 16 rotated pairs with the rotation
 // table, gate logits formed by the projection (ext), q written in the activation type - with everything a row needs
-// requested in two rounds: first what depends on the row index alone (position, cache row, token, the row's q / k / v and
+// requested in two batches: first what depends on the row index alone (position, cache row, token, the row's q / k / v and
 // logits), then what depends on those (the rotation table's row, the value embedding).  The general kernel above meets
 // these loads one after the other between branches and loops, a chain of six memory latencies per row; the arithmetic,
 // its order and its roundings are the same, so the two kernels agree bit for bit.
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256) void qkv_post_fast_kernel(QkvArgs A) {
   auto rnd = [](float f) { return round_t<DT>(f); };
   const int64_t base = r * A.ld;
   const int hh = lane >> 3, c = lane & 7;
-  // ---- round 1
+  // ---- requests that depend on the row index alone
   const int64_t p = A.pos[r];
   const int64_t row = A.rows ? A.rows[r] : r;
   const int64_t lastp = A.last_pos ? A.last_pos[r] : 0;
@@ -334,7 +334,7 @@ __global__ __launch_bounds__(256) void qkv_post_fast_kernel(QkvArgs A) {
   float v = elem<DT>::ld(A.qkv, base + 9 * 64 + lane);
   const float glog = A.gate_out ? elem<DT>::ld(A.qkv, base + W + hh) : 0.f;
   const float vlog = A.has_ve ? elem<DT>::ld(A.qkv, base + W + 8) : 0.f;
-  // ---- round 2
+  // ---- requests that depend on the position and the token
   const bool in_tab = p >= 0 && p < A.rope_n;   // (wave-uniform)
   const float* tab = A.rope_tab + (in_tab ? p : 0) * 32;
   float cs[8], sn[8], cs1 = 1.f, sn1 = 0.f;
