@@ -139,7 +139,7 @@ class UVEngine:
         # the folded plan's down projection runs on this library's tiled GEMM between these row counts (measured inside the
         # decode step: 4 - 11 us per step faster than the vendor library's there, slower below and above)
         self.fold_down_rows = (int(fold_down_rows[0]), int(fold_down_rows[1]))
-        self.head_own_rows = 448       # decode steps of at most this many rows run the head GEMM on this library's kernel (own_head_ok)
+        self.head_own_rows = 288       # decode steps of at most this many rows run the head GEMM on this library's kernel (own_head_ok)
         self.hidden_is_raw = False
         self._rope_tabs: dict[int, Tensor] = {}  # rotation tables by position count, kept for the engine's life (graphs hold them)
         if self.fuse_qkv:
@@ -501,10 +501,10 @@ class UVEngine:
     def own_head_ok(self, n: int) -> bool:
         """Whether head_of runs the head GEMM of n rows on this library's kernel with the final norm in it: 16-bit engines up
         to head_own_rows rows.  Measured on UV-50M (32 768 x 640 head) as the time of a whole graph-replayed decode step
-        against the vendor library's GEMM behind a norm launch: 0.327 against 0.335 ms at 128 rows, 0.369 against 0.373 at
-        256, equal at 512 and 1024, 0.546 against 0.543 at 768 - so the switch sits at 448 rows.  (Alone, on cold weights, the
-        kernel takes 11.5 - 25 us at 32 - 384 rows where the vendor library's takes 10 - 22 us plus ~6 us of norm launch; at
-        2048 rows 105 against 87 us.)"""
+        against the vendor library's GEMM behind a norm launch: 0.3325 against 0.3338 ms at 192 rows, 0.3644 against 0.3699
+        at 256, but 0.4137 against 0.4111 at 320 and 0.4363 against 0.4297 at 384 - so the switch sits at 288 rows.  (Alone,
+        on cold weights, the kernel takes 11.5 - 25 us at 32 - 384 rows where the vendor library's takes 10 - 22 us plus ~6 us
+        of norm launch; at 2048 rows 105 against 87 us.)"""
         cfg = self.cfg
         return (self.dtype in (torch.bfloat16, torch.float16) and n <= self.head_own_rows and cfg.d_model % 64 == 0
                 and cfg.d_model >= 128 and cfg.vocab_size % 16 == 0)
