@@ -402,6 +402,74 @@ def bench_attn_ceiling(args):
                                              "frac_if_only_the_stream_remained": round(at / (icpt + slope * at) / 1e3 / HBM_PEAK_GBS, 4)}}}))
 
 
+def bench_gemm(args):
+    """The projections of UV-50M as single launches, back to back in a graph on four rotating weight copies: this library's
+    GEMM forms (config 0 = what the dispatcher picks for the shape; 4 / 3 = 64 x 64 / 128 x 128 tiles staged through registers;
+    6 / 5 = 128 x 128 / 256 x 256 tiles loaded straight into LDS; 1 = the skinny form) beside the vendor library's (torch.mm /
+    addmm, without the norm or SwiGLU launch it needs around it), at a full decode step's 2048 rows and a mixed pass's 33 216."""
+    from ultraviolet_amd.kernels.gemm import RESID, STORE, SWIGLU, gemm_tn, interleave_gate_up
+    dev, dt = "cuda:0", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    shapes = [("qkv+gates, pre-norm", 656, 640, STORE, True), ("o, residual update", 640, 512, RESID, False),
+              ("gate-up, pre-norm + SwiGLU", 3328, 640, SWIGLU, True), ("down, residual update", 640, 1664, RESID, False),
+              ("head", 32768, 640, STORE, False)]
+
+    def timeit(fs, reps=4):
+        for f in fs:
+            f()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for _ in range(reps):
+                for f in fs:
+                    f()
+        gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * len(fs))
+
+    table = []
+    for M in (2048, 33216):
+        for name, N, K, epi, norm in shapes:
+            if name == "head" and M > 2048:
+                continue
+            ws = [(torch.randn(N, K, device=dev, generator=g) / K ** 0.5).to(dt) for _ in range(4)]
+            a = torch.randn(M, K, device=dev, generator=g).to(dt)
+            n_out = N // 2 if epi == SWIGLU else N
+            out = torch.empty(M, n_out, device=dev, dtype=dt)
+            x = torch.randn(M, N, device=dev, generator=g).to(dt) if epi == RESID else None
+            row = {"rows": M, "projection": name, "N": N, "K": K, "GFLOP": round(2e-9 * M * N * K, 2)}
+            timeit([(lambda w: (lambda: torch.mm(a, w.t())))(w) for w in ws])   # (the first graph on new buffers runs ~7 % slow)
+            for cfg in (0, 1, 4, 3, 6, 5):
+                kw = dict(epilogue=epi, norm_eps=1e-6 if norm else None, config=cfg)
+                if epi == RESID:
+                    kw.update(resid=x, ca=0.9, cb=1.1)
+                tgt = x if epi == RESID else out
+                try:
+                    gemm_tn(a, ws[0], tgt, **kw)
+                    torch.cuda.synchronize()
+                except Exception:
+                    continue
+                row[f"config{cfg}_us"] = round(timeit([(lambda w: (lambda: gemm_tn(a, w, tgt, **kw)))(w) for w in ws]), 2)
+            if epi == RESID:
+                lib = [(lambda w: (lambda: torch.addmm(x, a, w.t(), beta=0.9, alpha=1.1, out=x)))(w) for w in ws]
+            else:
+                full = torch.empty(M, N, device=dev, dtype=dt)
+                lib = [(lambda w: (lambda: torch.mm(a, w.t(), out=full)))(w) for w in ws]
+            row["vendor_us"] = round(timeit(lib), 2)
+            best = min(v for k, v in row.items() if k.endswith("_us") and k.startswith("config"))
+            row["config0_PFLOPs"] = round(row["GFLOP"] / row["config0_us"], 3)
+            row["best_own_us"] = best
+            table.append(row)
+    print(json.dumps({"metric": "projection GEMM launch time, UV-50M shapes", "value": None, "unit": "us", "n_gpus": 1, "steps": 16, "warmup": 1,
+                      "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "UV-50M projections at 2048 and 33 216 rows, one launch each, four rotating weight copies"},
+                      "table": table}))
+
+
 def bench_c4(args):
     """BASELINE configs[3]: mixed batch, 64 prompt chunks x 512 tokens + 448 decode rows, one forward pass per iteration."""
     from ultraviolet_amd.engine import KVState, UVEngine, UVWeights, make_config
@@ -550,7 +618,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed decode steps (0: the whole rollout after warm-up)")
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy", "attn-ceiling"])
+    ap.add_argument("--workload", default="c5", choices=["c5", "c2", "c3", "c4", "copy", "attn-ceiling", "gemm"])
     ap.add_argument("--host-admit", action="store_true", help="c3: the host chooses the slots of admitted prompts (default: the device does)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -573,6 +641,8 @@ def main():
         bench_c4(args)
     elif args.workload == "attn-ceiling":
         bench_attn_ceiling(args)
+    elif args.workload == "gemm":
+        bench_gemm(args)
     else:
         bench_c5(args)
 
