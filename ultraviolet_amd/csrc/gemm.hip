@@ -444,7 +444,12 @@ extern "C" int uvmi_gemm_tn_ex(const uvmi_gemm_args* a, void* stream) {
   if (a->M == 0) return UVMI_OK;
   const int BN = skinny_bn(a->K, a->epilogue);
   UVMI_REQUIRE(BN != 0 || a->config == 0 || a->config >= 3, UVMI_EUNSUPPORTED, "uvmi_gemm_tn: K = %d is beyond the skinny forms (config 1, 2)", a->K);
-  if (a->config == 5 || (a->config == 0 && a->M >= (a->epilogue == UVMI_GEMM_SWIGLU ? BIG_MIN_ROWS_SWIGLU : BIG_MIN_ROWS) && big_ok(a))) {
+  // (also a product of fewer rows whose 256 x 256 tiles still come to two rounds of the device or more - the tied head,
+  // 2048 x 32768: 104 us against 129 us on 128 x 128 tiles)
+  int cus_big = uvmi_device_cus();
+  if (cus_big <= 0) cus_big = 256;
+  const bool many_big_tiles = a->M >= 1024 && ((a->M + 255) / 256) * (((int64_t)a->N + 255) / 256) >= 2 * (int64_t)cus_big;
+  if (a->config == 5 || (a->config == 0 && (many_big_tiles || a->M >= (a->epilogue == UVMI_GEMM_SWIGLU ? BIG_MIN_ROWS_SWIGLU : BIG_MIN_ROWS)) && big_ok(a))) {
     UVMI_REQUIRE(big_ok(a), UVMI_EUNSUPPORTED,
                  "uvmi_gemm_tn: config 5 (256 x 256 tiles) needs K >= 128, C (and the residual) 16-byte aligned, ldc (ldr) %% 8 == 0");
     // An output whose width fills 128-wide tiles much better than 256-wide ones (N = 640: 5 tiles of 128 against 3 of 256, a
