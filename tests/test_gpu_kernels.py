@@ -707,6 +707,28 @@ def test_tiled_gemm_at_prefill_row_counts():
 
 
 @pytest.mark.gpu
+def test_gemm_builtin_choice_on_a_head_sized_product():
+    """A product of a few thousand rows whose 256 x 256 tiles make several rounds of the device (the tied head of a full decode
+    step: 2048 x 32768 x 640) goes to the 256 x 256 form by the built-in choice; with the final norm as its row scale it must
+    equal the float64 product of the normalised rows within an ulp of the output type, like the forced forms."""
+    from ultraviolet_amd.kernels.gemm import gemm_tn
+    dtype, M, K, N = torch.bfloat16, 2048, 640, 32768
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a = (torch.randn(M, K, device="cuda", generator=g) * 3).to(dtype)
+    w = (torch.randn(N, K, device="cuda", generator=g) / K ** 0.5).to(dtype)
+    eps, ulp = 1e-6, 2.0 ** -8
+    ad = a.double()
+    want = (ad * torch.rsqrt((ad * ad).mean(-1, keepdim=True) + eps)) @ w.double().t()
+    tol = ulp * want.abs().clamp_min(1.0) + 1e-3
+    outs = {}
+    for config in (0, 5, 6):
+        outs[config] = gemm_tn(a, w, norm_eps=eps, config=config)
+        err = (outs[config].double() - want).abs()
+        assert bool((err <= tol).all()), (config, float(err.max()))
+    assert torch.equal(outs[0], outs[5])   # the built-in choice is the 256 x 256 form here
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,K,N", [(1, 128, 16), (300, 640, 656), (257, 1664, 640), (1000, 512, 640), (700, 640, 3328), (1030, 2048, 224),
                                    (5000, 640, 672), (513, 192, 512)])
